@@ -1,0 +1,71 @@
+"""Engine-wide options.
+
+Reference: minivllm/config/config.py:6-59. Names and meanings are the reference's where it
+has them (``model``, ``max_model_len``, ``max_num_batched_tokens``, ``max_num_batched_seqs``,
+``eos_token_ids``, ``kv_cache_num_blocks``, ``kv_cache_block_size``,
+``gpu_memory_utilization``, ``use_cuda_graph``). Differences:
+
+* ``max_model_len`` is enforced (the reference never checks it);
+* ``kv_cache_num_blocks`` None sizes the cache from free device memory, a number is taken
+  as given (the reference treats it as an upper cap, executor.py:46);
+* ``use_cuda_graph`` keeps its name; the decode step is captured in a HIP graph;
+* the executor never writes into this object (the reference's does, executor.py:49).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional, Tuple
+
+
+@dataclass
+class EngineConfig:
+    # ---- model -------------------------------------------------------------------------
+    model: str = ""
+    # compute precision: "bfloat16" (serving) or "float32" (everything in IEEE 32-bit);
+    # None takes the model's own dtype from config.json
+    dtype: Optional[str] = None
+    # longest sequence (prompt + generated) a request may reach
+    max_model_len: int = 4096
+
+    # ---- scheduler ---------------------------------------------------------------------
+    # most tokens in one step, prompt portions and decoded tokens together
+    max_num_batched_tokens: int = 16384
+    # most requests in one step
+    max_num_batched_seqs: int = 512
+    # most prompt tokens of one request in one step (None: only the token budget limits it)
+    prefill_chunk: Optional[int] = None
+    # None takes config.json's eos_token_id
+    eos_token_ids: Optional[Tuple[int, ...]] = None
+
+    # ---- cache -------------------------------------------------------------------------
+    kv_cache_num_blocks: Optional[int] = None
+    kv_cache_block_size: int = 16
+    gpu_memory_utilization: float = 0.5
+    enable_prefix_caching: bool = False
+
+    # ---- executor ----------------------------------------------------------------------
+    use_cuda_graph: bool = True
+    seed: int = 0
+
+    def __post_init__(self) -> None:
+        self.validate()
+
+    def validate(self) -> None:
+        if self.dtype not in (None, "bfloat16", "float32"):
+            raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
+        if self.max_model_len < 1:
+            raise ValueError(f"max_model_len must be >= 1, got {self.max_model_len}")
+        if self.max_num_batched_tokens < 1:
+            raise ValueError(f"max_num_batched_tokens must be >= 1, got {self.max_num_batched_tokens}")
+        if self.max_num_batched_seqs < 1:
+            raise ValueError(f"max_num_batched_seqs must be >= 1, got {self.max_num_batched_seqs}")
+        if self.prefill_chunk is not None and self.prefill_chunk < 1:
+            raise ValueError(f"prefill_chunk must be >= 1, got {self.prefill_chunk}")
+        if self.kv_cache_block_size < 1:
+            raise ValueError(f"kv_cache_block_size must be >= 1, got {self.kv_cache_block_size}")
+        if self.kv_cache_num_blocks is not None and self.kv_cache_num_blocks < 1:
+            raise ValueError(f"kv_cache_num_blocks must be >= 1, got {self.kv_cache_num_blocks}")
+        if not (0.0 < self.gpu_memory_utilization <= 1.0):
+            raise ValueError(f"gpu_memory_utilization must be in (0, 1], got {self.gpu_memory_utilization}")
+        if self.eos_token_ids is not None:
+            self.eos_token_ids = tuple(int(e) for e in self.eos_token_ids)

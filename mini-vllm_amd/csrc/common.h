@@ -1,0 +1,112 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions, wave and
+// block reductions, and the error channel of the C entry points.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define MV_WAVE 64
+
+// ---------------------------------------------------------------------------------------
+// Storage types. Arithmetic is always done on float; bf16 is storage only.
+// ---------------------------------------------------------------------------------------
+struct bf16 {
+    uint16_t bits;
+};
+
+enum MvDtype { MV_F32 = 0, MV_BF16 = 1 };
+
+__device__ __forceinline__ float to_f(float v) { return v; }
+__device__ __forceinline__ float to_f(bf16 v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                               // nearest even
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_f(float f);
+template <> __device__ __forceinline__ float from_f<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16 from_f<bf16>(float f) {
+    bf16 r;
+    r.bits = f32_to_bf16_bits(f);
+    return r;
+}
+
+// A weight tensor whose element type is known only at run time (it is kept as stored:
+// bf16 or float). The branch is uniform over a launch.
+struct WeightPtr {
+    const void* p;
+    int dtype;
+    __device__ __forceinline__ float at(size_t i) const {
+        if (dtype == MV_F32) return ((const float*)p)[i];
+        return to_f(((const bf16*)p)[i]);
+    }
+};
+
+// ---------------------------------------------------------------------------------------
+// Reductions
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = MV_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, MV_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = MV_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MV_WAVE));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds at least 17 floats of LDS.
+// Every thread gets the result. The order of additions depends only on the block size.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x & (MV_WAVE - 1);
+    const int wave = threadIdx.x / MV_WAVE;
+    const int nwaves = (blockDim.x + MV_WAVE - 1) / MV_WAVE;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+        for (int i = 0; i < nwaves; ++i) t += scratch[i];
+        scratch[16] = t;
+    }
+    __syncthreads();
+    return scratch[16];
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x & (MV_WAVE - 1);
+    const int wave = threadIdx.x / MV_WAVE;
+    const int nwaves = (blockDim.x + MV_WAVE - 1) / MV_WAVE;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = scratch[0];
+        for (int i = 1; i < nwaves; ++i) t = fmaxf(t, scratch[i]);
+        scratch[16] = t;
+    }
+    __syncthreads();
+    return scratch[16];
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side: error reporting of the extern "C" entry points. Each returns 0 on success;
+// otherwise mv_last_error() holds the reason.
+// ---------------------------------------------------------------------------------------
+extern "C" const char* mv_last_error();
+int mv_fail(const char* fmt, ...);
+int mv_check_launch(const char* what);
+
+#define MV_REQUIRE(cond, ...)                      \
+    do {                                           \
+        if (!(cond)) return mv_fail(__VA_ARGS__);  \
+    } while (0)

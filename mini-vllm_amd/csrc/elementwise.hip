@@ -1,0 +1,293 @@
+// Row-wise kernels of the decoder: embedding gather, residual add fused with RMS
+// normalisation, rotary table, per-head q/k norm + rotary embedding + cache write, SwiGLU.
+// All arithmetic is float; T is the storage type of activations and cache pages. The
+// residual stream is always float.
+#include "dispatch.h"
+
+// ---------------------------------------------------------------------------------------
+// Embedding: resid[n, :] = table[ids[n], :] * scale        (float residual stream)
+// ---------------------------------------------------------------------------------------
+__global__ void embedding_kernel(const int* __restrict__ ids, WeightPtr table, float* __restrict__ resid,
+                                 int h, int vocab, float scale) {
+    const int row = blockIdx.x;
+    const int id = ids[row];
+    const bool valid = id >= 0 && id < vocab;
+    float* dst = resid + (size_t)row * h;
+    const size_t base = (size_t)(valid ? id : 0) * h;
+    for (int d = threadIdx.x; d < h; d += blockDim.x) dst[d] = valid ? table.at(base + d) * scale : 0.f;
+}
+
+extern "C" int mv_embedding(const int* ids, const void* table, int table_dtype, float* resid, int n, int h,
+                            int vocab, float scale, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && h > 0 && vocab > 0, "embedding: bad sizes n=%d h=%d vocab=%d", n, h, vocab);
+    MV_REQUIRE(mv_valid_dtype(table_dtype), "embedding: bad table dtype %d", table_dtype);
+    if (n == 0) return 0;
+    WeightPtr w{table, table_dtype};
+    hipLaunchKernelGGL(embedding_kernel, dim3(n), dim3(256), 0, stream, ids, w, resid, h, vocab, scale);
+    return mv_check_launch("embedding");
+}
+
+// ---------------------------------------------------------------------------------------
+// Residual add + RMSNorm.
+//   rows == null : for every row r: v = resid[r] + delta[r]; resid[r] = v; out[r] = norm(v) * w
+//   rows != null : for i < n_out, r = rows[i]: v = resid[r] + delta[r]; out[i] = norm(v) * w
+//                  (resid is left as it is; a negative row gives zeros)
+//   delta == null: nothing is added.  out == null: only the add is done.
+//   norm(v) = v / sqrt(mean(v^2) + eps);  weight is w, or 1 + w with unit_offset.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta, WeightPtr w, float eps,
+                                   int unit_offset, T* __restrict__ out, const int* __restrict__ rows, int h) {
+    __shared__ float scratch[17];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    if (r < 0) {
+        if (out)
+            for (int d = threadIdx.x; d < h; d += blockDim.x) out[(size_t)i * h + d] = from_f<T>(0.f);
+        return;
+    }
+    float* x = resid + (size_t)r * h;
+    const T* dl = delta ? delta + (size_t)r * h : nullptr;
+    float ss = 0.f;
+    if (out) {
+        for (int d = threadIdx.x; d < h; d += blockDim.x) {
+            float v = x[d];
+            if (dl) v += to_f(dl[d]);
+            ss += v * v;
+        }
+        ss = block_sum(ss, scratch);
+    }
+    const float rinv = out ? rsqrtf(ss / (float)h + eps) : 0.f;
+    const bool write_back = (rows == nullptr) && (dl != nullptr);
+    for (int d = threadIdx.x; d < h; d += blockDim.x) {
+        float v = x[d];
+        if (dl) v += to_f(dl[d]);
+        if (write_back) x[d] = v;
+        if (out) {
+            float wt = w.at(d);
+            if (unit_offset) wt += 1.f;
+            out[(size_t)i * h + d] = from_f<T>(v * rinv * wt);
+        }
+    }
+}
+
+extern "C" int mv_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype, float eps,
+                              int unit_offset, void* out, const int* rows, int n_out, int h, int dtype,
+                              hipStream_t stream) {
+    MV_REQUIRE(n_out >= 0 && h > 0, "add_rmsnorm: bad sizes n=%d h=%d", n_out, h);
+    MV_REQUIRE(out == nullptr || weight != nullptr, "add_rmsnorm: norm asked without a weight");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype), "add_rmsnorm: bad weight dtype %d", weight_dtype);
+    MV_REQUIRE(eps > 0.f || out == nullptr, "add_rmsnorm: eps must be positive");
+    if (n_out == 0) return 0;
+    WeightPtr w{weight, weight_dtype};
+    MV_DISPATCH_T(dtype, "add_rmsnorm",
+                  hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(256), 0, stream, resid,
+                                     (const T*)delta, w, eps, unit_offset, (T*)out, rows, h));
+    return mv_check_launch("add_rmsnorm");
+}
+
+// Plain RMSNorm over the last dimension of a strided [n, h] view.
+template <typename T>
+__global__ void rmsnorm_kernel(const T* __restrict__ in, long in_stride, WeightPtr w, float eps, int unit_offset,
+                               T* __restrict__ out, long out_stride, int h) {
+    __shared__ float scratch[17];
+    const T* x = in + (size_t)blockIdx.x * in_stride;
+    T* y = out + (size_t)blockIdx.x * out_stride;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < h; d += blockDim.x) {
+        float v = to_f(x[d]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float rinv = rsqrtf(ss / (float)h + eps);
+    for (int d = threadIdx.x; d < h; d += blockDim.x) {
+        float wt = w.at(d);
+        if (unit_offset) wt += 1.f;
+        y[d] = from_f<T>(to_f(x[d]) * rinv * wt);
+    }
+}
+
+extern "C" int mv_rmsnorm(const void* in, long in_stride, const void* weight, int weight_dtype, float eps,
+                          int unit_offset, void* out, long out_stride, int n, int h, int dtype,
+                          hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && h > 0, "rmsnorm: bad sizes n=%d h=%d", n, h);
+    MV_REQUIRE(in_stride >= h && out_stride >= h, "rmsnorm: row strides %ld/%ld shorter than h=%d", in_stride,
+               out_stride, h);
+    MV_REQUIRE(mv_valid_dtype(weight_dtype), "rmsnorm: bad weight dtype %d", weight_dtype);
+    MV_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive");
+    if (n == 0) return 0;
+    WeightPtr w{weight, weight_dtype};
+    const int threads = h >= 256 ? 256 : 64;
+    MV_DISPATCH_T(dtype, "rmsnorm",
+                  hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(n), dim3(threads), 0, stream, (const T*)in, in_stride,
+                                     w, eps, unit_offset, (T*)out, out_stride, h));
+    return mv_check_launch("rmsnorm");
+}
+
+// ---------------------------------------------------------------------------------------
+// Rotary table: table[pos, 0:R/2] = cos(pos * inv_freq), table[pos, R/2:R] = sin(...).
+// The angle is the float product of the float position and the float inverse frequency.
+// ---------------------------------------------------------------------------------------
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, float* __restrict__ table, int max_pos,
+                                  int half) {
+    const int pos = blockIdx.x;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        const float ang = (float)pos * inv_freq[i];
+        table[(size_t)pos * 2 * half + i] = cosf(ang);
+        table[(size_t)pos * 2 * half + half + i] = sinf(ang);
+    }
+}
+
+extern "C" int mv_rope_table(const float* inv_freq, float* table, int max_pos, int rot_dim, hipStream_t stream) {
+    MV_REQUIRE(max_pos > 0 && rot_dim > 0 && rot_dim % 2 == 0, "rope_table: bad sizes max_pos=%d rot_dim=%d",
+               max_pos, rot_dim);
+    hipLaunchKernelGGL(rope_table_kernel, dim3(max_pos), dim3(64), 0, stream, inv_freq, table, max_pos,
+                       rot_dim / 2);
+    return mv_check_launch("rope_table");
+}
+
+// ---------------------------------------------------------------------------------------
+// Per-head q/k RMSNorm + rotary embedding + cache write, one wave per (token, head).
+//   q heads: normalised and rotated in place in the qkv rows.
+//   k heads: normalised, rotated, written to the key page   K[page][kv_head][slot][d].
+//   v heads: copied to the value page (transposed)            V[page][kv_head][d][slot].
+// page = block_table[seq, pos / page_size], slot = pos % page_size. Rows of padding
+// (token_seq < 0) and unmapped pages (< 0) are skipped.
+// Rotation pairs: half-split (p, p + R/2) or interleaved (2p, 2p + 1), p < R/2; elements
+// at or beyond R pass through.
+// ---------------------------------------------------------------------------------------
+#define MV_MAX_HEAD_DIM 512
+
+template <typename T>
+__global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, long row_stride, int q_off, int k_off, int v_off,
+                                          const int* __restrict__ positions, const int* __restrict__ token_seq,
+                                          const int* __restrict__ block_table, int bt_width, int page_size,
+                                          T* __restrict__ k_pages, T* __restrict__ v_pages, int H, int Hkv, int D,
+                                          WeightPtr qw, WeightPtr kw, int has_norm, float eps, int unit_offset,
+                                          const float* __restrict__ table, int rot_dim, int interleaved,
+                                          int store_kv) {
+    __shared__ float sh[4][MV_MAX_HEAD_DIM];
+    const int tok = blockIdx.x;
+    const int wave = threadIdx.x / MV_WAVE;
+    const int lane = threadIdx.x % MV_WAVE;
+    const int head = blockIdx.y * 4 + wave;
+    const int total = H + (store_kv ? 2 * Hkv : 0);
+    const int seq = token_seq[tok];
+    const int pos = positions[tok];
+    const bool active = head < total && seq >= 0;
+    int kind = 0, hh = head;  // 0 q, 1 k, 2 v
+    if (head >= H + Hkv) {
+        kind = 2;
+        hh = head - H - Hkv;
+    } else if (head >= H) {
+        kind = 1;
+        hh = head - H;
+    }
+    T* row = qkv + (size_t)tok * row_stride;
+    T* src = row + (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) + (size_t)hh * D;
+    float* x = sh[wave];
+
+    float ss = 0.f;
+    if (active) {
+        for (int d = lane; d < D; d += MV_WAVE) {
+            const float v = to_f(src[d]);
+            x[d] = v;
+            ss += v * v;
+        }
+    }
+    ss = wave_sum(ss);
+    __syncthreads();
+    if (active && kind != 2 && has_norm) {
+        const float rinv = rsqrtf(ss / (float)D + eps);
+        const WeightPtr& w = kind == 0 ? qw : kw;
+        for (int d = lane; d < D; d += MV_WAVE) {
+            float wt = w.at(d);
+            if (unit_offset) wt += 1.f;
+            x[d] = x[d] * rinv * wt;
+        }
+    }
+    __syncthreads();
+    if (active && kind != 2 && table != nullptr) {
+        const int half = rot_dim / 2;
+        const float* cs = table + (size_t)pos * rot_dim;
+        for (int p = lane; p < half; p += MV_WAVE) {
+            const int i1 = interleaved ? 2 * p : p;
+            const int i2 = interleaved ? 2 * p + 1 : p + half;
+            const float c = cs[p], s = cs[half + p];
+            const float a = x[i1], b = x[i2];
+            x[i1] = a * c - b * s;
+            x[i2] = b * c + a * s;
+        }
+    }
+    __syncthreads();
+    if (!active) return;
+    if (kind == 0) {
+        for (int d = lane; d < D; d += MV_WAVE) src[d] = from_f<T>(x[d]);
+        return;
+    }
+    const int page = block_table[(size_t)seq * bt_width + pos / page_size];
+    if (page < 0) return;
+    const int slot = pos % page_size;
+    if (kind == 1) {
+        T* dst = k_pages + (((size_t)page * Hkv + hh) * page_size + slot) * D;
+        for (int d = lane; d < D; d += MV_WAVE) dst[d] = from_f<T>(x[d]);
+    } else {
+        T* dst = v_pages + ((size_t)page * Hkv + hh) * D * page_size + slot;
+        for (int d = lane; d < D; d += MV_WAVE) dst[(size_t)d * page_size] = from_f<T>(x[d]);
+    }
+}
+
+extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int k_off, int v_off,
+                                     const int* positions, const int* token_seq, const int* block_table,
+                                     int bt_width, int page_size, void* k_pages, void* v_pages, int n, int H,
+                                     int Hkv, int D, const void* q_weight, const void* k_weight, int weight_dtype,
+                                     float eps, int unit_offset, const float* table, int rot_dim, int interleaved,
+                                     int store_kv, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && Hkv >= 0 && D > 0, "qk_norm_rope_store: bad sizes n=%d H=%d Hkv=%d D=%d", n, H,
+               Hkv, D);
+    MV_REQUIRE(D <= MV_MAX_HEAD_DIM, "qk_norm_rope_store: head_dim %d exceeds the supported maximum %d", D,
+               MV_MAX_HEAD_DIM);
+    MV_REQUIRE(table == nullptr || (rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= D),
+               "qk_norm_rope_store: rotary dim %d must be even and at most head_dim %d", rot_dim, D);
+    MV_REQUIRE(!store_kv || (block_table && k_pages && v_pages && page_size > 0 && bt_width > 0),
+               "qk_norm_rope_store: cache write asked without pages or block table");
+    const int has_norm = q_weight != nullptr;
+    MV_REQUIRE(!has_norm || (k_weight != nullptr || !store_kv), "qk_norm_rope_store: q norm without k norm");
+    MV_REQUIRE(!has_norm || eps > 0.f, "qk_norm_rope_store: eps must be positive");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype), "qk_norm_rope_store: bad weight dtype %d", weight_dtype);
+    if (n == 0) return 0;
+    const int heads = H + (store_kv ? 2 * Hkv : 0);
+    WeightPtr qw{q_weight, weight_dtype}, kw{k_weight, weight_dtype};
+    dim3 grid(n, (heads + 3) / 4);
+    MV_DISPATCH_T(dtype, "qk_norm_rope_store",
+                  hipLaunchKernelGGL(qk_norm_rope_store_kernel<T>, grid, dim3(256), 0, stream, (T*)qkv, row_stride,
+                                     q_off, k_off, v_off, positions, token_seq, block_table, bt_width, page_size,
+                                     (T*)k_pages, (T*)v_pages, H, Hkv, D, qw, kw, has_norm, eps, unit_offset, table,
+                                     rot_dim, interleaved, store_kv));
+    return mv_check_launch("qk_norm_rope_store");
+}
+
+// ---------------------------------------------------------------------------------------
+// SwiGLU: out[n, i] = silu(gu[n, i]) * gu[n, I + i],  silu(z) = z / (1 + exp(-z))
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, long total, int I) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const long row = idx / I;
+    const int col = (int)(idx - row * I);
+    const float g = to_f(gu[row * 2 * I + col]);
+    const float u = to_f(gu[row * 2 * I + I + col]);
+    out[idx] = from_f<T>(g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int mv_swiglu(const void* gate_up, void* out, int n, int I, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && I > 0, "swiglu: bad sizes n=%d I=%d", n, I);
+    if (n == 0) return 0;
+    const long total = (long)n * I;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    MV_DISPATCH_T(dtype, "swiglu",
+                  hipLaunchKernelGGL(swiglu_kernel<T>, dim3(blocks), dim3(256), 0, stream, (const T*)gate_up,
+                                     (T*)out, total, I));
+    return mv_check_launch("swiglu");
+}

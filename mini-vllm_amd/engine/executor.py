@@ -1,0 +1,435 @@
+"""The executor: owns the model, the device memory of the cache and the one step function.
+
+Reference: minivllm/executor/executor.py (model load :18, warm-up :62-78, cache sizing and
+allocation :31-60, input building :81-163, forward :197-214) and minivllm/executor/graph.py
+(decode graphs for batch-size buckets with static inputs and inert padding rows). Differences:
+
+* ``step`` takes any mix of prompt portions and decoded tokens and returns float32 logits at
+  the wanted positions; sampling is a separate call (the reference returns token ids only);
+* step inputs are packed into one pinned buffer and copied with one transfer;
+* the cache is a pair of page tensors per call, K as [page][kv_head][slot][d] and V as
+  [page][kv_head][d][slot], grouped by retention; the reference holds one
+  [2, layers, blocks, block_size, kv_heads, head_dim] tensor (executor.py:51);
+* decode-only steps are replayed from a HIP graph captured per batch-size bucket on first use;
+  the block-table width of a graph is ceil(max_model_len / page_size), not the pool size
+  (graph.py:20);
+* nothing here writes into the configuration object (the reference's does, executor.py:49).
+"""
+from __future__ import annotations
+
+import logging
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, GroupSpec, groups_from_needs
+from ..config.engine_config import EngineConfig
+from ..kernels.ops import dtype_from_name, get_ops
+from ..models.causal_lm import CausalLM, expected_tensors
+from ..models.registry import Architecture, load_config
+from ..parts.base import Runtime, Workspace
+from ..weights.loader import check_tensors, open_model_folder
+from ..weights.source import DeviceTensors, TensorSource
+from .step import AttentionPlan, KVView, SeqStep, StepContext
+
+logger = logging.getLogger(__name__)
+
+GRAPH_BUCKETS = [1, 2, 4, 8] + list(range(16, 257, 16))     # as the reference's (graph.py:11-12)
+
+
+def _cdiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+class _Staging:
+    """Pinned host buffers for the step's integers, used in turn so that a buffer is never
+    rewritten while its copy to the device may still be running."""
+
+    def __init__(self, count: int = 4):
+        self.buffers: List[Optional[torch.Tensor]] = [None] * count
+        self.events: List[Optional[torch.cuda.Event]] = [None] * count
+        self.next = 0
+
+    def take(self, n: int) -> Tuple[torch.Tensor, int]:
+        i = self.next
+        self.next = (self.next + 1) % len(self.buffers)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        buf = self.buffers[i]
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 4096), dtype=torch.int32, pin_memory=True)
+            self.buffers[i] = buf
+        return buf, i
+
+    def sent(self, i: int) -> None:
+        ev = self.events[i]
+        if ev is None:
+            ev = self.events[i] = torch.cuda.Event()
+        ev.record()
+
+
+class Executor:
+    def __init__(self, config: EngineConfig, model: Optional[Tuple[Architecture, object, TensorSource]] = None,
+                 device: str = "cuda:0"):
+        """``model`` = (architecture, typed model config, tensor source) serves a model that is not
+        in a folder; otherwise ``config.model`` is read."""
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible; the engine has no CPU path")
+        self.config = config
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        if model is None:
+            arch, model_config = load_config(config.model)
+            source = open_model_folder(config.model)
+            where = config.model
+        else:
+            arch, model_config, source = model
+            where = "the given tensors"
+        self.arch, self.model_config = arch, model_config
+        dtype_name = config.dtype or getattr(model_config, "dtype", "bfloat16")
+        if dtype_name == "float16":
+            dtype_name = "bfloat16"
+        self.dtype = dtype_from_name(dtype_name)
+        self.page_size = config.kv_cache_block_size
+
+        plan = arch.plan(model_config)
+        if config.max_model_len > plan.max_positions:
+            raise ValueError(f"max_model_len {config.max_model_len} exceeds the model's "
+                             f"max_position_embeddings {plan.max_positions}")
+        check_tensors(source, expected_tensors(arch, model_config, plan), arch.ignorable(model_config), where)
+
+        self.ops = get_ops(self.dtype)
+        self.rt = Runtime(device=self.device, dtype=self.dtype, ops=self.ops, workspace=Workspace(self.device),
+                          max_positions=config.max_model_len)
+        tensors = DeviceTensors(source, self.device)
+        self.model = CausalLM(arch, model_config, plan, tensors, self.rt)
+        self.plan = plan
+        self.vocab_size = plan.vocab_size
+
+        self.needs = self.model.cache_needs()
+        self.groups: List[GroupSpec] = groups_from_needs(self.needs)
+        self.group_of_call: Dict[int, int] = {c: g for g, spec in enumerate(self.groups) for c in spec.calls}
+        for i, call in enumerate(plan.calls):
+            if call.cache_from is not None:
+                if call.cache_from not in self.group_of_call:
+                    raise ValueError(f"call {i} reads the cache of call {call.cache_from}, which keeps none")
+                self.group_of_call[i] = self.group_of_call[call.cache_from]
+        self.state_shapes = self.model.state_shapes()
+        self.has_state = any(s is not None for s in self.state_shapes)
+        self.num_state_slots = config.max_num_batched_seqs
+        self.max_pages_per_seq = _cdiv(config.max_model_len, self.page_size)
+
+        self._staging = _Staging()
+        self._meta_device: Optional[torch.Tensor] = None
+        self._graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, StepContext, torch.Tensor, torch.Tensor]] = {}
+        self._graph_pool = None
+        self._graph_workspace: Optional[Workspace] = None
+        self.kv_pages: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+        self.state_tensors: Dict[int, torch.Tensor] = {}
+        self.num_pages = 0
+        self._allocate_memory()
+
+    # ------------------------------------------------------------------------------------
+    # memory
+    # ------------------------------------------------------------------------------------
+    def bytes_per_page(self) -> int:
+        item = torch.empty((), dtype=self.dtype).element_size()
+        return sum(n.bytes_per_token(item) for n in self.needs if n is not None) * self.page_size
+
+    def _allocate_memory(self) -> None:
+        cfg = self.config
+        for call, shape in enumerate(self.state_shapes):
+            if shape is not None:
+                dims, dt = shape
+                self.state_tensors[call] = torch.zeros((self.num_state_slots,) + tuple(dims), dtype=dt,
+                                                       device=self.device)
+        if cfg.kv_cache_num_blocks is not None:
+            num_pages = cfg.kv_cache_num_blocks
+        else:
+            self._warmup(cfg.max_num_batched_tokens)
+            torch.cuda.synchronize()
+            free, total = torch.cuda.mem_get_info(self.device)
+            used = total - free
+            per_page = max(1, self.bytes_per_page())
+            budget = int(total * cfg.gpu_memory_utilization) - used
+            num_pages = budget // per_page
+            if num_pages < 1:
+                raise RuntimeError(f"no memory left for the cache: {used / 2**30:.1f} GiB are in use, "
+                                   f"gpu_memory_utilization {cfg.gpu_memory_utilization} of "
+                                   f"{total / 2**30:.1f} GiB allows {budget / 2**30:.2f} GiB more")
+            # never more than every request at full length can use
+            num_pages = min(num_pages, cfg.max_num_batched_seqs * self.max_pages_per_seq)
+        self._allocate_pages(num_pages)
+        logger.info("allocated %d cache pages of %d tokens (%.2f GiB)", num_pages, self.page_size,
+                    num_pages * self.bytes_per_page() / 2 ** 30)
+
+    def _allocate_pages(self, num_pages: int) -> None:
+        self.kv_pages.clear()
+        self.num_pages = num_pages
+        for call, need in enumerate(self.needs):
+            if need is None:
+                continue
+            k_shape, v_shape = need.page_shapes(self.page_size)
+            k = torch.zeros((num_pages,) + k_shape, dtype=self.dtype, device=self.device)
+            v = torch.zeros((num_pages,) + v_shape, dtype=self.dtype, device=self.device)
+            self.kv_pages[call] = (k, v)
+        self._graphs.clear()
+
+    def _warmup(self, num_tokens: int) -> None:
+        """One dry step of ``num_tokens`` tokens against a throw-away cache, so that every scratch
+        buffer reaches its final size before the cache is sized from what is left."""
+        ps = self.page_size
+        n_seqs = max(1, min(self.config.max_num_batched_seqs, _cdiv(num_tokens, ps)))
+        per_seq = max(1, num_tokens // n_seqs)
+        pages_per_seq = _cdiv(per_seq, ps)
+        self._allocate_pages(n_seqs * pages_per_seq)
+        seqs = []
+        for s in range(n_seqs):
+            table = list(range(s * pages_per_seq, (s + 1) * pages_per_seq))
+            seqs.append(SeqStep(tokens=[0] * per_seq, start=0, block_tables=[table] * len(self.groups),
+                                state_slot=s % self.num_state_slots, want=[per_seq - 1]))
+        self.step(seqs)
+        torch.cuda.synchronize()
+        self.kv_pages.clear()
+        torch.cuda.empty_cache()
+
+    def new_cache_manager(self, enable_prefix_caching: Optional[bool] = None) -> CacheManager:
+        """A manager for this executor's pages and state slots."""
+        if enable_prefix_caching is None:
+            enable_prefix_caching = self.config.enable_prefix_caching
+        return CacheManager(self.groups, self.num_pages, self.page_size, self.num_state_slots,
+                            enable_prefix_caching=enable_prefix_caching, has_state=self.has_state)
+
+    # ------------------------------------------------------------------------------------
+    # building a step
+    # ------------------------------------------------------------------------------------
+    def _validate(self, seqs: Sequence[SeqStep]) -> None:
+        ps = self.page_size
+        for i, s in enumerate(seqs):
+            n = len(s.tokens)
+            if n < 1:
+                raise ValueError(f"sequence {i} of the step brings no token")
+            if s.start < 0 or s.start + n > self.config.max_model_len:
+                raise ValueError(f"sequence {i}: positions {s.start}..{s.start + n - 1} exceed max_model_len "
+                                 f"{self.config.max_model_len}")
+            if len(s.block_tables) != len(self.groups):
+                raise ValueError(f"sequence {i} brings {len(s.block_tables)} block tables, the model has "
+                                 f"{len(self.groups)} cache groups")
+            if not (0 <= s.state_slot < self.num_state_slots):
+                raise ValueError(f"sequence {i}: state slot {s.state_slot} out of range")
+            for w in s.want:
+                if not (0 <= w < n):
+                    raise ValueError(f"sequence {i}: wanted index {w} outside its {n} tokens")
+            last_page = (s.start + n - 1) // ps
+            for g in range(len(self.groups)):
+                if len(s.block_tables[g]) <= last_page:
+                    raise ValueError(f"sequence {i}: group {g} has {len(s.block_tables[g])} pages, position "
+                                     f"{s.start + n - 1} needs {last_page + 1}")
+
+    def _fill(self, seqs: Sequence[SeqStep], pad_to: Optional[int] = None, bt_widths: Optional[List[int]] = None):
+        """Packs the step's integers into one int32 array. Returns (array, offsets dict, facts)."""
+        S = len(seqs)
+        q_lens = [len(s.tokens) for s in seqs]
+        N = sum(q_lens)
+        Sp = pad_to if pad_to is not None else S
+        Np = pad_to if pad_to is not None else N
+        want_rows: List[int] = []
+        base = 0
+        for s, n in zip(seqs, q_lens):
+            want_rows.extend(base + w for w in s.want)
+            base += n
+        M = len(want_rows)
+        Mp = pad_to if pad_to is not None else M
+        widths = bt_widths or [max(1, max(len(s.block_tables[g]) for s in seqs)) for g in range(len(self.groups))]
+        off = {}
+        cur = 0
+        for name, size in (("token_ids", Np), ("positions", Np), ("token_seq", Np), ("cu_seqlens", Sp + 1),
+                           ("context_lens", Sp), ("state_slots", Sp), ("logit_rows", Mp)):
+            off[name] = (cur, size)
+            cur += size
+        for g, w in enumerate(widths):
+            off[f"bt{g}"] = (cur, Sp * w)
+            cur += Sp * w
+        arr = np.zeros(cur, dtype=np.int32)
+        tok = arr[off["token_ids"][0]:off["token_ids"][0] + Np]
+        pos = arr[off["positions"][0]:off["positions"][0] + Np]
+        tsq = arr[off["token_seq"][0]:off["token_seq"][0] + Np]
+        tsq[:] = -1
+        cu = arr[off["cu_seqlens"][0]:off["cu_seqlens"][0] + Sp + 1]
+        cl = arr[off["context_lens"][0]:off["context_lens"][0] + Sp]
+        sl = arr[off["state_slots"][0]:off["state_slots"][0] + Sp]
+        lr = arr[off["logit_rows"][0]:off["logit_rows"][0] + Mp]
+        lr[:] = -1
+        lr[:M] = want_rows
+        base = 0
+        for i, (s, n) in enumerate(zip(seqs, q_lens)):
+            tok[base:base + n] = s.tokens
+            pos[base:base + n] = np.arange(s.start, s.start + n, dtype=np.int32)
+            tsq[base:base + n] = i
+            cu[i + 1] = base + n
+            cl[i] = s.start + n
+            sl[i] = s.state_slot
+            base += n
+        cu[S + 1:] = base
+        starts = np.fromiter((s.start for s in seqs), dtype=np.int64, count=S)
+        last_page = (cl[:S].astype(np.int64) - 1) // self.page_size
+        for g, w in enumerate(widths):
+            o, size = off[f"bt{g}"]
+            bt = arr[o:o + size].reshape(Sp, w)
+            bt[:] = -1
+            for i, s in enumerate(seqs):
+                t = s.block_tables[g]
+                if len(t) > w:
+                    raise ValueError(f"sequence {i}: {len(t)} pages exceed the block table width {w}")
+                bt[i, :len(t)] = t
+            # every page a kernel may touch must be a page of the pool
+            spec = self.groups[g]
+            first_pos = np.zeros(S, dtype=np.int64) if spec.retention == "full" else np.maximum(0, starts - spec.window)
+            idx = np.arange(w, dtype=np.int64)[None, :]
+            touched = (idx >= (first_pos // self.page_size)[:, None]) & (idx <= last_page[:, None])
+            ids = bt[:S][touched]
+            if ids.size and (ids.min() < 0 or ids.max() >= self.num_pages):
+                raise ValueError(f"cache group {g}: a block table names a page outside the pool of "
+                                 f"{self.num_pages} (or one that was given back) where the step reads or writes")
+        if N and (tok[:N].min() < 0 or tok[:N].max() >= self.vocab_size):
+            raise ValueError(f"token ids must lie in [0, {self.vocab_size})")
+        facts = dict(S=S, N=N, M=M, Sp=Sp, Np=Np, Mp=Mp, q_lens=q_lens, widths=widths)
+        return arr, off, facts
+
+    def _context(self, meta: torch.Tensor, off, facts, seqs: Sequence[SeqStep]) -> StepContext:
+        ctx = StepContext()
+        def view(name):
+            o, size = off[name]
+            return meta[o:o + size]
+        ctx.n_tokens, ctx.n_seqs, ctx.n_logit_rows = facts["Np"], facts["Sp"], facts["Mp"]
+        ctx.token_ids = view("token_ids")
+        ctx.positions = view("positions")
+        ctx.token_seq = view("token_seq")
+        ctx.cu_seqlens = view("cu_seqlens")
+        ctx.context_lens = view("context_lens")
+        ctx.state_slots = view("state_slots")
+        ctx.logit_rows = view("logit_rows")
+        ctx.block_tables = [view(f"bt{g}").view(facts["Sp"], w) for g, w in enumerate(facts["widths"])]
+        ctx.q_lens = facts["q_lens"]
+        ctx.starts = [s.start for s in seqs]
+        ctx.host_state_slots = [s.state_slot for s in seqs]
+        ctx.page_size = self.page_size
+        ctx.attention_plan = AttentionPlan(
+            decode_only=all(q == 1 for q in facts["q_lens"]),
+            max_q_len=max(facts["q_lens"]) if facts["q_lens"] else 0,
+            max_context_len=max((s.start + len(s.tokens) for s in seqs), default=0),
+            n_seqs=facts["Sp"])
+        for call in range(len(self.plan.calls)):
+            g = self.group_of_call.get(call)
+            if g is not None:
+                owner = self.plan.calls[call].cache_from
+                k, v = self.kv_pages[call if owner is None else owner]
+                ctx._kv[call] = KVView(k, v, ctx.block_tables[g], self.page_size)
+            if call in self.state_tensors:
+                ctx._state[call] = self.state_tensors[call]
+        return ctx
+
+    def _upload(self, arr: np.ndarray, dst: Optional[torch.Tensor] = None) -> torch.Tensor:
+        n = arr.size
+        host, idx = self._staging.take(n)
+        host[:n].numpy()[:] = arr
+        if dst is None:
+            if self._meta_device is None or self._meta_device.numel() < n:
+                self._meta_device = torch.empty(max(n, 1 << 16), dtype=torch.int32, device=self.device)
+            dst = self._meta_device
+        dst[:n].copy_(host[:n], non_blocking=True)
+        self._staging.sent(idx)
+        return dst
+
+    # ------------------------------------------------------------------------------------
+    # the step function
+    # ------------------------------------------------------------------------------------
+    @torch.inference_mode()
+    def step(self, seqs: Sequence[SeqStep]) -> torch.Tensor:
+        """Runs exactly the given tokens, as one batch, against the cache that earlier steps left,
+        writes their keys and values into it and returns float32 logits [wanted, vocab] in the
+        order of ``seqs`` and of each ``want``. The result lives in a buffer that the next step
+        overwrites."""
+        if not seqs:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        self._validate(seqs)
+        if self.has_state:
+            for s in seqs:
+                if s.start == 0:
+                    for t in self.state_tensors.values():
+                        t[s.state_slot].zero_()
+        S = len(seqs)
+        decode_only = all(len(s.tokens) == 1 for s in seqs)
+        if (self.config.use_cuda_graph and decode_only and S <= GRAPH_BUCKETS[-1]
+                and all(len(s.want) == 1 for s in seqs)):
+            return self._step_graph(seqs)
+        arr, off, facts = self._fill(seqs)
+        meta = self._upload(arr)
+        ctx = self._context(meta, off, facts, seqs)
+        return self.model.forward(ctx)
+
+    def _step_graph(self, seqs: Sequence[SeqStep]) -> torch.Tensor:
+        S = len(seqs)
+        bucket = next(b for b in GRAPH_BUCKETS if b >= S)
+        widths = [self.max_pages_per_seq] * len(self.groups)
+        arr, off, facts = self._fill(seqs, pad_to=bucket, bt_widths=widths)
+        entry = self._graphs.get(bucket)
+        if entry is None:
+            entry = self._capture(bucket, arr, off, facts, seqs)
+        graph, ctx, meta, logits = entry
+        ctx.attention_plan.max_context_len = max(s.start + 1 for s in seqs)
+        self._upload(arr, dst=meta)
+        graph.replay()
+        return logits[:S]
+
+    def _padding_step(self, bucket: int) -> StepContext:
+        """A context of ``bucket`` padding rows: every kernel runs, none touches the cache."""
+        widths = [self.max_pages_per_seq] * len(self.groups)
+        dummy = [SeqStep(tokens=[0], start=0, block_tables=[[0]] * len(self.groups), state_slot=0, want=[0])]
+        arr, off, facts = self._fill(dummy, pad_to=bucket, bt_widths=widths)
+        o, size = off["token_seq"]
+        arr[o:o + size] = -1
+        o, size = off["logit_rows"]
+        arr[o:o + size] = -1
+        meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
+        self._upload(arr, dst=meta)
+        return self._context(meta, off, facts, dummy)
+
+    def _capture(self, bucket: int, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
+        logger.info("capturing the decode graph for %d sequences", bucket)
+        library_gemm = self.ops.use_library_gemm
+        eager_workspace = self.rt.workspace
+        self.ops.use_library_gemm = False          # only the engine's own kernels inside a graph
+        try:
+            if self._graph_workspace is None:
+                # one scratch area for all graphs, sized once for the largest bucket and then
+                # never reallocated: captured graphs keep its addresses
+                self._graph_workspace = Workspace(self.device)
+                self.rt.workspace = self._graph_workspace
+                largest = next(b for b in GRAPH_BUCKETS
+                               if b >= min(self.config.max_num_batched_seqs, GRAPH_BUCKETS[-1]))
+                pad_ctx = self._padding_step(largest)
+                pad_ctx.attention_plan.max_context_len = self.config.max_model_len
+                self.model.forward(pad_ctx)
+                torch.cuda.synchronize()
+                self._graph_workspace.frozen = True
+            self.rt.workspace = self._graph_workspace
+            meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
+            self._upload(arr, dst=meta)
+            ctx = self._context(meta, off, facts, seqs)
+            # the graph must serve every later context length: plan for the longest
+            ctx.attention_plan.max_context_len = self.config.max_model_len
+            self.model.forward(ctx)                # loads every kernel before the capture
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits = self.model.forward(ctx)
+            self._graph_pool = graph.pool()
+        finally:
+            self.rt.workspace = eager_workspace
+            self.ops.use_library_gemm = library_gemm
+        torch.cuda.synchronize()
+        entry = (graph, ctx, meta, logits)
+        self._graphs[bucket] = entry
+        return entry

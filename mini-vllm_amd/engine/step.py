@@ -1,0 +1,95 @@
+"""The step function's input and the context every part sees during a step.
+
+A step is a batch of (request, its next tokens): portions of prompts beside single decoded
+tokens, cut anywhere. Reference: the reference builds either a prefill input (whole uncached
+prompts; minivllm/executor/executor.py:81-127) or a decode input (one token per request;
+executor.py:130-153) and hands the layers a ``Context`` with cu_seqlens / slot_mapping /
+cache_seqlens / block_table (minivllm/executor/context.py). Here one layout serves both and
+any mix: flat token ids and positions, the sequence each token belongs to, per sequence the
+range of its tokens and its context length, one block table per cache group; cache slots are
+computed by the kernels from position and block table.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+
+@dataclass
+class SeqStep:
+    """One request's share of a step.
+
+    tokens        the next tokens of the request (>= 1)
+    start         position of tokens[0] = number of the request's tokens already in the cache
+    block_tables  per cache group, the request's page ids by page index (-1: given back)
+    state_slot    row of the state tensors that belongs to the request
+    want          indices into ``tokens`` whose logits are returned, in this order
+    """
+    tokens: Sequence[int]
+    start: int
+    block_tables: Sequence[Sequence[int]]
+    state_slot: int = 0
+    want: Sequence[int] = ()
+
+
+@dataclass
+class KVView:
+    """Cache of one call as its mixer sees it."""
+    k_pages: torch.Tensor          # [pages, kv_heads, page_size, head_dim]
+    v_pages: torch.Tensor          # [pages, kv_heads, head_dim, page_size]
+    block_table: torch.Tensor      # int32 [sequences, width] of the call's group
+    page_size: int
+
+
+@dataclass
+class AttentionPlan:
+    """Host-side facts about the step that let the attention pick a kernel."""
+    decode_only: bool              # every sequence brings exactly one token
+    max_q_len: int
+    max_context_len: int
+    n_seqs: int
+    scratch: Optional[torch.Tensor] = None     # float32 work area for split-key partial results
+
+
+class StepContext:
+    """Device tensors (int32) and host facts describing the step, handed to every part.
+
+    token_ids [n]      positions [n]        token_seq [n] (sequence index, -1 = padding row)
+    cu_seqlens [s+1]   context_lens [s]     state_slots [s]      logit_rows [m]
+    """
+
+    def __init__(self):
+        self.n_tokens = 0
+        self.n_seqs = 0
+        self.n_logit_rows = 0
+        self.token_ids: torch.Tensor = None
+        self.positions: torch.Tensor = None
+        self.token_seq: torch.Tensor = None
+        self.cu_seqlens: torch.Tensor = None
+        self.context_lens: torch.Tensor = None
+        self.state_slots: torch.Tensor = None
+        self.logit_rows: torch.Tensor = None
+        self.block_tables: List[torch.Tensor] = []
+        # host copies
+        self.q_lens: List[int] = []
+        self.starts: List[int] = []
+        self.host_state_slots: List[int] = []
+        self.attention_plan: Optional[AttentionPlan] = None
+        # filled by the executor
+        self._kv: Dict[int, "KVView"] = {}
+        self._state: Dict[int, torch.Tensor] = {}
+        self.page_size = 0
+
+    def kv(self, call: int) -> KVView:
+        try:
+            return self._kv[call]
+        except KeyError:
+            raise KeyError(f"call {call} has no cache: its mixer declared no cache need") from None
+
+    def state(self, call: int) -> torch.Tensor:
+        try:
+            return self._state[call]
+        except KeyError:
+            raise KeyError(f"call {call} has no state: its mixer declared no state shape") from None

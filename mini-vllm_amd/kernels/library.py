@@ -1,0 +1,128 @@
+"""Loads the HIP kernel libraries and declares their C entry points.
+
+There is no fall-back: when a library is missing it is compiled once (hipcc, a few seconds
+per file); when that is impossible the import of an operation fails with the reason.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Dict
+
+from ..csrc import build as _build
+
+c_int = ctypes.c_int
+c_long = ctypes.c_long
+c_float = ctypes.c_float
+c_void_p = ctypes.c_void_p
+
+DTYPE_F32 = 0
+DTYPE_BF16 = 1
+
+_SIGNATURES = {
+    "mv_last_error": (ctypes.c_char_p, []),
+    "mv_built_dtypes": (c_int, []),
+    "mv_abi_version": (c_int, []),
+    "mv_embedding": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
+    "mv_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
+                               c_int, c_int, c_int, c_void_p]),
+    "mv_rmsnorm": (c_int, [c_void_p, c_long, c_void_p, c_int, c_float, c_int, c_void_p, c_long, c_int, c_int,
+                           c_int, c_void_p]),
+    "mv_rope_table": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "mv_qk_norm_rope_store": (c_int, [c_void_p, c_long, c_int, c_int, c_int,            # qkv, stride, offsets
+                                      c_void_p, c_void_p, c_void_p, c_int, c_int,      # pos, seq, bt, width, page
+                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int,  # k, v pages, n, H, Hkv, D
+                                      c_void_p, c_void_p, c_int, c_float, c_int,       # qw, kw, wdtype, eps, unit
+                                      c_void_p, c_int, c_int, c_int, c_int, c_void_p]),  # table, rot, inter, store, dtype
+    "mv_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "mv_gemm_ref": (c_int, [c_void_p, c_long, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_int,
+                            c_int, c_int, c_int, c_void_p]),
+    "mv_attention_ref": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+    "mv_sample": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_void_p]),
+}
+
+# entry points that only the bfloat16 library has
+_OPTIONAL_SIGNATURES = {
+    "mv_gemm_skinny": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int,
+                               c_int, c_int, c_int, c_void_p]),
+    "mv_attention_decode": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                    c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
+                                    c_void_p, c_int, c_int, c_void_p]),
+    "mv_attention_prefill": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                     c_void_p]),
+}
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+class KernelLibrary:
+    """One loaded ``libmvk_<variant>.so``."""
+
+    def __init__(self, variant: str, path: str):
+        self.variant = variant
+        self.path = path
+        try:
+            self.dll = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelLibraryError(f"cannot load the HIP kernel library {path}: {e}") from e
+        for name, (res, args) in _SIGNATURES.items():
+            try:
+                fn = getattr(self.dll, name)
+            except AttributeError as e:
+                raise KernelLibraryError(f"{path} lacks the entry point {name}; rebuild it") from e
+            fn.restype = res
+            fn.argtypes = args
+        self.optional = set()
+        for name, (res, args) in _OPTIONAL_SIGNATURES.items():
+            fn = getattr(self.dll, name, None)
+            if fn is not None:
+                fn.restype = res
+                fn.argtypes = args
+                self.optional.add(name)
+
+    def has(self, name: str) -> bool:
+        return name in self.optional or name in _SIGNATURES
+
+    def call(self, name: str, *args) -> None:
+        rc = getattr(self.dll, name)(*args)
+        if rc != 0:
+            msg = self.dll.mv_last_error()
+            raise KernelLibraryError(msg.decode("utf-8", "replace") if msg else f"{name} failed")
+
+
+_LOCK = threading.Lock()
+_LOADED: Dict[str, KernelLibrary] = {}
+
+
+def variant_of(dtype_name: str) -> str:
+    if dtype_name in ("float32", "f32"):
+        return "f32"
+    if dtype_name in ("bfloat16", "bf16"):
+        return "bf16"
+    raise ValueError(f"no kernel library for dtype {dtype_name!r}")
+
+
+def load(variant: str) -> KernelLibrary:
+    """The library of ``variant`` ("f32" or "bf16"), building it first if it is not there."""
+    with _LOCK:
+        lib = _LOADED.get(variant)
+        if lib is not None:
+            return lib
+        path = _build.find_library(variant)
+        if path is None:
+            try:
+                path = _build.build(variant)
+            except Exception as e:
+                stale = _build.find_library(variant, require_fresh=False)
+                hint = f" (a library built from other sources is at {stale})" if stale else ""
+                raise KernelLibraryError(
+                    f"the HIP kernel library '{variant}' is not built and building it failed{hint}: {e}") from e
+        lib = KernelLibrary(variant, path)
+        _LOADED[variant] = lib
+        return lib

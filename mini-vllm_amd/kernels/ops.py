@@ -1,0 +1,323 @@
+"""Operations of the decoder on device tensors, bound to one activation type.
+
+Each method checks shapes, types and placement on the host and then launches a kernel of
+the HIP library on the current stream. Tensors must live on the GPU: there is no CPU path.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import library
+from .library import DTYPE_BF16, DTYPE_F32, KernelLibraryError
+
+_CODES = {torch.float32: DTYPE_F32, torch.bfloat16: DTYPE_BF16}
+_NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
+
+# largest number of rows the weight-streaming product takes in one launch
+SKINNY_MAX_M = 64
+
+
+def dtype_from_name(name: str) -> torch.dtype:
+    if name in ("float32", "fp32", "f32"):
+        return torch.float32
+    if name in ("bfloat16", "bf16"):
+        return torch.bfloat16
+    raise ValueError(f"compute dtype must be 'bfloat16' or 'float32', got {name!r}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _dev(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise KernelLibraryError(f"{what} is on {t.device}; the engine's kernels run on the GPU only")
+
+
+def _weight_code(w: torch.Tensor, what: str) -> int:
+    code = _CODES.get(w.dtype)
+    if code is None:
+        raise KernelLibraryError(f"{what} has dtype {w.dtype}; weights are float32 or bfloat16")
+    return code
+
+
+class Ops:
+    def __init__(self, dtype: torch.dtype):
+        if dtype not in _CODES:
+            raise ValueError(f"unsupported compute dtype {dtype}")
+        self.dtype = dtype
+        self.code = _CODES[dtype]
+        self.lib = library.load(library.variant_of(_NAMES[dtype]))
+        self.use_fast_kernels = dtype == torch.bfloat16
+        self.use_library_gemm = dtype == torch.bfloat16
+
+    # ------------------------------------------------------------------------------------
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    def _act(self, t: torch.Tensor, what: str) -> None:
+        _dev(t, what)
+        if t.dtype != self.dtype:
+            raise KernelLibraryError(f"{what} has dtype {t.dtype}, expected {self.dtype}")
+
+    # ------------------------------------------------------------------------------------
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor, resid: torch.Tensor, scale: float = 1.0) -> None:
+        """resid[n] = table[ids[n]] * scale; ids int32 [n], resid float32 [n, h]."""
+        _dev(ids, "ids"); _dev(table, "embedding table"); _dev(resid, "residual")
+        n, h = resid.shape
+        if ids.dtype != torch.int32 or ids.numel() < n or resid.dtype != torch.float32:
+            raise KernelLibraryError("embedding: ids must be int32 [>= n] and the residual float32 [n, h]")
+        if table.dim() != 2 or table.shape[1] != h or not table.is_contiguous() or not resid.is_contiguous():
+            raise KernelLibraryError(f"embedding: table {tuple(table.shape)} does not fit residual {tuple(resid.shape)}")
+        self.lib.call("mv_embedding", ids.data_ptr(), table.data_ptr(), _weight_code(table, "embedding table"),
+                      resid.data_ptr(), n, h, table.shape[0], float(scale), self._stream())
+
+    def add_rmsnorm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional[torch.Tensor],
+                    eps: float, out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
+                    unit_offset: bool = False) -> None:
+        """resid += delta (when ``rows`` is None), out = rmsnorm(resid + delta) * weight.
+
+        With ``rows`` (int32 [n_out]) only those rows are normalised into ``out`` and the
+        residual is left unchanged. ``out`` None does the add alone."""
+        _dev(resid, "residual")
+        if resid.dtype != torch.float32 or resid.dim() != 2 or not resid.is_contiguous():
+            raise KernelLibraryError("add_rmsnorm: the residual must be a contiguous float32 [n, h]")
+        n, h = resid.shape
+        if delta is not None:
+            self._act(delta, "delta")
+            if delta.shape != resid.shape or not delta.is_contiguous():
+                raise KernelLibraryError(f"add_rmsnorm: delta {tuple(delta.shape)} does not match {tuple(resid.shape)}")
+        n_out = n
+        if rows is not None:
+            _dev(rows, "rows")
+            if rows.dtype != torch.int32:
+                raise KernelLibraryError("add_rmsnorm: rows must be int32")
+            n_out = rows.numel()
+        wcode = DTYPE_F32
+        if out is not None:
+            self._act(out, "norm output")
+            if weight is None:
+                raise KernelLibraryError("add_rmsnorm: a norm needs its weight")
+            _dev(weight, "norm weight")
+            wcode = _weight_code(weight, "norm weight")
+            if weight.numel() != h or not weight.is_contiguous():
+                raise KernelLibraryError(f"add_rmsnorm: weight of {weight.numel()} elements for rows of {h}")
+            if out.dim() != 2 or out.shape[0] < n_out or out.shape[1] != h or not out.is_contiguous():
+                raise KernelLibraryError(f"add_rmsnorm: output {tuple(out.shape)} does not fit [{n_out}, {h}]")
+        self.lib.call("mv_add_rmsnorm", resid.data_ptr(), _ptr(delta), _ptr(weight), wcode, float(eps),
+                      int(unit_offset), _ptr(out), _ptr(rows), n_out, h, self.code, self._stream())
+
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+                unit_offset: bool = False) -> None:
+        """out = rmsnorm(x) * weight over the last dimension of 2-d views (rows may be strided)."""
+        self._act(x, "rmsnorm input"); self._act(out, "rmsnorm output"); _dev(weight, "norm weight")
+        if x.dim() != 2 or out.shape != x.shape or x.stride(1) != 1 or out.stride(1) != 1:
+            raise KernelLibraryError("rmsnorm: input and output must be 2-d with a contiguous last dimension")
+        n, h = x.shape
+        if weight.numel() != h or not weight.is_contiguous():
+            raise KernelLibraryError(f"rmsnorm: weight of {weight.numel()} elements for rows of {h}")
+        self.lib.call("mv_rmsnorm", x.data_ptr(), x.stride(0) if n > 1 else h, weight.data_ptr(),
+                      _weight_code(weight, "norm weight"), float(eps), int(unit_offset), out.data_ptr(),
+                      out.stride(0) if n > 1 else h, n, h, self.code, self._stream())
+
+    def rope_table(self, inv_freq: torch.Tensor, max_pos: int) -> torch.Tensor:
+        """float32 [max_pos, 2 * len(inv_freq)] = cat(cos, sin) of position * inv_freq."""
+        _dev(inv_freq, "inv_freq")
+        if inv_freq.dtype != torch.float32 or inv_freq.dim() != 1 or not inv_freq.is_contiguous():
+            raise KernelLibraryError("rope_table: inv_freq must be a contiguous float32 vector")
+        rot = 2 * inv_freq.numel()
+        table = torch.empty((max_pos, rot), dtype=torch.float32, device=inv_freq.device)
+        self.lib.call("mv_rope_table", inv_freq.data_ptr(), table.data_ptr(), max_pos, rot, self._stream())
+        return table
+
+    def qk_norm_rope_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                           positions: torch.Tensor, token_seq: torch.Tensor,
+                           q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                           rope_table: Optional[torch.Tensor], interleaved: bool,
+                           k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
+                           block_table: Optional[torch.Tensor], page_size: int,
+                           unit_offset: bool = False) -> None:
+        """In place on the rows of ``qkv`` = [q | k | v]: per-head RMSNorm of q and k (when
+        weights are given), rotary embedding (when a table is given); k and v are written to
+        the cache pages when pages are given. Without pages the rows hold only q."""
+        self._act(qkv, "qkv")
+        n = qkv.shape[0]
+        store = k_pages is not None
+        width = (num_heads + (2 * num_kv_heads if store else 0)) * head_dim
+        if qkv.dim() != 2 or qkv.shape[1] != width or qkv.stride(1) != 1:
+            raise KernelLibraryError(f"qk_norm_rope_store: qkv {tuple(qkv.shape)} does not hold {width} columns")
+        for t, what in ((positions, "positions"), (token_seq, "token_seq")):
+            _dev(t, what)
+            if t.dtype != torch.int32 or t.numel() < n:
+                raise KernelLibraryError(f"qk_norm_rope_store: {what} must be int32 with at least {n} elements")
+        wcode = DTYPE_F32
+        if q_weight is not None:
+            wcode = _weight_code(q_weight, "q_norm weight")
+            if q_weight.numel() != head_dim or (store and (k_weight is None or k_weight.numel() != head_dim
+                                                          or k_weight.dtype != q_weight.dtype)):
+                raise KernelLibraryError("qk_norm_rope_store: q/k norm weights must both hold head_dim elements")
+        rot = 0
+        if rope_table is not None:
+            _dev(rope_table, "rope table")
+            if rope_table.dtype != torch.float32 or rope_table.dim() != 2 or not rope_table.is_contiguous():
+                raise KernelLibraryError("qk_norm_rope_store: the rope table must be a contiguous float32 matrix")
+            rot = rope_table.shape[1]
+        bt_width = 0
+        if store:
+            assert v_pages is not None and block_table is not None
+            self._act(k_pages, "key pages"); self._act(v_pages, "value pages"); _dev(block_table, "block table")
+            if tuple(k_pages.shape[1:]) != (num_kv_heads, page_size, head_dim) or \
+                    tuple(v_pages.shape[1:]) != (num_kv_heads, head_dim, page_size) or \
+                    not k_pages.is_contiguous() or not v_pages.is_contiguous():
+                raise KernelLibraryError(
+                    f"qk_norm_rope_store: pages {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not match "
+                    f"[pages, {num_kv_heads}, {page_size}, {head_dim}] / [pages, {num_kv_heads}, {head_dim}, {page_size}]")
+            if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+                raise KernelLibraryError("qk_norm_rope_store: the block table must be a contiguous int32 matrix")
+            bt_width = block_table.shape[1]
+        q_dim = num_heads * head_dim
+        kv_dim = num_kv_heads * head_dim
+        self.lib.call("mv_qk_norm_rope_store", qkv.data_ptr(), qkv.stride(0) if n > 1 else width, 0, q_dim,
+                      q_dim + kv_dim, positions.data_ptr(), token_seq.data_ptr(), _ptr(block_table), bt_width,
+                      page_size, _ptr(k_pages), _ptr(v_pages), n, num_heads, num_kv_heads, head_dim,
+                      _ptr(q_weight), _ptr(k_weight), wcode, float(eps), int(unit_offset), _ptr(rope_table), rot,
+                      int(interleaved), int(store), self.code, self._stream())
+
+    def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
+        """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+        self._act(gate_up, "gate_up"); self._act(out, "swiglu output")
+        n, two_i = gate_up.shape
+        if two_i % 2 or out.shape != (n, two_i // 2) or not gate_up.is_contiguous() or not out.is_contiguous():
+            raise KernelLibraryError(f"swiglu: {tuple(gate_up.shape)} -> {tuple(out.shape)} is not [n, 2I] -> [n, I]")
+        self.lib.call("mv_swiglu", gate_up.data_ptr(), out.data_ptr(), n, two_i // 2, self.code, self._stream())
+
+    # ------------------------------------------------------------------------------------
+    def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+             exact: bool = False) -> None:
+        """out[M, N] = a[M, K] @ w[N, K]^T (+ bias). ``out`` is the activation type or float32.
+
+        float32 compute always takes the exact kernel. bfloat16 compute takes the
+        weight-streaming MFMA kernel for up to SKINNY_MAX_M rows, the library's matrix product
+        for more rows, and the exact kernel when the weight is stored in float32, when
+        ``exact`` is set or when no other kernel takes the shape."""
+        self._act(a, "gemm input"); _dev(w, "gemm weight"); _dev(out, "gemm output")
+        if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+            raise KernelLibraryError("gemm: operands must be matrices")
+        M, K = a.shape
+        N = w.shape[0]
+        if w.shape[1] != K or out.shape != (M, N):
+            raise KernelLibraryError(f"gemm: [{M}, {K}] x {tuple(w.shape)}^T -> {tuple(out.shape)} does not fit")
+        if a.stride(1) != 1 or out.stride(1) != 1 or not w.is_contiguous():
+            raise KernelLibraryError("gemm: operands need a contiguous last dimension")
+        if out.dtype not in (self.dtype, torch.float32):
+            raise KernelLibraryError(f"gemm: output dtype {out.dtype} must be {self.dtype} or float32")
+        wcode = _weight_code(w, "gemm weight")
+        if bias is not None:
+            _dev(bias, "bias")
+            if bias.dtype != w.dtype or bias.numel() != N:
+                raise KernelLibraryError("gemm: the bias must have the weight's dtype and N elements")
+        if M == 0:
+            return
+        lda = a.stride(0) if M > 1 else K
+        ldc = out.stride(0) if M > 1 else N
+        fast = self.use_fast_kernels and not exact and wcode == DTYPE_BF16
+        if fast and K % 32 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.lib.has("mv_gemm_skinny"):
+            if M <= SKINNY_MAX_M or out.dtype == torch.float32 or not self.use_library_gemm:
+                for m0 in range(0, M, SKINNY_MAX_M):
+                    m = min(SKINNY_MAX_M, M - m0)
+                    self.lib.call("mv_gemm_skinny", a.data_ptr() + m0 * lda * 2, lda, w.data_ptr(), K, _ptr(bias),
+                                  out.data_ptr() + m0 * ldc * out.element_size(), ldc, _CODES[out.dtype], m, N, K,
+                                  self._stream())
+                return
+        if fast and self.use_library_gemm and out.dtype == self.dtype and M > SKINNY_MAX_M:
+            if bias is None:
+                torch.mm(a, w.t(), out=out)
+            else:
+                torch.addmm(bias, a, w.t(), out=out)
+            return
+        self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
+                      out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
+
+    # ------------------------------------------------------------------------------------
+    def attention(self, q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                  block_table: torch.Tensor, page_size: int, positions: torch.Tensor, token_seq: torch.Tensor,
+                  num_heads: int, num_kv_heads: int, head_dim: int, scale: float, window: Optional[int],
+                  plan: Optional["AttentionPlan"] = None) -> None:
+        """Causal attention of the step's queries over the paged cache.
+
+        q: [n, >= H*D] rows (a view into the qkv rows), out: [n, H*D]. The query at position p
+        of sequence s sees keys max(0, p - window) .. p of s. ``plan`` carries what the faster
+        kernels need to know about the step (see AttentionPlan); without it, or in float32, the
+        general kernel runs."""
+        self._act(q, "queries"); self._act(out, "attention output")
+        self._act(k_pages, "key pages"); self._act(v_pages, "value pages")
+        n = q.shape[0]
+        hd = num_heads * head_dim
+        if q.dim() != 2 or q.shape[1] < hd or q.stride(1) != 1 or out.shape != (n, hd) or out.stride(1) != 1:
+            raise KernelLibraryError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not hold "
+                                     f"{num_heads} heads of {head_dim}")
+        if tuple(k_pages.shape[1:]) != (num_kv_heads, page_size, head_dim) or \
+                tuple(v_pages.shape[1:]) != (num_kv_heads, head_dim, page_size) or \
+                not k_pages.is_contiguous() or not v_pages.is_contiguous():
+            raise KernelLibraryError(f"attention: pages {tuple(k_pages.shape)} / {tuple(v_pages.shape)} have the "
+                                     f"wrong layout for {num_kv_heads} heads of {head_dim}, page {page_size}")
+        for t, what in ((positions, "positions"), (token_seq, "token_seq")):
+            _dev(t, what)
+            if t.dtype != torch.int32 or t.numel() < n:
+                raise KernelLibraryError(f"attention: {what} must be int32 with at least {n} elements")
+        _dev(block_table, "block table")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+            raise KernelLibraryError("attention: the block table must be a contiguous int32 matrix")
+        if num_heads % num_kv_heads:
+            raise KernelLibraryError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if n == 0:
+            return
+        w = -1 if window is None else int(window)
+        qs = q.stride(0) if n > 1 else q.shape[1]
+        os_ = out.stride(0) if n > 1 else hd
+        self.lib.call("mv_attention_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
+                      v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+                      positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim,
+                      float(scale), w, self.code, self._stream())
+
+    # ------------------------------------------------------------------------------------
+    def sample(self, logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+               top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+               rng: Optional[torch.Tensor] = None) -> None:
+        """One token id per row of float32 ``logits`` into int32 ``out``.
+
+        temperature float32 [M] (None or 0: arg-max), top_k int32 [M], top_p float32 [M],
+        rng int64 [M, 2] = (seed, counter) of each row's random stream."""
+        _dev(logits, "logits"); _dev(out, "sampled ids")
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise KernelLibraryError("sample: logits must be float32 [M, V] with a contiguous last dimension")
+        M, V = logits.shape
+        if out.dtype != torch.int32 or out.numel() < M:
+            raise KernelLibraryError("sample: the output must be int32 with at least M elements")
+        for t, dt, what in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
+                            (top_p, torch.float32, "top_p")):
+            if t is not None:
+                _dev(t, what)
+                if t.dtype != dt or t.numel() < M or not t.is_contiguous():
+                    raise KernelLibraryError(f"sample: {what} must be {dt} with at least M elements")
+        if temperature is not None:
+            if rng is None or rng.dtype != torch.int64 or rng.shape != (M, 2) or not rng.is_contiguous():
+                raise KernelLibraryError("sample: rng must be int64 [M, 2] when temperatures are given")
+            _dev(rng, "rng")
+        if M == 0:
+            return
+        self.lib.call("mv_sample", logits.data_ptr(), logits.stride(0) if M > 1 else V, M, V, _ptr(temperature),
+                      _ptr(top_k), _ptr(top_p), _ptr(rng), out.data_ptr(), self._stream())
+
+
+_OPS = {}
+
+
+def get_ops(dtype: torch.dtype) -> Ops:
+    ops = _OPS.get(dtype)
+    if ops is None:
+        ops = _OPS[dtype] = Ops(dtype)
+    return ops

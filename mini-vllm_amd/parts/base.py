@@ -1,0 +1,235 @@
+"""What a layer is made of, and how a part is declared, registered and built.
+
+A model is data: a ``ModelPlan`` lists layers, each layer names the kind and the sizes of
+its mixer, feed-forward, norms and the block arrangement that wires them. A part never
+learns which model it is in; it sees its own spec, its own tensors and the step's context.
+
+A part class has three duties:
+
+* ``tensors(spec)`` declares the tensors it needs, by logical name (``"q"``, ``"gate"``),
+  with shape and the law random weights are drawn from. The architecture maps logical
+  names to names on disk; the loader checks shapes and hands the tensors over.
+* ``__init__(spec, tensors, runtime)`` takes them (it may pack several into one).
+* ``forward(...)`` launches its kernels on the step's tensors.
+
+Mixers additionally state what memory they need per request: ``cache_need(spec)`` for pages
+of keys and values, ``state_shape(spec)`` for a fixed-size state.
+
+New kinds are added with ``register_mixer`` / ``register_feed_forward`` / ``register_norm`` /
+``register_position_encoding`` / ``register_block``; nothing else in the engine changes.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, ClassVar, Dict, List, Mapping, Optional, Sequence, Tuple, Type
+
+import torch
+
+
+# ---------------------------------------------------------------------------------------
+# Declarations
+# ---------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class TensorDecl:
+    """One tensor a part needs. ``init``: "normal" = N(0, std), "ones_normal" = 1 + N(0, std),
+    "zeros_normal" = N(0, std) for biases. ``integer`` tensors are kept as int32."""
+    shape: Tuple[int, ...]
+    init: str = "normal"
+    integer: bool = False
+
+
+class PartSpec:
+    """Base of the frozen dataclasses that describe one part; ``kind`` selects the class."""
+    kind: ClassVar[str] = ""
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """Paged memory a mixer needs for each token of a request.
+
+    ``retention``: "full" keeps every position; "window" keeps the last ``window`` positions
+    besides the current one, older pages go back to the pool. ``k_shape`` / ``v_shape`` give the
+    per-page tensor shapes as functions of the page size."""
+    retention: str
+    window: Optional[int]
+    num_kv_heads: int
+    head_dim: int
+
+    def group_key(self) -> Tuple:
+        return (self.retention, self.window)
+
+    def page_shapes(self, page_size: int) -> Tuple[Tuple[int, ...], Tuple[int, ...]]:
+        return ((self.num_kv_heads, page_size, self.head_dim), (self.num_kv_heads, self.head_dim, page_size))
+
+    def bytes_per_token(self, itemsize: int) -> int:
+        return 2 * self.num_kv_heads * self.head_dim * itemsize
+
+
+# ---------------------------------------------------------------------------------------
+# Registries
+# ---------------------------------------------------------------------------------------
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._classes: Dict[str, type] = {}
+
+    def register(self, kind: str, cls: Optional[type] = None):
+        def deco(c):
+            if kind in self._classes and self._classes[kind] is not c:
+                raise ValueError(f"{self.what} kind {kind!r} is already registered")
+            self._classes[kind] = c
+            return c
+        return deco(cls) if cls is not None else deco
+
+    def unregister(self, kind: str) -> None:
+        self._classes.pop(kind, None)
+
+    def get(self, kind: str) -> type:
+        try:
+            return self._classes[kind]
+        except KeyError:
+            raise KeyError(f"no {self.what} of kind {kind!r} is registered "
+                           f"(known: {sorted(self._classes)})") from None
+
+    def kinds(self) -> List[str]:
+        return sorted(self._classes)
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+BLOCKS = Registry("block arrangement")
+
+register_mixer = MIXERS.register
+register_feed_forward = FEED_FORWARDS.register
+register_norm = NORMS.register
+register_position_encoding = POSITION_ENCODINGS.register
+register_block = BLOCKS.register
+
+
+# ---------------------------------------------------------------------------------------
+# Runtime handed to every part
+# ---------------------------------------------------------------------------------------
+class Workspace:
+    """Named device buffers that live across steps and are shared between layers.
+
+    ``get`` returns a view of the wanted shape; the backing buffer grows when a step needs
+    more. While a graph is being captured nothing may be allocated, so the buffers have to be
+    grown (``reserve``) before."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self.frozen = False
+
+    def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < n:
+            if self.frozen:
+                raise RuntimeError(f"workspace buffer {name!r} would have to grow to {n} elements while frozen")
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:n].view(*shape)
+
+    def bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._buffers.values())
+
+
+@dataclass
+class Runtime:
+    """What parts share: the device, the activation type, the kernels and scratch memory."""
+    device: torch.device
+    dtype: torch.dtype
+    ops: Any
+    workspace: Workspace
+    max_positions: int          # longest sequence the engine serves (rows of position tables)
+
+
+class HiddenStream:
+    """The residual stream of a step: a float32 sum ``resid`` and the last part's output
+    ``delta`` that has not been added yet. A norm consumes the pending delta (one fused
+    kernel adds it and normalises the sum)."""
+
+    __slots__ = ("resid", "delta")
+
+    def __init__(self, resid: torch.Tensor):
+        self.resid = resid
+        self.delta: Optional[torch.Tensor] = None
+
+
+# ---------------------------------------------------------------------------------------
+# Part base classes (interfaces)
+# ---------------------------------------------------------------------------------------
+class Part:
+    spec_class: ClassVar[Optional[type]] = None
+
+    @classmethod
+    def tensors(cls, spec) -> Dict[str, TensorDecl]:
+        """Logical name -> declaration of every tensor this part reads from the model folder."""
+        return {}
+
+
+class Norm(Part):
+    """forward(stream, rows=None) -> normalised activations [n or len(rows), h]; adds the
+    stream's pending delta first (and keeps the sum in the stream unless ``rows`` is given).
+    apply(x, out) normalises a plain tensor."""
+
+    def forward(self, stream: HiddenStream, ctx, rows: Optional[torch.Tensor] = None,
+                tag: str = "normed") -> torch.Tensor:
+        raise NotImplementedError
+
+    def apply(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Either hands a rotary table to the mixer's fused kernel (``rotary()``) or rewrites q and
+    k itself (``apply``)."""
+
+    def rotary(self) -> Optional[Tuple[torch.Tensor, bool]]:
+        """(float32 table [positions, rotary_dim] = cat(cos, sin), interleaved) or None."""
+        return None
+
+    def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], ctx) -> None:
+        """In place on q [n, H, D] and k [n, Hkv, D] views, for encodings without a table."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """forward(x, ctx, call) -> y: mixes information along the sequence. ``call`` identifies
+    this execution of the layer in the model's order; ``ctx.kv(call)`` and ``ctx.state(call)``
+    give its cache pages and its per-request state."""
+
+    @classmethod
+    def cache_need(cls, spec) -> Optional[CacheNeed]:
+        return None
+
+    @classmethod
+    def state_shape(cls, spec) -> Optional[Tuple[Tuple[int, ...], torch.dtype]]:
+        """Shape and dtype of the fixed-size state each request holds for this mixer."""
+        return None
+
+    def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(x, ctx) -> y, token by token."""
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block:
+    """Wires the parts of one layer: forward(stream, ctx, call) updates the stream."""
+
+    def __init__(self, spec, norms: Dict[str, Norm], mixer: Mixer, ffn: FeedForward):
+        raise NotImplementedError
+
+    def forward(self, stream: HiddenStream, ctx, call: int) -> None:
+        raise NotImplementedError

@@ -1,0 +1,60 @@
+"""Checks a model folder against what the architecture's plan asks for, then builds the model.
+
+Reference: minivllm/models/loader.py:24-29 and qwen3.py:223-245. The reference raises a bare
+``KeyError`` for an unknown tensor name, does not notice missing tensors and leaves a wrong
+shape to ``copy_``. Here every problem of a folder is found before any data is read and is
+reported in one ``WeightError`` that lists missing tensors, unexpected tensors and wrong
+shapes.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..parts.base import TensorDecl
+from .source import DeviceTensors, SafetensorsSource, TensorSource
+
+
+class WeightError(ValueError):
+    def __init__(self, where: str, missing: List[str], unexpected: List[str],
+                 wrong_shape: List[Tuple[str, Tuple[int, ...], Tuple[int, ...]]],
+                 wrong_type: List[Tuple[str, str]]):
+        self.missing, self.unexpected, self.wrong_shape, self.wrong_type = missing, unexpected, wrong_shape, wrong_type
+        lines = [f"the weights in {where} do not fit the model:"]
+        if missing:
+            lines.append(f"  missing tensors ({len(missing)}):")
+            lines += [f"    {n}" for n in missing]
+        if unexpected:
+            lines.append(f"  unexpected tensors ({len(unexpected)}):")
+            lines += [f"    {n}" for n in unexpected]
+        if wrong_shape:
+            lines.append(f"  wrong shapes ({len(wrong_shape)}):")
+            lines += [f"    {n}: found {list(got)}, expected {list(want)}" for n, got, want in wrong_shape]
+        if wrong_type:
+            lines.append(f"  wrong kinds ({len(wrong_type)}):")
+            lines += [f"    {n}: {why}" for n, why in wrong_type]
+        super().__init__("\n".join(lines))
+
+
+def check_tensors(source: TensorSource, expected: Dict[str, TensorDecl], ignorable=frozenset(),
+                  where: str = "the model folder") -> None:
+    have = set(source.names())
+    missing = sorted(n for n in expected if n not in have)
+    unexpected = sorted(n for n in have if n not in expected and n not in ignorable)
+    wrong_shape, wrong_type = [], []
+    for name, decl in expected.items():
+        if name not in have:
+            continue
+        got = tuple(source.shape(name))
+        if got != tuple(decl.shape):
+            wrong_shape.append((name, got, tuple(decl.shape)))
+        if source.is_integer(name) != decl.integer:
+            wrong_type.append((name, "integer tensor where a floating one is expected" if not decl.integer
+                               else "floating tensor where an integer table is expected"))
+    if missing or unexpected or wrong_shape or wrong_type:
+        raise WeightError(where, missing, unexpected, sorted(wrong_shape), sorted(wrong_type))
+
+
+def open_model_folder(model_dir: str) -> TensorSource:
+    return SafetensorsSource(model_dir)

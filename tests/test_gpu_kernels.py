@@ -1,0 +1,341 @@
+"""Each HIP kernel alone against a plain float32/float64 PyTorch reference of the same
+operation, at sizes other than the engine's test models (odd widths, head sizes in steps of
+16, head counts and groups that are no power of two)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+# relative error allowed for one operation: float32 arithmetic vs one bf16 rounding of the result
+OP_TOL = {torch.float32: 2e-6, torch.bfloat16: 6e-3}
+
+
+def ops_for(dtype):
+    from minivllm_amd.kernels.ops import get_ops
+    return get_ops(dtype)
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", DTYPES)
+def test_embedding(dtype, wdtype):
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(0)
+    V, h, n = 301, 72, 19
+    table = torch.randn(V, h, generator=g).to(wdtype)
+    ids = torch.randint(0, V, (n,), generator=g, dtype=torch.int32)
+    resid = torch.full((n, h), 7.0, device="cuda")
+    ops.embedding(dev(ids), dev(table), resid, scale=1.5)
+    want = table.float()[ids.long()] * 1.5
+    assert rel_err(resid.cpu().numpy(), want.numpy()) <= 1e-7
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("h", [72, 1000, 2049])
+def test_add_rmsnorm(dtype, h):
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(1)
+    n, eps = 7, 1e-5
+    resid = torch.randn(n, h, generator=g)
+    delta = torch.randn(n, h, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(h, generator=g)).to(dtype)
+    r_dev, out = dev(resid).clone(), torch.empty(n, h, dtype=dtype, device="cuda")
+    ops.add_rmsnorm(r_dev, dev(delta), dev(w), eps, out)
+    s = resid.double() + delta.double()
+    want = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    assert rel_err(r_dev.cpu().numpy(), s.float().numpy()) <= 1e-7
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[dtype]
+    # rows: only the chosen rows, the residual untouched, a negative row gives zeros
+    rows = torch.tensor([5, -1, 0], dtype=torch.int32)
+    r2, out2 = dev(resid).clone(), torch.empty(3, h, dtype=dtype, device="cuda")
+    ops.add_rmsnorm(r2, dev(delta), dev(w), eps, out2, rows=dev(rows))
+    assert torch.equal(r2.cpu(), resid)
+    assert rel_err(out2[0].float().cpu().numpy(), want[5].numpy()) <= OP_TOL[dtype]
+    assert rel_err(out2[2].float().cpu().numpy(), want[0].numpy()) <= OP_TOL[dtype]
+    assert float(out2[1].float().abs().max()) == 0.0
+    # unit offset: the weight is 1 + w
+    out3 = torch.empty(n, h, dtype=dtype, device="cuda")
+    ops.add_rmsnorm(dev(resid).clone(), None, dev(w), eps, out3, unit_offset=True)
+    r = resid.double()
+    want3 = r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps) * (1 + w.double())
+    assert rel_err(out3.float().cpu().numpy(), want3.numpy()) <= OP_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_strided(dtype):
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(9, 200, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(48, generator=g)).float()       # a weight kept in float32
+    xd = dev(x)
+    view = xd[:, 16:64]
+    out = torch.empty(9, 48, dtype=dtype, device="cuda")
+    ops.rmsnorm(view, dev(w), 1e-6, out)
+    v = x[:, 16:64].double()
+    want = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-6) * w.double()
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[dtype]
+
+
+def test_rope_table():
+    ops = ops_for(torch.float32)
+    rot, theta, max_pos = 48, 50000.0, 700
+    inv = 1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float) / rot))
+    table = ops.rope_table(dev(inv), max_pos).cpu()
+    ang = torch.arange(max_pos, dtype=torch.float)[:, None] * inv[None, :]      # float32 product, as the kernel
+    want = torch.cat([ang.double().cos(), ang.double().sin()], dim=-1)
+    assert table.shape == (max_pos, rot)
+    assert float((table.double() - want).abs().max()) <= 3e-7
+
+
+def paged_cache(num_pages, Hkv, ps, D, dtype):
+    k = torch.zeros(num_pages, Hkv, ps, D, dtype=dtype, device="cuda")
+    v = torch.zeros(num_pages, Hkv, D, ps, dtype=dtype, device="cuda")
+    return k, v
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,D,rot,inter", [(6, 3, 48, 48, False), (5, 5, 16, 8, True), (8, 2, 128, 128, False)])
+def test_qk_norm_rope_store(dtype, H, Hkv, D, rot, inter):
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(3)
+    ps, n = 4, 11
+    eps = 1e-5
+    # two sequences: tokens 0..6 of seq 0 at positions 3..9, tokens 7..10 of seq 1 at positions 0..3
+    positions = torch.tensor(list(range(3, 10)) + list(range(0, 4)), dtype=torch.int32)
+    token_seq = torch.tensor([0] * 7 + [1] * 4, dtype=torch.int32)
+    token_seq[5] = -1                                   # a padding row: nothing may be written for it
+    bt = torch.tensor([[5, 2, 7], [1, -1, -1]], dtype=torch.int32)
+    width = (H + 2 * Hkv) * D
+    qkv = torch.randn(n, width, generator=g).to(dtype)
+    qw = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype)
+    kw = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float) / rot))
+    table = ops.rope_table(dev(inv), 64)
+    kp, vp = paged_cache(9, Hkv, ps, D, dtype)
+    kp.fill_(9.0); vp.fill_(9.0)
+    qkv_dev = dev(qkv).clone()
+    ops.qk_norm_rope_store(qkv_dev, H, Hkv, D, dev(positions), dev(token_seq), dev(qw), dev(kw), eps, table, inter,
+                           kp, vp, dev(bt), ps)
+
+    def norm_rope(x, w):           # x [n, heads, D] float64
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+        ang = positions.double()[:, None] * inv.double()[None, :]
+        c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        y = x.clone()
+        half = rot // 2
+        if inter:
+            a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+            y[..., 0:rot:2] = a * c - b * s
+            y[..., 1:rot:2] = b * c + a * s
+        else:
+            a, b = x[..., :half], x[..., half:rot]
+            y[..., :half] = a * c - b * s
+            y[..., half:rot] = b * c + a * s
+        return y
+
+    q = qkv[:, :H * D].double().view(n, H, D)
+    k = qkv[:, H * D:(H + Hkv) * D].double().view(n, Hkv, D)
+    v = qkv[:, (H + Hkv) * D:].double().view(n, Hkv, D)
+    q_want, k_want = norm_rope(q, qw), norm_rope(k, kw)
+    got_q = qkv_dev[:, :H * D].float().cpu().view(n, H, D)
+    tol = max(OP_TOL[dtype], 3e-6)      # the table's angles are float32
+    live = [i for i in range(n) if token_seq[i] >= 0]
+    assert rel_err(got_q[live].numpy(), q_want[live].numpy()) <= tol
+    assert torch.equal(got_q[5], qkv[5, :H * D].float().view(H, D))          # padding row untouched
+    kc, vc = kp.float().cpu(), vp.float().cpu()
+    written = set()
+    for i in live:
+        page = int(bt[token_seq[i], positions[i] // ps]); slot = int(positions[i] % ps)
+        written.add((page, slot))
+        assert rel_err(kc[page, :, slot, :].numpy(), k_want[i].numpy()) <= tol
+        assert rel_err(vc[page, :, :, slot].numpy(), v[i].to(dtype).double().numpy()) <= 1e-7
+    for page in range(9):
+        for slot in range(ps):
+            if (page, slot) not in written:
+                assert float((kc[page, :, slot, :] - 9.0).abs().max()) == 0.0
+                assert float((vc[page, :, :, slot] - 9.0).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(dtype):
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(4)
+    n, I = 5, 173
+    gu = (3 * torch.randn(n, 2 * I, generator=g)).to(dtype)
+    out = torch.empty(n, I, dtype=dtype, device="cuda")
+    ops.swiglu(dev(gu), out)
+    want = torch.nn.functional.silu(gu[:, :I].double()) * gu[:, I:].double()
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 70, 96), (33, 129, 200), (130, 64, 1000)])
+def test_gemm_exact(dtype, wdtype, M, N, K):
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(wdtype)
+    b = torch.randn(N, generator=g).to(wdtype)
+    want = a.double() @ w.double().T + b.double()
+    for out_dtype in {dtype, torch.float32}:
+        out = torch.empty(M, N, dtype=out_dtype, device="cuda")
+        ops.gemm(dev(a), dev(w), out, dev(b), exact=True)
+        tol = 3e-6 if out_dtype == torch.float32 else OP_TOL[dtype]
+        assert rel_err(out.float().cpu().numpy(), want.numpy()) <= tol
+    # a row's result does not depend on the rows around it
+    out_all = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    out_one = torch.empty(1, N, dtype=torch.float32, device="cuda")
+    ops.gemm(dev(a), dev(w), out_all, exact=True)
+    ops.gemm(dev(a[M - 1:M]), dev(w), out_one, exact=True)
+    assert torch.equal(out_all[M - 1:M], out_one)
+
+
+def reference_attention(q, k_all, v_all, positions, token_seq, H, Hkv, scale, window):
+    """q [n, H, D] float64; k_all/v_all: per sequence [ctx, Hkv, D]."""
+    n, _, D = q.shape
+    out = torch.zeros(n, H, D, dtype=torch.float64)
+    for i in range(n):
+        s = int(token_seq[i])
+        if s < 0:
+            continue
+        p = int(positions[i])
+        lo = 0 if window is None else max(0, p - window)
+        for h in range(H):
+            kh = h // (H // Hkv)
+            keys = k_all[s][lo:p + 1, kh]
+            vals = v_all[s][lo:p + 1, kh]
+            sc = torch.softmax((keys @ q[i, h]) * scale, dim=0)
+            out[i, h] = sc @ vals
+    return out
+
+
+def fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype):
+    kp, vp = paged_cache(num_pages, Hkv, ps, D, dtype)
+    kc, vc = torch.full(kp.shape, float("nan")), torch.full(vp.shape, float("nan"))
+    for s, table in enumerate(tables):
+        for pos in range(k_all[s].shape[0]):
+            page, slot = table[pos // ps], pos % ps
+            if page < 0:
+                continue
+            kc[page, :, slot, :] = k_all[s][pos]
+            vc[page, :, :, slot] = v_all[s][pos]
+    kp.copy_(kc.to(dtype)); vp.copy_(vc.to(dtype))
+    return kp, vp
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,D,ps,window", [(6, 3, 48, 4, None), (4, 1, 16, 8, 9), (8, 2, 128, 16, None),
+                                                (5, 5, 80, 3, 130), (16, 8, 128, 16, 40)])
+def test_attention_general(dtype, H, Hkv, D, ps, window):
+    """Mixed step: a long portion, a short one and single decoded tokens, over pages in
+    scrambled order; unused pages hold NaN."""
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(6)
+    ctx_lens = [150, 37, 1, 290]            # context after the step
+    q_lens = [150, 5, 1, 1]                 # whole prompt, portion, first token, decoded token
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    pages_per = [-(-c // ps) for c in ctx_lens]
+    num_pages = sum(pages_per) + 5
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, cur = [], 0
+    for n_p in pages_per:
+        tables.append(perm[cur:cur + n_p]); cur += n_p
+    if window is not None:                  # pages wholly behind the window of the first query are gone
+        for s, (c, ql) in enumerate(zip(ctx_lens, q_lens)):
+            first_needed = max(0, (c - ql) - window) // ps
+            for i in range(first_needed):
+                tables[s][i] = -1
+    kp, vp = fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype)
+    width = max(pages_per)
+    bt = torch.full((len(tables), width), -1, dtype=torch.int32)
+    for s, t in enumerate(tables):
+        bt[s, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    positions, token_seq = [], []
+    for s, (c, ql) in enumerate(zip(ctx_lens, q_lens)):
+        positions += list(range(c - ql, c)); token_seq += [s] * ql
+    n = len(positions)
+    positions = torch.tensor(positions, dtype=torch.int32)
+    token_seq = torch.tensor(token_seq, dtype=torch.int32)
+    # sharpen: one far key gets a large score for the last query of sequence 3
+    q = torch.randn(n, H, D, generator=g)
+    q[-1] = 6.0 * k_all[3][2 if window is None else 290 - 1 - window].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
+    q = q.to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    # queries live in a wider row, as in the packed qkv buffer
+    qrow = torch.zeros(n, H * D + 24, dtype=dtype)
+    qrow[:, :H * D] = q.view(n, H * D)
+    qd = dev(qrow)
+    out = torch.empty(n, H * D, dtype=dtype, device="cuda")
+    ops.attention(qd[:, :H * D], out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale, window)
+    want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
+    assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= max(OP_TOL[dtype], 5e-6)
+
+
+def test_attention_reduces_to_library_softmax():
+    """One head, no window, whole sequence: equals torch's scaled_dot_product_attention."""
+    ops = ops_for(torch.float32)
+    g = torch.Generator().manual_seed(7)
+    n, D, ps = 45, 32, 16
+    q, k, v = (torch.randn(n, 1, D, generator=g) for _ in range(3))
+    kp, vp = fill_pages([k.double()], [v.double()], [[2, 0, 1]], ps, 1, D, 3, torch.float32)
+    bt = torch.tensor([[2, 0, 1]], dtype=torch.int32)
+    pos = torch.arange(n, dtype=torch.int32)
+    out = torch.empty(n, D, device="cuda")
+    ops.attention(dev(q.view(n, D)), out, kp, vp, dev(bt), ps, dev(pos), dev(torch.zeros(n, dtype=torch.int32)),
+                  1, 1, D, D ** -0.5, None)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(0, 1)[None].double(), k.transpose(0, 1)[None].double(), v.transpose(0, 1)[None].double(),
+        is_causal=True)[0, 0]
+    assert rel_err(out.cpu().numpy(), want.numpy()) <= 3e-6
+
+
+def test_sampling_greedy_and_draws():
+    from plain import qwen3_plain as plain
+    ops = ops_for(torch.float32)
+    g = torch.Generator().manual_seed(8)
+    M, V = 6, 1531
+    logits = (2.5 * torch.randn(M, V, generator=g)).float()
+    logits[1, 7] = logits[1, 900] = logits[1].max() + 1          # a tie: the lowest id wins
+    out = torch.empty(M, dtype=torch.int32, device="cuda")
+    ops.sample(dev(logits), out)
+    want = [int(torch.argmax(logits[i])) for i in range(M)]
+    want[1] = 7
+    assert out.cpu().tolist() == want
+    temps = torch.tensor([0.0, 0.7, 1.0, 1.3, 0.9, 2.0])
+    top_k = torch.tensor([0, 0, 40, 0, 12, 3], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 1.0, 0.8, 0.6, 0.95])
+    for counter in range(4):
+        rng = torch.tensor([[1234 + i, counter] for i in range(M)], dtype=torch.int64)
+        ops.sample(dev(logits), out, dev(temps), dev(top_k), dev(top_p), dev(rng))
+        got = out.cpu().tolist()
+        for i in range(M):
+            tok, score = plain.sample_token(logits[i].numpy(), float(temps[i]), int(top_k[i]), float(top_p[i]),
+                                            seed=1234 + i, counter=counter)
+            # the same token, or one whose perturbed score ties within float rounding
+            assert np.isfinite(score[got[i]]), f"row {i}: token {got[i]} is outside the kept set"
+            assert score[got[i]] >= score[tok] - 1e-4 * max(1.0, abs(float(score[tok]))), (i, got[i], tok)
+
+
+def test_sampling_frequencies():
+    """Draws follow softmax(logits / T) on a small vocabulary."""
+    ops = ops_for(torch.float32)
+    V, T, draws = 11, 0.8, 4000
+    logits = torch.linspace(-2, 2, V)[None].repeat(draws, 1).contiguous()
+    out = torch.empty(draws, dtype=torch.int32, device="cuda")
+    temps = torch.full((draws,), T)
+    rng = torch.tensor([[99, c] for c in range(draws)], dtype=torch.int64)
+    ops.sample(dev(logits), out, dev(temps), None, None, dev(rng))
+    freq = np.bincount(out.cpu().numpy(), minlength=V) / draws
+    p = torch.softmax(logits[0].double() / T, dim=0).numpy()
+    assert np.abs(freq - p).max() < 4 * np.sqrt(p.max() / draws)

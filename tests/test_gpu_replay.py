@@ -1,0 +1,149 @@
+"""The engine against the plain model under every way of cutting the same requests: whole,
+last 32 tokens one by one, portions of changing size down to two tokens, and mixed with other
+requests on so few pages that they are used again; in float32 and in bfloat16, for tiny
+configurations that differ in every size and option."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import trace_tools
+from helpers import TINY, TOL, make_weights, plain_logits, random_tokens, rel_err, write_model_dir
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+STORED = {"A": torch.float32, "B": torch.bfloat16, "C": torch.bfloat16}
+LENGTHS = {"A": [70, 5, 33, 17, 1 + 32, 49], "B": [91, 40, 66, 2, 58, 35], "C": [50, 36, 77]}
+
+
+class Case:
+    def __init__(self, name, tmp, qk_gain=1.0):
+        self.cfg = TINY[name]
+        self.weights = make_weights(self.cfg, seed=sum(map(ord, name)), stored=STORED[name], qk_gain=qk_gain)
+        self.dir = write_model_dir(str(tmp / f"tiny{name}"), self.cfg, self.weights)
+        self.reqs = {f"r{i}": random_tokens(self.cfg, n, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
+        self.want = {rid: plain_logits(self.cfg, self.weights, toks) for rid, toks in self.reqs.items()}
+
+    def check(self, got, dtype, what):
+        worst = 0.0
+        for (rid, pos), row in got.items():
+            worst = max(worst, rel_err(row, self.want[rid][pos]))
+        n_expected = sum(len(t) for t in self.reqs.values())
+        print(f"{what} [{dtype}]: {len(got)} rows, worst relative error {worst:.3e}")
+        assert worst <= TOL[dtype], f"{what}: worst relative error {worst:.3e} exceeds {TOL[dtype]:.1e}"
+        return n_expected
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("models")
+    return {name: Case(name, tmp, qk_gain=2.5) for name in ("A", "B", "C")}
+
+
+def runner_for(case, dtype, steps, page_size=16, use_graph=True, slack=0):
+    from minivllm_amd.engine.trace import TraceRunner
+    return TraceRunner(case.dir, dtype, trace_tools.max_live_tokens(steps) + slack, page_size=page_size,
+                       use_graph=use_graph)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole(cases, name, dtype):
+    case = cases[name]
+    steps = trace_tools.whole(case.reqs)
+    got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+    assert len(got) == case.check(got, dtype, f"tiny {name} whole")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("use_graph", [True, False])
+def test_tail_decode(cases, name, dtype, use_graph):
+    case = cases[name]
+    steps = trace_tools.tail_decode(case.reqs, tail=32)
+    got = trace_tools.collect(steps, runner_for(case, dtype, steps, use_graph=use_graph).run_step)
+    case.check(got, dtype, f"tiny {name} last 32 one by one (graph={use_graph})")
+    for rid, toks in case.reqs.items():
+        assert (rid, len(toks) - 1) in got
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("page_size", [16, 4])
+def test_portions(cases, name, dtype, page_size):
+    case = cases[name]
+    steps = trace_tools.portions(case.reqs)
+    got = trace_tools.collect(steps, runner_for(case, dtype, steps, page_size=page_size).run_step)
+    assert len(got) == case.check(got, dtype, f"tiny {name} portions (page {page_size})")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed(cases, name, dtype):
+    case = cases[name]
+    prompt_lens = {rid: max(2, len(t) - 12) if len(t) > 3 else len(t) for rid, t in case.reqs.items()}
+    for seed in (0, 1):
+        steps = trace_tools.mixed(case.reqs, prompt_lens, max_live=4 if name != "C" else 2, seed=seed)
+        runner = runner_for(case, dtype, steps)
+        got = trace_tools.collect(steps, runner.run_step)
+        assert len(got) == case.check(got, dtype, f"tiny {name} mixed seed {seed}")
+        runner.manager.check_invariants()
+        assert not runner.manager.seqs                       # everything was given back
+        for pool in runner.manager.pools:
+            assert pool.num_free == pool.num_pages
+
+
+def test_first_tokens_and_single_token_requests(cases):
+    """The first positions of a sequence, and requests of one and two tokens."""
+    case = cases["A"]
+    reqs = {"one": case.reqs["r0"][:1], "two": case.reqs["r0"][:2], "three": case.reqs["r1"][:3]}
+    steps = trace_tools.whole(reqs)
+    for dtype in ("float32", "bfloat16"):
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+        for (rid, pos), row in got.items():
+            src = "r0" if rid in ("one", "two") else "r1"
+            assert rel_err(row, case.want[src][pos]) <= TOL[dtype]
+
+
+def test_long_decoding(cases):
+    """One token after another from the very first, 300 of them, across many pages."""
+    case = cases["B"]
+    toks = random_tokens(case.cfg, 300, seed=77)
+    want = plain_logits(case.cfg, case.weights, toks)
+    steps = [{"step": p, "entries": [{"id": "x", "tokens": [toks[p]], "want": [0]}], "end": []} for p in range(300)]
+    for dtype in ("float32", "bfloat16"):
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+        worst = max(rel_err(got[("x", p)], want[p]) for p in range(300))
+        print(f"long decoding [{dtype}]: worst relative error {worst:.3e}")
+        assert worst <= TOL[dtype]
+
+
+def test_trace_run_program(cases, tmp_path):
+    """bin/trace_run as a user calls it: steps on standard input, logits in files."""
+    case = cases["A"]
+    prompt_lens = {rid: max(2, len(t) - 6) for rid, t in case.reqs.items()}
+    steps = trace_tools.mixed(case.reqs, prompt_lens, max_live=3, seed=5)
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / f"out_{dtype}"
+        proc = subprocess.run(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", case.dir, "--dtype", dtype,
+             "--out", str(out), "--max-tokens", str(trace_tools.max_live_tokens(steps))],
+            input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-4000:]
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {s['step']}" for s in steps]
+
+        def read(step):
+            path = out / f"{step['step']}.f32"
+            n = sum(len(e["want"]) for e in step["entries"])
+            if n == 0:
+                assert not path.exists()
+                return None
+            return np.fromfile(path, dtype="<f4").reshape(n, case.cfg["vocab_size"])
+
+        got = trace_tools.collect(steps, read)
+        case.check(got, dtype, "bin/trace_run mixed")
