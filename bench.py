@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X, with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 0.6b|8b|32b] [--batch B] ...
+
+The default run has the layer sizes of the Qwen3-0.6B shape (28 layers, hidden 1024, 16 query
+heads, 8 key/value heads, head_dim 128, intermediate 3072, vocabulary 151936, tied head), a
+batch of 8 requests with 1,024-token prompts inside a 4,096-token context limit, bfloat16. A
+"step" is one decode step of the whole engine (schedule, run the batch from a HIP graph,
+sample, update). W warm-up steps, then exactly K timed steps between synchronisations. One
+JSON line is printed:
+
+  value        decoded tokens per second at the default batch
+  prefill      one 2,048-token prompt run whole: tokens/s, ms, and its share of the bf16 MFMA peak
+  roofline     bytes the decode step has to read (every weight once, the live requests' cache)
+               divided by its time, against 8 TB/s of HBM
+  points       decode tokens/s at batch 1 and batch 64
+
+Weights are seeded random tensors of the named shape and prompts are seeded uniform token ids
+(there is no network for checkpoints or datasets). The reference publishes no number for this
+metric, so ``vs_baseline`` is null.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+SHAPES = {
+    "0.6b": dict(num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+                 intermediate_size=3072, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
+                 tie_word_embeddings=True),
+    "8b": dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
+               tie_word_embeddings=False),
+    "32b": dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                intermediate_size=25600, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
+                tie_word_embeddings=False),
+}
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+
+def model_numbers(c, layers):
+    h, I, V = c["hidden_size"], c["intermediate_size"], c["vocab_size"]
+    q, kv = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
+    layer_params = h * (q + 2 * kv) + q * h + 3 * h * I + 2 * h + 2 * c["head_dim"]
+    matrix_params = layers * (h * (q + 2 * kv) + q * h + 3 * h * I)
+    return dict(layer_params=layer_params, step_params=layers * layer_params + h + V * h,
+                matrix_params=matrix_params, kv_bytes_per_token=layers * 2 * kv)
+
+
+def build_llm(args, shape, layers):
+    import torch
+    from minivllm_amd import LLM
+    from minivllm_amd.config import EngineConfig
+    from minivllm_amd.models import config_from_dict, expected_tensors
+    from minivllm_amd.weights.device_random import DeviceRandomSource
+
+    raw = dict(shape, architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers,
+               max_position_embeddings=40960, torch_dtype=args.dtype)
+    arch, cfg = config_from_dict(raw)
+    dev = torch.device("cuda:0")
+    stored = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    source = DeviceRandomSource(expected_tensors(arch, cfg), args.seed, stored, dev)
+    pages_per_seq = -(-args.context // args.block_size)
+    ec = EngineConfig(model="", dtype=args.dtype, max_model_len=args.context,
+                      max_num_batched_tokens=max(args.prefill_tokens, 2048), max_num_batched_seqs=max(64, args.batch),
+                      kv_cache_block_size=args.block_size,
+                      kv_cache_num_blocks=max(64, args.batch) * pages_per_seq + 16,
+                      use_cuda_graph=not args.no_graph, seed=args.seed)
+    return LLM(config=ec, model_source=(arch, cfg, source)), cfg
+
+
+def random_prompt(vocab, n, seed):
+    import numpy as np
+    return [int(t) for t in np.random.default_rng(seed).integers(0, vocab, size=n)]
+
+
+def measure_decode(llm, vocab, batch, prompt_len, steps, warmup, seed):
+    """Tokens per second of ``steps`` decode steps at ``batch`` after the prompts are in the cache."""
+    import torch
+    from minivllm_amd import SamplingParams
+    sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8, ignore_eos=True)
+    reqs = [llm.submit(random_prompt(vocab, prompt_len, seed + i), sp) for i in range(batch)]
+    while any(r.num_completion_tokens == 0 for r in reqs):          # prompts in, first token drawn
+        llm.step()
+    for _ in range(warmup):
+        llm.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        llm.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mean_ctx = prompt_len + 1 + warmup + steps / 2.0
+    # finish and free
+    for r in reqs:
+        r.sampling_params.max_tokens = r.num_completion_tokens
+    while llm.has_unfinished():
+        llm.step()
+    return batch * steps / dt, dt / steps * 1e3, mean_ctx
+
+
+def measure_prefill(llm, vocab, tokens, repeats, seed):
+    import torch
+    from minivllm_amd import SamplingParams
+    times = []
+    for i in range(repeats + 1):
+        r = llm.submit(random_prompt(vocab, tokens, seed + 100 + i), SamplingParams(temperature=0.0, max_tokens=1,
+                                                                                     ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while not r.finished:
+            llm.step()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    return min(times[1:]) if repeats else times[0]
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="0.6b")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in the record)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=1024)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    if args.prompt_len + args.warmup + args.steps + 16 > args.context:
+        print(f"bench.py: prompt {args.prompt_len} + {args.warmup + args.steps} steps exceed the context {args.context}")
+        return 2
+
+    import torch
+    shape = SHAPES[args.shape]
+    layers_full = shape["num_hidden_layers"]
+    layers = args.layers or layers_full
+    llm, cfg = build_llm(args, shape, layers)
+    nums = model_numbers(shape, layers)
+    item = 2 if args.dtype == "bfloat16" else 4
+
+    prefill_s = measure_prefill(llm, cfg.vocab_size, args.prefill_tokens, repeats=3, seed=args.seed)
+    T = args.prefill_tokens
+    attn_flops = layers * 2 * cfg.num_attention_heads * cfg.head_dim * T * T       # causal half of 4 H D T^2
+    prefill_flops = 2 * T * nums["matrix_params"] + attn_flops + 2 * cfg.vocab_size * cfg.hidden_size
+    prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+               "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+
+    tok_s, ms_step, mean_ctx = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len, args.steps,
+                                              args.warmup, args.seed)
+    step_bytes = nums["step_params"] * item + args.batch * mean_ctx * nums["kv_bytes_per_token"] * item
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(achieved / PEAK_HBM_GBS, 4)}
+
+    points = {}
+    if not args.no_points:
+        for b, key in ((1, "decode_b1"), (64, "decode_b64")):
+            n = min(args.steps, 128)
+            v, _, _ = measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8), args.seed + b)
+            points[key] = round(v, 1)
+
+    config = {"model": f"qwen3-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
+              "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+              "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+              "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch, "seq_len": args.context,
+              "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
+              "parallelism": "single-gpu"}
+    line = {"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
+            "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic", "config": config,
+            "prefill": prefill, "roofline": roofline, "points": points}
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -106,6 +106,14 @@ class CacheManager:
         total = -(-(seq.num_computed + num_new_tokens) // self.page_size)
         return [max(0, total - len(seq.pages[g])) for g in range(len(self.groups))]
 
+    def reservable_tokens(self, req) -> int:
+        """How many more positions the request could be given right now: room left in its last
+        pages plus what the free pages of the tightest group hold."""
+        seq = self.seqs[req]
+        room = min((len(seq.pages[g]) + self.pools[g].num_free) * self.page_size
+                   for g in range(len(self.groups))) if self.groups else 1 << 60
+        return max(0, room - seq.num_computed)
+
     def can_reserve(self, req, num_new_tokens: int) -> bool:
         return all(n <= self.pools[g].num_free for g, n in enumerate(self.pages_needed(req, num_new_tokens)))
 

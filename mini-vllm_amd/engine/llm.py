@@ -1,0 +1,162 @@
+"""The Python entry point: ``LLM(model=...).generate(prompts, sampling_params)``.
+
+Reference: minivllm/engine/engine.py — ``Engine(config)`` with ``submit`` / ``step`` /
+``finished`` / ``generate``; ``generate`` takes prompts as lists of token ids and one
+``SamplingParams`` or a list, steps until everything finished and returns, in order of
+submission, one record per request with the keys ``prompt``, ``completion`` and ``tokens``
+(engine.py:40-90). Those names are kept (``RequestOutput`` also answers to them); prompts may
+also be strings when the model folder holds a tokenizer. ``step`` runs one mixed batch:
+schedule, execute, sample, update.
+"""
+from __future__ import annotations
+
+import logging
+import time
+from typing import Dict, List, Optional, Sequence, Tuple, Union
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..config.sampling_params import SamplingParams
+from ..sampling.sampler import Sampler, request_seed
+from .executor import Executor
+from .metrics import Metrics
+from .request import Request, RequestOutput
+from .scheduler import ScheduledStep, Scheduler
+from .step import SeqStep
+
+logger = logging.getLogger(__name__)
+
+
+def _load_tokenizer(model_dir: str):
+    """The tokenizer stored in the model folder, or None (random-weight models have none)."""
+    import os
+    if not model_dir or not any(os.path.isfile(os.path.join(model_dir, f))
+                                for f in ("tokenizer.json", "tokenizer_config.json", "vocab.json")):
+        return None
+    try:
+        from transformers import AutoTokenizer
+        return AutoTokenizer.from_pretrained(model_dir, use_fast=True)
+    except Exception as e:  # a tokenizer is optional
+        logger.warning("could not load a tokenizer from %s: %s", model_dir, e)
+        return None
+
+
+class LLM:
+    def __init__(self, model: Optional[str] = None, config: Optional[EngineConfig] = None,
+                 model_source: Optional[Tuple] = None, **options):
+        """``LLM(model="/path", max_num_batched_tokens=2048, ...)`` or ``LLM(config=EngineConfig(...))``.
+        ``model_source`` = (architecture, model config, tensor source) serves tensors that are not
+        in a folder."""
+        if config is None:
+            config = EngineConfig(model=model or "", **options)
+        elif model is not None or options:
+            raise ValueError("give either a config or a model path with options")
+        self.config = config
+        self.tokenizer = _load_tokenizer(config.model)
+        self.executor = Executor(config, model=model_source)
+        self.manager = self.executor.new_cache_manager()
+        eos = config.eos_token_ids
+        if eos is None:
+            eos = tuple(getattr(self.executor.model_config, "eos_token_ids", ()))
+        self.scheduler = Scheduler(self.manager, config.max_num_batched_tokens, config.max_num_batched_seqs,
+                                   config.max_model_len, eos, config.prefill_chunk)
+        self.sampler = Sampler(self.executor.ops, self.executor.device)
+        self.metrics = Metrics()
+        self._seeds: Dict[int, int] = {}
+
+    # ---- the reference's streaming interface ---------------------------------------------
+    def submit(self, tokens: Sequence[int], sampling_params: Optional[SamplingParams] = None) -> Request:
+        req = Request(list(tokens), sampling_params)
+        vocab = self.executor.vocab_size
+        if any((t < 0 or t >= vocab) for t in req.tokens):
+            raise ValueError(f"prompt token ids must lie in [0, {vocab})")
+        self.scheduler.submit(req)
+        self._seeds[req.id] = request_seed(self.config.seed, req.id, req.sampling_params)
+        return req
+
+    add_request = submit
+
+    @property
+    def finished(self) -> bool:
+        return self.scheduler.finished
+
+    def has_unfinished(self) -> bool:
+        return not self.scheduler.finished
+
+    def step(self) -> Optional[ScheduledStep]:
+        """One step of the engine: schedule, run the batch, draw tokens, record them."""
+        t0 = time.perf_counter()
+        step = self.scheduler.schedule()
+        if step is None:
+            return None
+        groups = range(len(self.manager.groups))
+        seqs = []
+        for s in step.seqs:
+            r = s.request
+            cache = self.manager.sequence(r.id)
+            seqs.append(SeqStep(tokens=r.tokens[s.start:s.start + s.num_tokens], start=s.start,
+                                block_tables=[cache.pages[g] for g in groups], state_slot=cache.state_slot,
+                                want=[s.num_tokens - 1] if s.sample else []))
+        logits = self.executor.step(seqs)
+        drawing = [s.request for s in step.seqs if s.sample]
+        tokens = self.sampler.sample(logits, [r.sampling_params for r in drawing],
+                                     [self._seeds[r.id] for r in drawing],
+                                     [r.num_completion_tokens for r in drawing])
+        it = iter(tokens)
+        sampled = [next(it) if s.sample else None for s in step.seqs]
+        preempted_before = self.scheduler.num_preemptions
+        done = self.scheduler.update(step, sampled)
+        for r in done:
+            self._seeds.pop(r.id, None)
+        self.metrics.update(step, done, time.perf_counter() - t0)
+        self.metrics.preemptions = self.scheduler.num_preemptions
+        step.finished = done
+        return step
+
+    # ---- batch generation ---------------------------------------------------------------------
+    def _encode(self, prompt: Union[str, Sequence[int]]) -> List[int]:
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise ValueError("a text prompt needs a tokenizer in the model folder; pass token ids instead")
+            return list(self.tokenizer.encode(prompt))
+        return list(prompt)
+
+    def generate(self, prompts: Sequence[Union[str, Sequence[int]]],
+                 sampling_params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 use_tqdm: bool = True) -> List[RequestOutput]:
+        if sampling_params is None:
+            sampling_params = SamplingParams()
+        if not isinstance(sampling_params, (list, tuple)):
+            sampling_params = [sampling_params] * len(prompts)
+        if len(sampling_params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt is needed")
+        requests = [self.submit(self._encode(p), sp) for p, sp in zip(prompts, sampling_params)]
+        pbar = None
+        if use_tqdm:
+            try:
+                from tqdm.auto import tqdm
+                pbar = tqdm(total=len(prompts), desc="Generating", dynamic_ncols=True)
+            except ImportError:
+                pbar = None
+        finished_before = self.metrics.finished_request_count
+        while not self.finished:
+            self.step()
+            if pbar is not None:
+                s = self.metrics.stats()
+                pbar.set_postfix({"Prefill(token/s)": f"{s.prefill_throughput:4.0f}",
+                                  "Decode(token/s)": f"{s.decode_throughput:4.0f}",
+                                  "TTFT": f"{s.time_to_first_token:4.2f}", "ITL": f"{s.inter_token_latency:4.4f}",
+                                  "TPS": f"{s.tokens_per_second:4.2f}", "RPS": f"{s.requests_per_second:4.2f}"})
+                pbar.update(s.finished_requests - finished_before - pbar.n)
+        if pbar is not None:
+            pbar.close()
+        return [self._output(r) for r in sorted(requests, key=lambda r: r.id)]
+
+    def _output(self, r: Request) -> RequestOutput:
+        prompt_text = completion_text = None
+        if self.tokenizer is not None:
+            prompt_text = self.tokenizer.decode(r.prompt_tokens)
+            completion_text = self.tokenizer.decode(r.completion_tokens)
+        return RequestOutput(request_id=r.id, prompt_token_ids=r.prompt_tokens, token_ids=r.completion_tokens,
+                             finish_reason=r.finish_reason, prompt=prompt_text, text=completion_text)

@@ -113,5 +113,20 @@ def rel_err(got: np.ndarray, want: np.ndarray) -> float:
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
 
 
-# tolerances on rel_err of logits against the float64 plain model
-TOL = {"float32": 3e-5, "bfloat16": 4e-2}
+def plain_logits_bf16(cfg: Dict, weights: Dict[str, torch.Tensor], tokens: List[int]) -> np.ndarray:
+    """The plain model with every stored activation rounded to bfloat16."""
+    return plain.forward(cfg, weights, tokens, dtype=torch.float64, rnd=plain.round_to_bfloat16).numpy()
+
+
+# Tolerance on rel_err of float32 logits against the float64 plain model.
+TOL_F32 = 3e-5
+# bfloat16: how far rounding moves the logits depends on the model and the input (sharp attention
+# amplifies it). The bound is therefore taken from the case itself: the error that bfloat16
+# storage alone causes in the plain model (plain_logits_bf16 against plain_logits), with a
+# factor for the different order of roundings, plus a floor.
+BF16_FACTOR = 1.5
+BF16_FLOOR = 5e-3
+
+
+def bf16_tolerance(emulation_error: float) -> float:
+    return BF16_FACTOR * emulation_error + BF16_FLOOR

@@ -28,11 +28,13 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 
 def rope_cos_sin(positions: torch.Tensor, rotary_dim: int, theta: float, dtype=torch.float64):
     """minivllm/models/layers/rotary.py:35-46 — inv_freq = 1 / theta^(arange(0, d, 2) / d),
-    freqs = position (outer) inv_freq, table = cat(cos, sin). Returns (cos, sin), each
+    freqs = position (outer) inv_freq, table = cat(cos, sin). The reference evaluates inv_freq
+    and the angles in float32 (``dtype=torch.float``, rotary.py:35,38); so does this, and then
+    takes cosine and sine of those float32 angles in ``dtype``. Returns (cos, sin), each
     [n, rotary_dim / 2]."""
-    inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=dtype) / rotary_dim))
-    freqs = torch.einsum("i,j->ij", positions.to(dtype), inv_freq)
-    return freqs.cos(), freqs.sin()
+    inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float) / rotary_dim))
+    freqs = torch.einsum("i,j->ij", positions.to(torch.float), inv_freq)
+    return freqs.to(dtype).cos(), freqs.to(dtype).sin()
 
 
 def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
@@ -68,11 +70,13 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
     return out
 
 
-def swiglu_mlp(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor) -> torch.Tensor:
+def swiglu_mlp(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
+               rnd=None) -> torch.Tensor:
     """minivllm/models/models/qwen3.py:116-121 — down(silu(gate(x)) * up(x)), no biases."""
-    gate = x @ gate_w.T
-    up = x @ up_w.T
-    return (gate * torch.sigmoid(gate) * up) @ down_w.T
+    rnd = rnd or (lambda t: t)
+    gate = rnd(x @ gate_w.T)
+    up = rnd(x @ up_w.T)
+    return rnd(rnd(gate * torch.sigmoid(gate) * up) @ down_w.T)
 
 
 def layer_window(cfg: Dict, layer: int) -> Optional[int]:
@@ -84,8 +88,17 @@ def layer_window(cfg: Dict, layer: int) -> Optional[int]:
     return None
 
 
+def _identity(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
+def round_to_bfloat16(x: torch.Tensor) -> torch.Tensor:
+    """What storing an activation in bfloat16 does to it."""
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
 def attention_block(cfg: Dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tensor,
-                    positions: torch.Tensor) -> torch.Tensor:
+                    positions: torch.Tensor, rnd=_identity) -> torch.Tensor:
     """minivllm/models/models/qwen3.py:73-101 — q/k/v projections, view as heads, RMSNorm of q
     and k over head_dim with one weight per projection (qwen3.py:64-65,89-90), rotary embedding
     (qwen3.py:92), attention, output projection."""
@@ -100,6 +113,7 @@ def attention_block(cfg: Dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tens
         q = q + w[p + "q_proj.bias"]
         k = k + w[p + "k_proj.bias"]
         v = v + w[p + "v_proj.bias"]
+    q, k, v = rnd(q), rnd(k), rnd(v)
     n = x.shape[0]
     q = q.view(n, H, d)
     k = k.view(n, Hkv, d)
@@ -107,39 +121,44 @@ def attention_block(cfg: Dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tens
     q = rms_norm(q, w[p + "q_norm.weight"], eps)
     k = rms_norm(k, w[p + "k_norm.weight"], eps)
     cos, sin = rope_cos_sin(positions, d, cfg.get("rope_theta", 10000.0), dtype=x.dtype)
-    q = apply_rope(q, cos, sin)
-    k = apply_rope(k, cos, sin)
-    o = causal_attention(q, k, v, d ** -0.5, layer_window(cfg, i))
+    q = rnd(apply_rope(q, cos, sin))
+    k = rnd(apply_rope(k, cos, sin))
+    o = rnd(causal_attention(q, k, v, d ** -0.5, layer_window(cfg, i)))
     o = o.reshape(n, H * d) @ w[p + "o_proj.weight"].T
     if cfg.get("attention_bias"):
         o = o + w[p + "o_proj.bias"]
-    return o
+    return rnd(o)
 
 
 def decoder_layer(cfg: Dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tensor,
-                  positions: torch.Tensor) -> torch.Tensor:
+                  positions: torch.Tensor, rnd=_identity) -> torch.Tensor:
     """minivllm/models/models/qwen3.py:141-156 — x += attn(input_layernorm(x));
     x += mlp(post_attention_layernorm(x))."""
     eps = cfg.get("rms_norm_eps", 1e-6)
     p = f"model.layers.{i}."
-    x = x + attention_block(cfg, w, i, rms_norm(x, w[p + "input_layernorm.weight"], eps), positions)
-    h = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
-    x = x + swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    x = x + attention_block(cfg, w, i, rnd(rms_norm(x, w[p + "input_layernorm.weight"], eps)), positions, rnd)
+    h = rnd(rms_norm(x, w[p + "post_attention_layernorm.weight"], eps))
+    x = x + swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                       w[p + "mlp.down_proj.weight"], rnd)
     return x
 
 
 def forward(cfg: Dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=torch.float64,
-            first_position: int = 0) -> torch.Tensor:
+            first_position: int = 0, rnd=_identity) -> torch.Tensor:
     """minivllm/models/models/qwen3.py:178-190,206-220 — embed, layers, final norm, head (tied
     to the embedding when ``tie_word_embeddings``, qwen3.py:203-204). Returns the logits of every
-    position, [n, vocab]. ``first_position`` shifts all positions (for invariance tests)."""
+    position, [n, vocab]. ``first_position`` shifts all positions (for invariance tests).
+    ``rnd`` is applied to every activation a reduced-precision implementation would store
+    (outputs of projections, norms, rotary embedding, attention, activation); with
+    ``round_to_bfloat16`` the result shows how far bfloat16 storage alone moves the logits of
+    this model and input, which is what an engine's bfloat16 error is measured against."""
     w = {k: v.to(dtype) for k, v in weights.items()}
     ids = torch.tensor(tokens, dtype=torch.long)
     positions = torch.arange(first_position, first_position + len(tokens))
     x = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
-        x = decoder_layer(cfg, w, i, x, positions)
-    x = rms_norm(x, w["model.norm.weight"], cfg.get("rms_norm_eps", 1e-6))
+        x = decoder_layer(cfg, w, i, x, positions, rnd)
+    x = rnd(rms_norm(x, w["model.norm.weight"], cfg.get("rms_norm_eps", 1e-6)))
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
     return x @ head.T
 

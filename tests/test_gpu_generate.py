@@ -1,0 +1,173 @@
+"""Generation through the Python entry point against the plain model: greedy and seeded
+temperature sampling, chunked prompts, few pages (preemption), prefix reuse, graphs."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (TINY, TOL_F32, bf16_tolerance, make_weights, plain_logits, plain_logits_bf16, random_tokens,
+                     rel_err, write_model_dir)
+from plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("gen_models")
+    out = {}
+    for name, stored in (("A", torch.float32), ("B", torch.bfloat16)):
+        cfg = TINY[name]
+        w = make_weights(cfg, seed=40 + ord(name), stored=stored, qk_gain=1.5)
+        out[name] = (cfg, w, write_model_dir(str(tmp / name), cfg, w))
+    return out
+
+
+def check_against_plain(cfg, w, outputs, params, dtype, seeds=None):
+    """Every generated token must be the plain model's choice at its position, given the tokens
+    before it (or tie with it within the logits' tolerance)."""
+    for i, out in enumerate(outputs):
+        seq = list(out.prompt_token_ids) + list(out.token_ids)
+        logits = plain_logits(cfg, w, seq)
+        tol = TOL_F32 if dtype == "float32" else bf16_tolerance(
+            max(rel_err(plain_logits_bf16(cfg, w, seq)[p], logits[p]) for p in range(len(seq))))
+        sp = params[i]
+        for t, tok in enumerate(out.token_ids):
+            row = logits[len(out.prompt_token_ids) + t - 1]
+            slack = 2 * tol * float(np.abs(row).max()) / max(sp.temperature, 1.0 if sp.temperature == 0 else 1e-3)
+            want, score = plain.sample_token(row, sp.temperature, sp.top_k, sp.top_p,
+                                             seed=0 if seeds is None else seeds[i], counter=t)
+            assert np.isfinite(score[tok]), f"request {i} token {t}: {tok} is outside the kept set"
+            assert score[tok] >= score[want] - slack, \
+                f"request {i} token {t}: engine drew {tok} (score {score[tok]}), plain {want} (score {score[want]})"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_tiny_a(models, dtype):
+    from minivllm_amd import LLM, SamplingParams
+    cfg, w, path = models["A"]
+    llm = LLM(model=path, dtype=dtype, kv_cache_block_size=16, kv_cache_num_blocks=32, max_model_len=128,
+              max_num_batched_tokens=64, max_num_batched_seqs=8)
+    prompts = [random_tokens(cfg, n, seed=n) for n in (5, 17, 33, 1)]
+    sp = SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)
+    outs = llm.generate(prompts, sp, use_tqdm=False)
+    assert [o.prompt_token_ids for o in outs] == prompts
+    assert all(len(o.token_ids) == 8 and o.finish_reason == "length" for o in outs)
+    assert outs[0]["tokens"] == outs[0].token_ids          # the reference's record keys
+    check_against_plain(cfg, w, outs, [sp] * 4, dtype)
+    llm.manager.check_invariants()
+    assert all(p.num_free == p.num_pages for p in llm.manager.pools)
+    # the same prompts again, each alone: identical tokens whatever the batch was
+    for p, o in zip(prompts, outs):
+        alone = llm.generate([p], sp, use_tqdm=False)[0]
+        if dtype == "float32":
+            assert alone.token_ids == o.token_ids
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sampled_generation_tiny_b_chunked(models, dtype):
+    """Block size 8, prompt portions of 7, requests arriving over the steps, temperature 0.8
+    with seeds, top-k/top-p on some."""
+    from minivllm_amd import LLM, SamplingParams
+    cfg, w, path = models["B"]
+    llm = LLM(model=path, dtype=dtype, kv_cache_block_size=8, kv_cache_num_blocks=40, max_model_len=96,
+              max_num_batched_tokens=24, max_num_batched_seqs=4, prefill_chunk=7, seed=5)
+    lengths = [1, 40, 9, 23, 16, 31]
+    prompts = [random_tokens(cfg, n, seed=200 + n) for n in lengths]
+    params = [SamplingParams(temperature=0.8, max_tokens=12, ignore_eos=True, seed=1000 + i,
+                             top_k=(20 if i % 3 == 1 else 0), top_p=(0.9 if i % 3 == 2 else 1.0))
+              for i in range(len(prompts))]
+    reqs = []
+    pending = list(zip(prompts, params))
+    while pending or llm.has_unfinished():
+        if pending:                                    # one new request per step
+            p, sp = pending.pop(0)
+            reqs.append(llm.submit(p, sp))
+        llm.step()
+    outs = [llm._output(r) for r in reqs]
+    assert all(len(o.token_ids) == 12 for o in outs)
+    check_against_plain(cfg, w, outs, params, dtype, seeds=[1000 + i for i in range(len(prompts))])
+    assert any(s > 1 for s in [llm.metrics.steps])
+    # a request's draws do not depend on the batch: alone it gives the same tokens
+    if dtype == "float32":
+        for p, sp, o in zip(prompts, params, outs):
+            assert llm.generate([p], sp, use_tqdm=False)[0].token_ids == o.token_ids
+
+
+def test_preemption_gives_the_same_tokens(models):
+    from minivllm_amd import LLM, SamplingParams
+    cfg, w, path = models["A"]
+    prompts = [random_tokens(cfg, n, seed=300 + n) for n in (30, 25, 20, 28, 12)]
+    sp = SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True)
+    roomy = LLM(model=path, dtype="float32", kv_cache_block_size=4, kv_cache_num_blocks=200, max_model_len=64,
+                max_num_batched_tokens=48, max_num_batched_seqs=8)
+    want = [o.token_ids for o in roomy.generate(prompts, sp, use_tqdm=False)]
+    assert roomy.scheduler.num_preemptions == 0
+    tight = LLM(model=path, dtype="float32", kv_cache_block_size=4, kv_cache_num_blocks=34, max_model_len=64,
+                max_num_batched_tokens=48, max_num_batched_seqs=8)
+    got = [o.token_ids for o in tight.generate(prompts, sp, use_tqdm=False)]
+    assert tight.scheduler.num_preemptions > 0, "the pool was not tight enough to preempt"
+    assert got == want
+    tight.manager.check_invariants()
+
+
+def test_prefix_reuse_gives_the_same_tokens(models):
+    from minivllm_amd import LLM, SamplingParams
+    cfg, w, path = models["A"]
+    shared = random_tokens(cfg, 16, seed=1)
+    prompts = [shared + random_tokens(cfg, n, seed=400 + n) for n in (3, 9)] + [shared]
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    plain_llm = LLM(model=path, dtype="float32", kv_cache_block_size=16, kv_cache_num_blocks=32, max_model_len=64)
+    want = [o.token_ids for o in plain_llm.generate(prompts, sp, use_tqdm=False)]
+    llm = LLM(model=path, dtype="float32", kv_cache_block_size=16, kv_cache_num_blocks=32, max_model_len=64,
+              enable_prefix_caching=True)
+    first = llm.generate(prompts[:1], sp, use_tqdm=False)
+    rest = llm.generate(prompts[1:], sp, use_tqdm=False)
+    assert [o.token_ids for o in first + rest] == want
+    assert llm.manager.prefix_caching
+    assert llm.metrics.prefill_tokens < plain_llm.metrics.prefill_tokens      # the shared page was not run again
+
+
+def test_eos_and_max_model_len(models):
+    from minivllm_amd import LLM, SamplingParams
+    cfg, w, path = models["A"]
+    llm = LLM(model=path, dtype="float32", kv_cache_num_blocks=16, max_model_len=40)
+    p = random_tokens(cfg, 10, seed=9)
+    free_run = llm.generate([p], SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True), use_tqdm=False)[0]
+    assert len(free_run.token_ids) == 30 and free_run.finish_reason == "length"
+    stop_at = free_run.token_ids[4]
+    llm2 = LLM(model=path, dtype="float32", kv_cache_num_blocks=16, max_model_len=40, eos_token_ids=(stop_at,))
+    stopped = llm2.generate([p], SamplingParams(temperature=0.0, max_tokens=30), use_tqdm=False)[0]
+    n = free_run.token_ids.index(stop_at) + 1
+    assert stopped.token_ids == free_run.token_ids[:n] and stopped.finish_reason == "stop"   # the end token stays
+    with pytest.raises(ValueError, match="max_model_len"):
+        llm.submit(random_tokens(cfg, 40, seed=1))
+    with pytest.raises(ValueError, match="token ids"):
+        llm.submit([cfg["vocab_size"]])
+
+
+def test_graph_replays_match_eager(models):
+    """A captured decode graph is replayed many times, with eager steps of other shapes and
+    synchronisations in between; every replay must give what the eager step gives."""
+    from minivllm_amd.engine.trace import TraceRunner
+    cfg, w, path = models["B"]
+    toks = {f"g{i}": random_tokens(cfg, 60 + 5 * i, seed=500 + i) for i in range(3)}
+    for dtype in ("float32", "bfloat16"):
+        runs = {}
+        for use_graph in (False, True):
+            r = TraceRunner(path, dtype, 512, page_size=16, use_graph=use_graph)
+            rows = []
+            for rid, t in toks.items():
+                r.run_step({"step": 0, "entries": [{"id": rid, "tokens": t[:20], "want": []}], "end": []})
+            for p in range(20, 60):
+                out = r.run_step({"step": p, "entries": [{"id": rid, "tokens": [t[p]], "want": [0]}
+                                                          for rid, t in toks.items()], "end": []})
+                rows.append(out.copy())
+                if p % 7 == 0:          # eager work of another shape between the replays
+                    r.run_step({"step": 1000 + p, "entries": [{"id": f"x{p}", "tokens": toks["g0"][:p % 11 + 2],
+                                                               "want": [0]}], "end": [f"x{p}"]})
+                    torch.cuda.synchronize()
+            runs[use_graph] = np.stack(rows)
+        if dtype == "float32":
+            assert np.array_equal(runs[True], runs[False])
+        else:
+            assert rel_err(runs[True], runs[False]) <= 2e-2

@@ -1,0 +1,225 @@
+"""The scheduler's decisions on the CPU, driven by a fake step function that keeps a simulated
+cache: every page slot remembers the token written to it, and the "model" computes the next
+token from what it reads back through the block tables. A wrong page, a stale page or a lost
+token changes the output."""
+import random
+import zlib
+
+import pytest
+
+from minivllm_amd.cache import CacheManager, GroupSpec
+from minivllm_amd.config import SamplingParams
+from minivllm_amd.engine.request import Request, RequestState
+from minivllm_amd.engine.scheduler import Scheduler
+
+VOCAB = 97
+EOS = 5
+
+
+def next_token(context):
+    """The fake model: a function of the whole context."""
+    return zlib.crc32(bytes(str(list(context)), "ascii")) % VOCAB
+
+
+def expected_output(prompt, max_tokens, ignore_eos=True):
+    toks, out = list(prompt), []
+    while len(out) < max_tokens:
+        t = next_token(toks)
+        toks.append(t); out.append(t)
+        if t == EOS and not ignore_eos:
+            break
+    return out
+
+
+class FakeEngine:
+    def __init__(self, num_pages, page_size, groups=None, max_tokens=64, max_seqs=8, chunk=None, prefix=False,
+                 max_model_len=4096):
+        self.groups = groups or [GroupSpec("full", None, (0,))]
+        self.manager = CacheManager(self.groups, num_pages, page_size, max_seqs, enable_prefix_caching=prefix)
+        self.sched = Scheduler(self.manager, max_tokens, max_seqs, max_model_len, eos_token_ids=(EOS,),
+                               prefill_chunk=chunk)
+        self.ps = page_size
+        self.mem = [dict() for _ in self.groups]          # per group: (page, slot) -> token
+        self.steps = []
+
+    def run_step(self):
+        step = self.sched.schedule()
+        if step is None:
+            return None
+        assert step.num_tokens <= self.sched.max_num_batched_tokens
+        assert len(step.seqs) <= self.sched.max_num_batched_seqs
+        assert len({s.request.id for s in step.seqs}) == len(step.seqs)
+        sampled = []
+        for s in step.seqs:
+            r = s.request
+            seq = self.manager.sequence(r.id)
+            assert s.start == seq.num_computed
+            assert 1 <= s.num_tokens <= len(r.tokens) - s.start
+            for g, spec in enumerate(self.groups):
+                table = seq.pages[g]
+                for pos in range(s.start, s.start + s.num_tokens):
+                    page = table[pos // self.ps]
+                    assert page >= 0
+                    self.mem[g][(page, pos % self.ps)] = r.tokens[pos]
+            if s.sample:
+                end = s.start + s.num_tokens
+                assert end == len(r.tokens)
+                contexts = []
+                for g, spec in enumerate(self.groups):
+                    lo = 0 if spec.retention == "full" else max(0, end - 1 - spec.window)
+                    table = seq.pages[g]
+                    ctx = [self.mem[g][(table[p // self.ps], p % self.ps)] for p in range(lo, end)]
+                    assert ctx == r.tokens[lo:end], "the cache does not hold the request's tokens"
+                    contexts.append(ctx)
+                sampled.append(next_token(contexts[0]))
+            else:
+                sampled.append(None)
+        self.steps.append(step)
+        done = self.sched.update(step, sampled)
+        self.manager.check_invariants()
+        return step, done
+
+    def run_all(self, limit=100000):
+        n = 0
+        while not self.sched.finished:
+            assert self.run_step() is not None
+            n += 1
+            assert n < limit, "the scheduler does not terminate"
+        return n
+
+
+def submit(engine, prompt, **sp):
+    r = Request(prompt, SamplingParams(temperature=0.0, **sp))
+    engine.sched.submit(r)
+    return r
+
+
+def test_mixed_steps_and_token_budget():
+    e = FakeEngine(num_pages=64, page_size=4, max_tokens=16, max_seqs=8)
+    rng = random.Random(1)
+    reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=6, ignore_eos=True)
+            for n in (5, 17, 33, 1)]
+    e.run_all()
+    for r in reqs:
+        assert r.completion_tokens == expected_output(r.prompt_tokens, 6)
+        assert r.finish_reason == "length" and r.state == RequestState.FINISHED
+    # the 33-token prompt was cut into portions under the budget of 16, beside other work
+    long_portions = [s.num_tokens for st in e.steps for s in st.seqs if s.request is reqs[2] and not s.is_decode]
+    assert len(long_portions) >= 3 and sum(long_portions) == 33 and max(long_portions) <= 16
+    assert any(any(s.is_decode for s in st.seqs) and any(not s.is_decode for s in st.seqs) for st in e.steps), \
+        "no step mixed decoded tokens with a prompt portion"
+    assert all(p.num_free == p.num_pages for p in e.manager.pools)
+
+
+def test_prefill_chunk_and_first_come_first_served():
+    e = FakeEngine(num_pages=64, page_size=8, max_tokens=64, max_seqs=2, chunk=7)
+    rng = random.Random(2)
+    reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=3, ignore_eos=True) for n in (20, 9, 4)]
+    e.run_all()
+    for r in reqs:
+        assert r.completion_tokens == expected_output(r.prompt_tokens, 3)
+    assert max(s.num_tokens for st in e.steps for s in st.seqs) <= 7
+    first_step_of = {r.id: next(i for i, st in enumerate(e.steps) if r in st.requests) for r in reqs}
+    assert first_step_of[reqs[0].id] <= first_step_of[reqs[1].id] <= first_step_of[reqs[2].id]
+    # only two requests may run at once: the third waits until one finishes
+    assert all(len(st.seqs) <= 2 for st in e.steps)
+
+
+def test_eos_stops_unless_ignored():
+    # find a prompt whose greedy continuation hits EOS early
+    rng = random.Random(3)
+    while True:
+        prompt = [rng.randrange(VOCAB) for _ in range(6)]
+        out = expected_output(prompt, 40, ignore_eos=False)
+        if len(out) < 40:
+            break
+    e = FakeEngine(num_pages=64, page_size=4)
+    a = submit(e, prompt, max_tokens=40)
+    b = submit(e, prompt, max_tokens=40, ignore_eos=True)
+    e.run_all()
+    assert a.completion_tokens == out and a.completion_tokens[-1] == EOS and a.finish_reason == "stop"
+    assert len(b.completion_tokens) == 40 and b.finish_reason == "length"
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_preemption_under_page_pressure(seed):
+    """So few pages that running requests must give way; every request still gets exactly its
+    tokens, identical to running it alone (minivllm/scheduler/scheduler.py:66-72,91-98)."""
+    rng = random.Random(seed)
+    ps = 4
+    e = FakeEngine(num_pages=14, page_size=ps, max_tokens=32, max_seqs=6)
+    reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(rng.randint(1, 20))], max_tokens=rng.randint(4, 24),
+                   ignore_eos=True) for _ in range(7)]
+    e.run_all()
+    assert e.sched.num_preemptions > 0, "the test did not create page pressure"
+    for r in reqs:
+        assert r.completion_tokens == expected_output(r.prompt_tokens, r.sampling_params.max_tokens)
+    assert all(p.num_free == p.num_pages for p in e.manager.pools) and e.manager.slots.num_free == 6
+
+
+def test_preempted_request_returns_to_the_front_and_the_newest_gives_way():
+    ps = 4
+    e = FakeEngine(num_pages=6, page_size=ps, max_tokens=64, max_seqs=4)
+    a = submit(e, [1] * 7, max_tokens=12, ignore_eos=True)      # may reach 19 tokens = 5 pages
+    b = submit(e, [2] * 7, max_tokens=12, ignore_eos=True)      # together they would need 10 of 6
+    e.run_step()
+    assert [r.id for r in e.sched.running] == [a.id, b.id]
+    c = submit(e, [3] * 3, max_tokens=2, ignore_eos=True)       # arrives later, waits behind a preempted b
+    while b.num_preemptions == 0:
+        e.run_step()
+    assert a.num_preemptions == 0                  # the newer one gave way
+    assert b.state in (RequestState.WAITING, RequestState.RUNNING)
+    if b.state == RequestState.WAITING:
+        assert e.sched.waiting[0] is b and b.id not in e.manager   # back at the front, before c
+    e.run_all()
+    for r in (a, b, c):
+        assert r.completion_tokens == expected_output(r.prompt_tokens, r.sampling_params.max_tokens)
+    assert b.finish_time >= a.finish_time or b.num_preemptions > 0
+
+
+def test_windowed_group_and_recycled_pages():
+    groups = [GroupSpec("full", None, (0,)), GroupSpec("window", 6, (1,))]
+    e = FakeEngine(num_pages=40, page_size=4, groups=groups, max_tokens=24, max_seqs=4)
+    rng = random.Random(5)
+    reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=20, ignore_eos=True) for n in (30, 3, 18, 9, 25)]
+    e.run_all()
+    for r in reqs:
+        assert r.completion_tokens == expected_output(r.prompt_tokens, 20)
+
+
+def test_prefix_reuse_skips_cached_pages():
+    e = FakeEngine(num_pages=64, page_size=4, prefix=True, max_tokens=64)
+    shared = list(range(10, 26))                   # 16 tokens = 4 full pages
+    a = submit(e, shared + [1, 2, 3], max_tokens=4, ignore_eos=True)
+    e.run_all()
+    b = submit(e, shared + [7, 8], max_tokens=4, ignore_eos=True)
+    e.run_step()
+    first = next(s for s in e.steps[-1].seqs if s.request is b)
+    assert first.start == 16 and first.num_tokens == 2          # the shared pages were not run again
+    e.run_all()
+    assert a.completion_tokens == expected_output(a.prompt_tokens, 4)
+    assert b.completion_tokens == expected_output(b.prompt_tokens, 4)
+    # a prompt that is cached entirely still computes its last token
+    c = submit(e, shared, max_tokens=2, ignore_eos=True)
+    e.run_step()
+    first = next(s for s in e.steps[-1].seqs if s.request is c)
+    assert first.start == 12 and first.num_tokens == 4
+    e.run_all()
+    assert c.completion_tokens == expected_output(shared, 2)
+
+
+def test_refused_at_submit():
+    e = FakeEngine(num_pages=4, page_size=4, max_model_len=64)
+    with pytest.raises(ValueError, match="max_model_len"):
+        submit(e, [1] * 64, max_tokens=1)
+    with pytest.raises(ValueError, match="pages"):
+        submit(e, [1] * 10, max_tokens=30)          # 40 tokens = 10 pages, the pool has 4
+    with pytest.raises(ValueError):
+        Request([], SamplingParams())
+
+
+def test_max_model_len_ends_a_request():
+    e = FakeEngine(num_pages=64, page_size=4, max_model_len=12)
+    r = submit(e, [1, 2, 3, 4, 5], max_tokens=100, ignore_eos=True)
+    e.run_all()
+    assert len(r.tokens) == 12 and r.finish_reason == "length"
