@@ -319,7 +319,8 @@ class Executor:
             decode_only=all(q == 1 for q in facts["q_lens"]),
             max_q_len=max(facts["q_lens"]) if facts["q_lens"] else 0,
             max_context_len=max((s.start + len(s.tokens) for s in seqs), default=0),
-            n_seqs=facts["Sp"])
+            n_seqs=facts["Sp"], q_lens=list(facts["q_lens"]) + [0] * (facts["Sp"] - facts["S"]),
+            cu_seqlens=ctx.cu_seqlens, workspace=self.rt.workspace)
         for call in range(len(self.plan.calls)):
             g = self.group_of_call.get(call)
             if g is not None:
@@ -378,7 +379,6 @@ class Executor:
         if entry is None:
             entry = self._capture(bucket, arr, off, facts, seqs)
         graph, ctx, meta, logits = entry
-        ctx.attention_plan.max_context_len = max(s.start + 1 for s in seqs)
         self._upload(arr, dst=meta)
         graph.replay()
         return logits[:S]

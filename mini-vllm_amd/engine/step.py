@@ -48,9 +48,11 @@ class AttentionPlan:
     """Host-side facts about the step that let the attention pick a kernel."""
     decode_only: bool              # every sequence brings exactly one token
     max_q_len: int
-    max_context_len: int
-    n_seqs: int
-    scratch: Optional[torch.Tensor] = None     # float32 work area for split-key partial results
+    max_context_len: int           # longest context the step (or the graph it is captured in) must serve
+    n_seqs: int                    # rows of cu_seqlens - 1, padding sequences included
+    q_lens: Sequence[int] = ()     # tokens per sequence, on the host
+    cu_seqlens: Optional[torch.Tensor] = None   # int32 [n_seqs + 1] on the device
+    workspace: Optional[object] = None          # where kernels take scratch memory from
 
 
 class StepContext:

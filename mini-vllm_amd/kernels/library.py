@@ -48,12 +48,14 @@ _SIGNATURES = {
 _OPTIONAL_SIGNATURES = {
     "mv_gemm_skinny": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int,
                                c_int, c_int, c_int, c_void_p]),
+    "mv_gemm_skinny_swiglu": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),
     "mv_attention_decode": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
-                                    c_void_p, c_int, c_int, c_void_p]),
+                                    c_void_p, c_int, c_void_p, c_void_p]),
     "mv_attention_prefill": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                      c_void_p]),
+    "mv_attention_prefill_unit_tokens": (c_int, [c_int]),
 }
 
 

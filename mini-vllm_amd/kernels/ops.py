@@ -241,6 +241,25 @@ class Ops:
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
 
+    def gemm_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> bool:
+        """out[M, I] = silu(a Wg^T) * (a Wu^T) for the packed weight [2I, K] in one pass over the
+        weight, when the weight-streaming kernel takes the shape. Returns False (and does nothing)
+        otherwise; the caller then runs the product and the activation separately."""
+        if not (self.use_fast_kernels and self.lib.has("mv_gemm_skinny_swiglu")):
+            return False
+        M, K = a.shape
+        two_i = w_gate_up.shape[0]
+        if (M > SKINNY_MAX_M or M == 0 or w_gate_up.dtype != torch.bfloat16 or K % 32 or two_i % 2
+                or a.stride(1) != 1 or (M > 1 and a.stride(0) % 8) or a.data_ptr() % 16
+                or not w_gate_up.is_contiguous() or w_gate_up.shape[1] != K):
+            return False
+        self._act(a, "gemm input"); self._act(out, "swiglu output"); _dev(w_gate_up, "gate_up weight")
+        if out.shape != (M, two_i // 2) or out.stride(1) != 1:
+            raise KernelLibraryError(f"gemm_swiglu: output {tuple(out.shape)} is not [{M}, {two_i // 2}]")
+        self.lib.call("mv_gemm_skinny_swiglu", a.data_ptr(), a.stride(0) if M > 1 else K, w_gate_up.data_ptr(),
+                      out.data_ptr(), out.stride(0) if M > 1 else two_i // 2, M, two_i // 2, K, self._stream())
+        return True
+
     # ------------------------------------------------------------------------------------
     def attention(self, q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                   block_table: torch.Tensor, page_size: int, positions: torch.Tensor, token_seq: torch.Tensor,
@@ -278,10 +297,47 @@ class Ops:
         w = -1 if window is None else int(window)
         qs = q.stride(0) if n > 1 else q.shape[1]
         os_ = out.stride(0) if n > 1 else hd
+        if self._attention_fast(q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
+                                num_heads, num_kv_heads, head_dim, scale, w, plan):
+            return
         self.lib.call("mv_attention_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim,
                       float(scale), w, self.code, self._stream())
+
+    def _attention_fast(self, q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
+                        H, Hkv, D, scale, window, plan) -> bool:
+        """The MFMA kernels, when the step and the sizes allow them."""
+        if not self.use_fast_kernels or plan is None or not self.lib.has("mv_attention_decode"):
+            return False
+        if D not in (64, 128) or page_size % 16 or qs % 8 or os_ % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
+            return False
+        group = H // Hkv
+        n_seqs = plan.n_seqs
+        if plan.decode_only and group <= 16:
+            # split the keys over workgroups until the chip is filled; the count is a property of
+            # the plan (a captured graph keeps it), each split takes its share of the actual keys
+            blocks = max(1, -(-plan.max_context_len // 32))
+            nsplit = max(1, min(1024 // max(1, n_seqs * Hkv), blocks // 4, 64))
+            partials = None
+            if nsplit > 1:
+                # n_seqs * nsplit never exceeds 1024 / Hkv: one size serves every batch
+                rows = max(n_seqs * nsplit, 1024 // Hkv)
+                partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
+            self.lib.call("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
+                          v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+                          positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
+                          _ptr(partials), nsplit, token_seq.data_ptr(), self._stream())
+            return True
+        unit = self.lib.dll.mv_attention_prefill_unit_tokens(group)
+        if unit <= 0:
+            return False
+        n_units = sum(-(-ql // unit) for ql in plan.q_lens)
+        self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
+                      v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, H, Hkv, D, float(scale),
+                      window, self._stream())
+        return True
 
     # ------------------------------------------------------------------------------------
     def sample(self, logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,

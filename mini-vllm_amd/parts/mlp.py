@@ -42,10 +42,11 @@ class SwiGLU(FeedForward):
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         spec, rt, ops = self.spec, self.rt, self.rt.ops
         n = x.shape[0]
-        gu = rt.workspace.get("ffn.gate_up", (n, 2 * spec.intermediate_size), rt.dtype)
-        ops.gemm(x, self.w_gate_up, gu)
         act = rt.workspace.get("ffn.act", (n, spec.intermediate_size), rt.dtype)
-        ops.swiglu(gu, act)
+        if not ops.gemm_swiglu(x, self.w_gate_up, act):      # one pass over the weight for few rows
+            gu = rt.workspace.get("ffn.gate_up", (n, 2 * spec.intermediate_size), rt.dtype)
+            ops.gemm(x, self.w_gate_up, gu)
+            ops.swiglu(gu, act)
         y = rt.workspace.get("ffn.out", (n, spec.hidden_size), rt.dtype)
         ops.gemm(act, self.w_down, y)
         return y

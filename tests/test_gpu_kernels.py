@@ -233,12 +233,24 @@ def fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype):
     return kp, vp
 
 
+def make_plan(q_lens, ctx_lens, max_context_len=None):
+    from minivllm_amd.engine.step import AttentionPlan
+    from minivllm_amd.parts import Workspace
+    cu = torch.tensor([0] + list(np.cumsum(q_lens)), dtype=torch.int32, device="cuda")
+    return AttentionPlan(decode_only=all(q == 1 for q in q_lens), max_q_len=max(q_lens),
+                         max_context_len=max_context_len or max(ctx_lens), n_seqs=len(q_lens), q_lens=list(q_lens),
+                         cu_seqlens=cu, workspace=Workspace(torch.device("cuda:0")))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("with_plan", [False, True])
 @pytest.mark.parametrize("H,Hkv,D,ps,window", [(6, 3, 48, 4, None), (4, 1, 16, 8, 9), (8, 2, 128, 16, None),
-                                                (5, 5, 80, 3, 130), (16, 8, 128, 16, 40)])
-def test_attention_general(dtype, H, Hkv, D, ps, window):
+                                                (5, 5, 80, 3, 130), (16, 8, 128, 16, 40), (4, 4, 64, 32, None),
+                                                (14, 2, 64, 16, 25), (32, 1, 128, 16, None)])
+def test_attention_general(dtype, with_plan, H, Hkv, D, ps, window):
     """Mixed step: a long portion, a short one and single decoded tokens, over pages in
-    scrambled order; unused pages hold NaN."""
+    scrambled order; unused pages hold NaN. With a plan the bfloat16 path takes the MFMA kernel
+    where the sizes allow it."""
     ops = ops_for(dtype)
     g = torch.Generator().manual_seed(6)
     ctx_lens = [150, 37, 1, 290]            # context after the step
@@ -277,9 +289,97 @@ def test_attention_general(dtype, H, Hkv, D, ps, window):
     qrow[:, :H * D] = q.view(n, H * D)
     qd = dev(qrow)
     out = torch.empty(n, H * D, dtype=dtype, device="cuda")
-    ops.attention(qd[:, :H * D], out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale, window)
+    plan = make_plan(q_lens, ctx_lens) if with_plan else None
+    ops.attention(qd[:, :H * D], out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale, window,
+                  plan=plan)
     want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
-    assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= max(OP_TOL[dtype], 5e-6)
+    # the MFMA kernel rounds the probabilities to bfloat16 before the second product
+    tol = max(OP_TOL[dtype], 5e-6) * (2 if with_plan else 1)
+    assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= tol
+
+
+@pytest.mark.parametrize("H,Hkv,D,ps,window", [(16, 8, 128, 16, None), (8, 1, 128, 32, None), (6, 2, 64, 16, 50),
+                                                (16, 1, 64, 16, None)])
+@pytest.mark.parametrize("max_context", [None, 4096, 40000])
+def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
+    """Decode steps on the MFMA kernel: one token per sequence at very different context
+    lengths, a padding sequence in the middle, keys split over 1, a few and many workgroups."""
+    ops = ops_for(torch.bfloat16)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(16)
+    ctx_lens = [1, 17, 300, 1200, 33, 64]
+    q_lens = [1, 1, 1, 0, 1, 1]                     # sequence 3 is padding: no token
+    live = [s for s, ql in enumerate(q_lens) if ql]
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    pages_per = [-(-c // ps) for c in ctx_lens]
+    num_pages = sum(pages_per) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, cur = [], 0
+    for n_p in pages_per:
+        tables.append(perm[cur:cur + n_p]); cur += n_p
+    if window is not None:
+        for s, c in enumerate(ctx_lens):
+            for i in range(max(0, (c - 1) - window) // ps):
+                tables[s][i] = -1
+    kp, vp = fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype)
+    bt = torch.full((len(tables), max(pages_per)), -1, dtype=torch.int32)
+    for s, t in enumerate(tables):
+        bt[s, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    positions = torch.tensor([ctx_lens[s] - 1 for s in live], dtype=torch.int32)
+    token_seq = torch.tensor(live, dtype=torch.int32)
+    n = len(live)
+    q = torch.randn(n, H, D, generator=g)
+    far = 5 if window is None else 300 - 1 - window         # a far key, or the one at the window's edge
+    q[2] = 6.0 * k_all[2][far].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
+    q = q.to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.empty(n, H * D, dtype=dtype, device="cuda")
+    plan = make_plan(q_lens, ctx_lens, max_context_len=max_context)
+    ops.attention(dev(q.view(n, H * D)), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale,
+                  window, plan=plan)
+    want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
+    assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 70, 96), (8, 1024, 1024), (17, 4100, 64), (64, 333, 3072), (33, 2048, 512),
+                                    (5, 151936 // 8, 1024)])
+def test_gemm_weight_streaming(out_dtype, M, N, K):
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(17)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    want = a.double() @ w.double().T
+    out = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+    ops.gemm(dev(a), dev(w), out)
+    tol = 3e-6 if out_dtype == torch.float32 else OP_TOL[torch.bfloat16]
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= tol
+    ops.gemm(dev(a), dev(w), out, dev(b))
+    assert rel_err(out.float().cpu().numpy(), (want + b.double()).numpy()) <= tol
+    # rows in a wider buffer, and a row's result does not depend on the rows around it
+    wide = torch.zeros(M, K + 40, dtype=torch.bfloat16)
+    wide[:, :K] = a
+    out_w = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    ops.gemm(dev(wide)[:, :K], dev(w), out_w)
+    out_one = torch.empty(1, N, dtype=torch.float32, device="cuda")
+    ops.gemm(dev(a[M - 1:M]), dev(w), out_one)
+    assert torch.equal(out_w[M - 1:M], out_one)
+    assert rel_err(out_w.cpu().numpy(), want.numpy()) <= 3e-6
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 3072, 1024), (40, 100, 96), (64, 560, 256)])
+def test_gemm_swiglu_fused(M, I, K):
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(18)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (2 * torch.randn(2 * I, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ops.gemm_swiglu(dev(a), dev(w), out)
+    gu = a.double() @ w.double().T
+    want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[torch.bfloat16]
 
 
 def test_attention_reduces_to_library_softmax():
