@@ -162,16 +162,60 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
     }
     const float sc_mul = scale * LOG2E;
 
-    for (int b = b_begin; b < b_end; b += b_step) {
-        const int base = 32 * b;
-        int page[2], slot0[2];
+    // Pages and operands of a block. K operands are fetched one block ahead and V operands
+    // before the scores are computed, so that their latency hides behind the MFMA work.
+    auto block_pages = [&](int b, int* page, int* slot0) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int key0 = base + 16 * t;
+            const int key0 = 32 * b + 16 * t;
             const int pidx = key0 / page_size;
-            page[t] = (key0 <= hi_w && pidx < bt_width) ? bt[pidx] : -1;
+            page[t] = (b < b_end && key0 <= hi_w && pidx < bt_width) ? bt[pidx] : -1;
             slot0[t] = key0 % page_size;
         }
+    };
+    auto load_k = [&](const int* page, const int* slot0, Frag (*kop)[DS]) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (page[t] >= 0) {
+                const bf16* kptr =
+                    k_pages + (((size_t)page[t] * Hkv + kvh) * page_size + slot0[t] + i) * D + 8 * g;
+#pragma unroll
+                for (int s = 0; s < DS; ++s) kop[t][s].u = *reinterpret_cast<const uint4*>(kptr + 32 * s);
+            } else {
+#pragma unroll
+                for (int s = 0; s < DS; ++s) kop[t][s].u = uint4{0u, 0u, 0u, 0u};
+            }
+        }
+    };
+
+    int page[2], slot0[2];
+    Frag kop[2][DS];
+    block_pages(b_begin, page, slot0);
+    load_k(page, slot0, kop);
+
+    for (int b = b_begin; b < b_end; b += b_step) {
+        const int base = 32 * b;
+        // V^T operands of this block
+        Frag vop[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (page[t] >= 0) {
+                    const bf16* vptr = v_pages + (((size_t)page[t] * Hkv + kvh) * D + 16 * dt + i) * page_size +
+                                       slot0[t] + 4 * g;
+                    vop[dt].h[t] = *reinterpret_cast<const uint2*>(vptr);
+                } else {
+                    vop[dt].h[t] = uint2{0u, 0u};
+                }
+            }
+        }
+        // K operands of the next block
+        int npage[2], nslot0[2];
+        Frag knext[2][DS];
+        block_pages(b + b_step, npage, nslot0);
+        load_k(npage, nslot0, knext);
+
         // scores^T for two tiles of 16 keys
         float p[NT][2][4];
 #pragma unroll
@@ -180,16 +224,11 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct) sacc[ct] = floatx4_t{0.f, 0.f, 0.f, 0.f};
             if (page[t] >= 0) {
-                const bf16* kptr =
-                    k_pages + (((size_t)page[t] * Hkv + kvh) * page_size + slot0[t] + i) * D + 8 * g;
-                Frag kop[DS];
-#pragma unroll
-                for (int s = 0; s < DS; ++s) kop[s].u = *reinterpret_cast<const uint4*>(kptr + 32 * s);
 #pragma unroll
                 for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
                     for (int s = 0; s < DS; ++s)
-                        sacc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[s].v, qop[ct][s].v, sacc[ct], 0, 0, 0);
+                        sacc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[t][s].v, qop[ct][s].v, sacc[ct], 0, 0, 0);
             }
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct)
@@ -228,30 +267,27 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
             for (int dt = 0; dt < DT; ++dt) acc_o[ct][dt] *= corr;
         }
         // out^T += V^T P^T
-        const bool tail = base + 31 > hi_w;
+        if (base + 31 > hi_w) {  // slots above the newest key were never written
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            Frag vop;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (page[t] >= 0) {
-                    const bf16* vptr = v_pages + (((size_t)page[t] * Hkv + kvh) * D + 16 * dt + i) * page_size +
-                                       slot0[t] + 4 * g;
-                    vop.h[t] = *reinterpret_cast<const uint2*>(vptr);
-                } else {
-                    vop.h[t] = uint2{0u, 0u};
-                }
-            }
-            if (tail) {  // slots above the newest key were never written
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (base + 16 * t + 4 * g + r > hi_w) vop.s[t * 4 + r] = 0;
-            }
+                        if (base + 16 * t + 4 * g + r > hi_w) vop[dt].s[t * 4 + r] = 0;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct)
-                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
+                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
+        // the prefetched block becomes the current one
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            page[t] = npage[t];
+            slot0[t] = nslot0[t];
+#pragma unroll
+            for (int s = 0; s < DS; ++s) kop[t][s] = knext[t][s];
         }
     }
 
@@ -342,8 +378,10 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
 }
 
 // Merges the partial results of the key splits: out[token][head] = sum_z o_z 2^(m_z - m) / l.
+#define AF_MAX_SPLITS 64
 __global__ void attention_merge_kernel(const float* __restrict__ partials, bf16* __restrict__ out, long out_stride,
                                        const int* __restrict__ token_seq, int H, int D, int nsplit) {
+    __shared__ float sh_m[AF_MAX_SPLITS], sh_w[AF_MAX_SPLITS];
     const int tok = blockIdx.x, head = blockIdx.y;
     bf16* orow = out + (size_t)tok * out_stride + (size_t)head * D;
     if (token_seq[tok] < 0) {
@@ -351,21 +389,25 @@ __global__ void attention_merge_kernel(const float* __restrict__ partials, bf16*
         return;
     }
     const float* base = partials + ((size_t)tok * H + head) * nsplit * (D + 2);
-    float m = -INFINITY;
-    for (int z = 0; z < nsplit; ++z) m = fmaxf(m, base[(size_t)z * (D + 2) + D]);
-    float l = 0.f;
-    for (int z = 0; z < nsplit; ++z) {
-        const float mz = base[(size_t)z * (D + 2) + D];
-        if (mz != -INFINITY) l += exp2f(mz - m) * base[(size_t)z * (D + 2) + D + 1];
+    if ((int)threadIdx.x < nsplit) {
+        sh_m[threadIdx.x] = base[(size_t)threadIdx.x * (D + 2) + D];
+        sh_w[threadIdx.x] = base[(size_t)threadIdx.x * (D + 2) + D + 1];
     }
-    const float inv = 1.f / l;
+    __syncthreads();
+    float m = -INFINITY;
+    for (int z = 0; z < nsplit; ++z) m = fmaxf(m, sh_m[z]);
+    float l = 0.f;
+    for (int z = 0; z < nsplit; ++z)
+        if (sh_m[z] != -INFINITY) l += exp2f(sh_m[z] - m) * sh_w[z];
+    __syncthreads();
+    if ((int)threadIdx.x < nsplit)
+        sh_w[threadIdx.x] = (sh_m[threadIdx.x] == -INFINITY) ? 0.f : exp2f(sh_m[threadIdx.x] - m) / l;
+    __syncthreads();
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float a = 0.f;
-        for (int z = 0; z < nsplit; ++z) {
-            const float mz = base[(size_t)z * (D + 2) + D];
-            if (mz != -INFINITY) a += exp2f(mz - m) * base[(size_t)z * (D + 2) + d];
-        }
-        orow[d] = from_f<bf16>(a * inv);
+#pragma unroll 8
+        for (int z = 0; z < nsplit; ++z) a += sh_w[z] * base[(size_t)z * (D + 2) + d];
+        orow[d] = from_f<bf16>(a);
     }
 }
 
@@ -410,7 +452,7 @@ extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long
                                    hipStream_t stream) {
     if (int rc = check_common("attention_decode", q_stride, out_stride, page_size, bt_width, H, Hkv, D)) return rc;
     MV_REQUIRE(H / Hkv <= 16, "attention_decode: %d query heads per kv head exceed 16", H / Hkv);
-    MV_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || partials != nullptr),
+    MV_REQUIRE(nsplit >= 1 && nsplit <= AF_MAX_SPLITS && (nsplit == 1 || partials != nullptr),
                "attention_decode: bad split count %d or missing work area", nsplit);
     if (n_seqs <= 0) return 0;
     dim3 grid(n_seqs, Hkv, nsplit);

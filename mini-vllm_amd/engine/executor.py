@@ -122,7 +122,7 @@ class Executor:
 
         self._staging = _Staging()
         self._meta_device: Optional[torch.Tensor] = None
-        self._graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, StepContext, torch.Tensor, torch.Tensor]] = {}
+        self._graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, StepContext, torch.Tensor, torch.Tensor]] = {}
         self._graph_pool = None
         self._graph_workspace: Optional[Workspace] = None
         self.kv_pages: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
@@ -370,14 +370,25 @@ class Executor:
         ctx = self._context(meta, off, facts, seqs)
         return self.model.forward(ctx)
 
+    def _context_cap(self, seqs: Sequence[SeqStep]) -> int:
+        """The context length a decode graph is planned for: the next power of two (at least
+        1024) above the longest context of the step. Kernels that split the keys choose their
+        split for this length, so short contexts do not pay for the longest one."""
+        longest = max(s.start + 1 for s in seqs)
+        cap = 1024
+        while cap < longest:
+            cap *= 2
+        return min(cap, max(self.config.max_model_len, 1))
+
     def _step_graph(self, seqs: Sequence[SeqStep]) -> torch.Tensor:
         S = len(seqs)
         bucket = next(b for b in GRAPH_BUCKETS if b >= S)
+        cap = self._context_cap(seqs)
         widths = [self.max_pages_per_seq] * len(self.groups)
         arr, off, facts = self._fill(seqs, pad_to=bucket, bt_widths=widths)
-        entry = self._graphs.get(bucket)
+        entry = self._graphs.get((bucket, cap))
         if entry is None:
-            entry = self._capture(bucket, arr, off, facts, seqs)
+            entry = self._capture(bucket, cap, arr, off, facts, seqs)
         graph, ctx, meta, logits = entry
         self._upload(arr, dst=meta)
         graph.replay()
@@ -396,8 +407,8 @@ class Executor:
         self._upload(arr, dst=meta)
         return self._context(meta, off, facts, dummy)
 
-    def _capture(self, bucket: int, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
-        logger.info("capturing the decode graph for %d sequences", bucket)
+    def _capture(self, bucket: int, cap: int, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
+        logger.info("capturing the decode graph for %d sequences, contexts up to %d", bucket, cap)
         library_gemm = self.ops.use_library_gemm
         eager_workspace = self.rt.workspace
         self.ops.use_library_gemm = False          # only the engine's own kernels inside a graph
@@ -418,8 +429,8 @@ class Executor:
             meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
             self._upload(arr, dst=meta)
             ctx = self._context(meta, off, facts, seqs)
-            # the graph must serve every later context length: plan for the longest
-            ctx.attention_plan.max_context_len = self.config.max_model_len
+            # the graph serves every context length up to its cap
+            ctx.attention_plan.max_context_len = cap
             self.model.forward(ctx)                # loads every kernel before the capture
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -431,5 +442,5 @@ class Executor:
             self.ops.use_library_gemm = library_gemm
         torch.cuda.synchronize()
         entry = (graph, ctx, meta, logits)
-        self._graphs[bucket] = entry
+        self._graphs[(bucket, cap)] = entry
         return entry
