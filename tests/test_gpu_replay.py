@@ -157,3 +157,33 @@ def test_trace_run_program(cases, tmp_path):
 
         got = trace_tools.collect(steps, read)
         case.check(got, dtype, "bin/trace_run mixed")
+
+
+def test_layer_sizes_of_the_0_6b_shape(tmp_path):
+    """The layer sizes of Qwen3-0.6B (hidden 1024, 16/8 heads of 128, intermediate 3072, vocabulary
+    151936, tied head, theta 1e6) with four layers: portions, decoded tokens and a second request
+    on recycled pages, in float32 and bfloat16, against the plain model. This is the shape the
+    MFMA kernels are tuned for (head size 128, K = 1024/2048/3072)."""
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 4, "hidden_size": 1024,
+           "num_attention_heads": 16, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 3072,
+           "vocab_size": 151936, "max_position_embeddings": 40960, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+           "tie_word_embeddings": True, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
+    weights = make_weights(cfg, seed=6, stored=torch.bfloat16, std=0.02, qk_gain=1.5)
+    path = write_model_dir(str(tmp_path / "shape06"), cfg, weights)
+    reqs = {"p": random_tokens(cfg, 83, seed=1), "q": random_tokens(cfg, 40, seed=2)}
+    w64 = {k: v.double() for k, v in weights.items()}            # converted once: the table is large
+    want = {r: plain_logits(cfg, w64, t) for r, t in reqs.items()}
+    emulated = {r: plain_logits_bf16(cfg, w64, t) for r, t in reqs.items()}
+    del w64
+    bf16_err = max(rel_err(emulated[r][p], want[r][p]) for r, t in reqs.items() for p in range(len(t)))
+    steps = trace_tools.mixed(reqs, {"p": 70, "q": 33}, max_live=2, seed=3, max_portion=40)
+    from minivllm_amd.engine.trace import TraceRunner
+    for dtype in ("float32", "bfloat16"):
+        runner = TraceRunner(path, dtype, trace_tools.max_live_tokens(steps), page_size=16)
+        got = trace_tools.collect(steps, runner.run_step)
+        worst = max(rel_err(row, want[rid][pos]) for (rid, pos), row in got.items())
+        tol = TOL_F32 if dtype == "float32" else bf16_tolerance(bf16_err)
+        print(f"0.6B layer sizes [{dtype}]: {len(got)} rows, worst relative error {worst:.3e} (allowed {tol:.3e})")
+        assert len(got) == 123 and worst <= tol
+        del runner
+        torch.cuda.empty_cache()
