@@ -422,15 +422,6 @@ static void launch_attention(dim3 grid, hipStream_t stream, const void* q, long 
                        window, partials, nsplit);
 }
 
-#define AF_PREFILL_NT 2
-
-// How many query tokens one workgroup of the prompt kernel serves, for `group` query heads per
-// key/value head; 0 if the kernel does not take this group size.
-extern "C" int mv_attention_prefill_unit_tokens(int group) {
-    const int cols = 16 * AF_WAVES * AF_PREFILL_NT;
-    return group > 0 && group <= cols ? cols / group : 0;
-}
-
 static int check_common(const char* what, long q_stride, long out_stride, int page_size, int bt_width, int H, int Hkv,
                         int D) {
     MV_REQUIRE(H > 0 && Hkv > 0 && H % Hkv == 0, "%s: %d heads are not a multiple of %d kv heads", what, H, Hkv);
@@ -473,23 +464,3 @@ extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long
     return 0;
 }
 
-// Prompt portions and mixed steps. n_units = sum over sequences of ceil(q_len / unit tokens).
-extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
-                                    const void* v_pages, const int* block_table, int bt_width, int page_size,
-                                    const int* positions, const int* cu_seqlens, int n_seqs, int n_units, int H,
-                                    int Hkv, int D, float scale, int window, hipStream_t stream) {
-    if (int rc = check_common("attention_prefill", q_stride, out_stride, page_size, bt_width, H, Hkv, D)) return rc;
-    MV_REQUIRE(mv_attention_prefill_unit_tokens(H / Hkv) > 0, "attention_prefill: %d query heads per kv head "
-               "exceed what a workgroup holds", H / Hkv);
-    if (n_seqs <= 0 || n_units <= 0) return 0;
-    dim3 grid(n_units, Hkv, 1);
-    if (D == 128)
-        launch_attention<128, AF_PREFILL_NT, false>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages,
-                                                    block_table, bt_width, page_size, positions, cu_seqlens, n_seqs,
-                                                    0, H, Hkv, scale, window, nullptr, 1);
-    else
-        launch_attention<64, AF_PREFILL_NT, false>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages,
-                                                   block_table, bt_width, page_size, positions, cu_seqlens, n_seqs, 0,
-                                                   H, Hkv, scale, window, nullptr, 1);
-    return mv_check_launch("attention_prefill");
-}

@@ -1,0 +1,422 @@
+// Paged causal attention for prompt portions and mixed steps on the MFMA units of gfx950,
+// bf16 in and out, float inside.
+//
+// A workgroup of four waves serves one key/value head of one unit: up to 64*NT columns, a column
+// being a (query token, query head of the group) pair of a run of consecutive tokens of one
+// sequence. Each wave owns 16*NT columns. The workgroup walks the keys the unit may see in blocks
+// of 32; every block's K tile [32 keys x D] and transposed V tile [D x 32 keys] are copied from
+// the cache pages into LDS once, in the order the MFMA operands are read (so the reads are
+// conflict-free 16-byte loads), double-buffered: the copy of block b+1 is in flight while block
+// b is computed, with one barrier per block.
+//
+//   scores^T = K Q^T     A operand: 16 keys x 32 d from LDS, B operand: the wave's queries (registers);
+//                        result: lane l holds column l%16, keys 4*(l/16)+0..3 of the 16-key tile.
+//   out^T    = V^T P^T   A operand: 16 d x 32 keys from LDS, B operand: the probabilities the lane
+//                        already holds: its eight k-slots are bound to keys {4g..4g+3} of the two
+//                        16-key tiles of the block (g = l/16), and V is stored in LDS for exactly
+//                        those keys, so nothing is shuffled between the two products.
+// Online softmax (base 2) per column. A wave skips blocks that lie outside the range of all its
+// columns. Value slots above the unit's newest key were never written and are copied as zero.
+//
+// Layouts: K[page][kv_head][slot][d], V[page][kv_head][d][slot]; page size a multiple of 16.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+union Frag {
+    uint4 u;
+    uint2 h[2];
+    uint16_t s[8];
+    bf16x8_t v;
+};
+
+#define AP_WAVES 4
+#define AP_THREADS (64 * AP_WAVES)
+#define LOG2E 1.4426950408889634f
+
+template <int D, int NT>
+__global__ void __launch_bounds__(AP_THREADS)
+attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
+                         const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+                         const int* __restrict__ block_table, int bt_width, int page_size, int page_shift,
+                         const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs, int H,
+                         int Hkv, float scale, int window) {
+    constexpr int DS = D / 32;                 // k-steps of the score product
+    constexpr int DT = D / 16;                 // d tiles of the output product
+    constexpr int COLS = 16 * AP_WAVES * NT;   // columns of a workgroup
+    constexpr int KCHUNKS = 2 * DS * 64;       // 16-byte chunks of a K tile
+    constexpr int VCHUNKS = DT * 64;           // 16-byte chunks of a V tile (two 8-byte halves each)
+    constexpr int KREP = KCHUNKS / AP_THREADS;
+    constexpr int VREP = 2 * VCHUNKS / AP_THREADS / 2;  // 16-byte global loads per thread
+    static_assert(KCHUNKS % AP_THREADS == 0 && (D * 2 * 2) % AP_THREADS == 0, "tile does not divide the workgroup");
+
+    __shared__ uint4 sK[2][KCHUNKS];
+    __shared__ uint2 sV[2][VCHUNKS * 2];
+    __shared__ int sh_unit[3];
+    __shared__ int sh_range[2][AP_WAVES];
+
+    const int G = H / Hkv;
+    // the key/value head is the fastest grid dimension: workgroups are dealt to the eight XCDs in
+    // turn, so all units of a head land on the same XCD and share its L2
+    const int kvh = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int wave = tid / MV_WAVE;
+    const int lane = tid % MV_WAVE;
+    const int i = lane % 16;
+    const int g = lane / 16;
+    const int tpu = COLS / G;  // tokens of a unit (the host made sure it is >= 1)
+
+    if (tid == 0) {
+        int seq = -1, t0 = 0, nt = 0;
+        int u = gridDim.y - 1 - blockIdx.y;  // units with the most keys start first
+        for (int s = 0; s < n_seqs; ++s) {
+            const int ql = cu_seqlens[s + 1] - cu_seqlens[s];
+            const int nu = (ql + tpu - 1) / tpu;
+            if (u < nu) {
+                seq = s;
+                t0 = cu_seqlens[s] + u * tpu;
+                nt = ql - u * tpu;
+                if (nt > tpu) nt = tpu;
+                break;
+            }
+            u -= nu;
+        }
+        sh_unit[0] = seq;
+        sh_unit[1] = t0;
+        sh_unit[2] = nt;
+    }
+    __syncthreads();
+    const int seq = sh_unit[0], t0 = sh_unit[1], nt = sh_unit[2];
+    if (seq < 0 || nt <= 0) return;
+    const int ncols = nt * G;
+    const int* bt = block_table + (size_t)seq * bt_width;
+
+    // ---- this lane's columns
+    int col_tok[NT], col_head[NT], col_pos[NT], col_lo[NT];
+    bool col_ok[NT];
+    Frag qop[NT][DS];
+    int hi_w = -1, lo_w = 0x7fffffff;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
+        const int col = (wave * NT + ct) * 16 + i;
+        col_ok[ct] = col < ncols;
+        col_tok[ct] = t0 + (col_ok[ct] ? col / G : 0);
+        col_head[ct] = kvh * G + (col_ok[ct] ? col % G : 0);
+        col_pos[ct] = col_ok[ct] ? positions[col_tok[ct]] : -1;
+        col_lo[ct] = (window >= 0 && col_pos[ct] - window > 0) ? col_pos[ct] - window : 0;
+        if (col_ok[ct]) {
+            hi_w = col_pos[ct] > hi_w ? col_pos[ct] : hi_w;
+            lo_w = col_lo[ct] < lo_w ? col_lo[ct] : lo_w;
+        }
+        const bf16* qrow = q + (size_t)col_tok[ct] * q_stride + (size_t)col_head[ct] * D + 8 * g;
+#pragma unroll
+        for (int s = 0; s < DS; ++s)
+            qop[ct][s].u = col_ok[ct] ? *reinterpret_cast<const uint4*>(qrow + 32 * s) : uint4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int o = MV_WAVE / 2; o > 0; o >>= 1) {
+        const int a = __shfl_xor(hi_w, o, MV_WAVE), b = __shfl_xor(lo_w, o, MV_WAVE);
+        hi_w = a > hi_w ? a : hi_w;
+        lo_w = b < lo_w ? b : lo_w;
+    }
+    if (lane == 0) {
+        sh_range[0][wave] = hi_w;
+        sh_range[1][wave] = lo_w;
+    }
+    __syncthreads();
+    int hi_g = -1, lo_g = 0x7fffffff;
+#pragma unroll
+    for (int w = 0; w < AP_WAVES; ++w) {
+        hi_g = sh_range[0][w] > hi_g ? sh_range[0][w] : hi_g;
+        lo_g = sh_range[1][w] < lo_g ? sh_range[1][w] : lo_g;
+    }
+    if (hi_g < 0) return;
+    const int b0 = lo_g / 32, b1 = hi_g / 32;
+
+    float m_run[NT], l_run[NT];
+    floatx4_t acc_o[NT][DT];
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
+        m_run[ct] = -INFINITY;
+        l_run[ct] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc_o[ct][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    const float sc_mul = scale * LOG2E;
+
+    // ---- copy of a block from the pages: global -> registers -> LDS.
+    // Two blocks are in flight: while block b is computed, block b+1 waits in one register set
+    // and block b+2 is being loaded into the other. Everything that does not depend on the block
+    // (which chunk of the tile a thread copies, where it goes in LDS) is worked out once.
+    struct Staged {
+        uint4 k[KREP];
+        uint4 v[VREP];
+    };
+    int k_tile[KREP], k_off[KREP], k_lds[KREP];
+#pragma unroll
+    for (int rep = 0; rep < KREP; ++rep) {
+        const int r = tid + AP_THREADS * rep;
+        const int key = r / (D / 8);  // 0..31
+        const int dchunk = r % (D / 8);
+        k_tile[rep] = key / 16;
+        k_off[rep] = (key % 16) * D + 8 * dchunk;
+        k_lds[rep] = (k_tile[rep] * DS + dchunk / 4) * 64 + key % 16 + 16 * (dchunk % 4);
+    }
+    int v_tile[VREP], v_off[VREP], v_lds[VREP], v_key[VREP];
+#pragma unroll
+    for (int rep = 0; rep < VREP; ++rep) {
+        const int r = tid + AP_THREADS * rep;
+        const int d = (r % (D * 2)) / 2;  // D * 2 sixteen-byte chunks per 16-key tile
+        const int hq = r % 2;
+        v_tile[rep] = r / (D * 2);
+        v_off[rep] = d * page_size + 8 * hq;
+        v_key[rep] = 16 * v_tile[rep] + 8 * hq;
+        // keys 8hq .. 8hq+3 go to lane group 2hq, keys 8hq+4 .. 8hq+7 to lane group 2hq+1 (32 further)
+        v_lds[rep] = ((d / 16) * 64 + d % 16 + 16 * (2 * hq)) * 2 + v_tile[rep];
+    }
+    const int page_mask = page_size - 1;
+    auto fetch = [&](int b, Staged& st) {
+        if (b > b1) return;
+        const bf16* kbase[2];
+        const bf16* vbase[2];
+        bool gone[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int key0 = 32 * b + 16 * t;
+            int pidx = key0 >> page_shift;
+            pidx = pidx < bt_width ? pidx : bt_width - 1;
+            int pg = bt[pidx];
+            gone[t] = pg < 0;      // a page that was given back (it lies below every column's range):
+            pg = gone[t] ? 0 : pg; // read some page, then put zeros in its place
+            const int slot0 = key0 & page_mask;
+            const size_t head = (size_t)pg * Hkv + kvh;
+            kbase[t] = k_pages + (head * page_size + slot0) * D;
+            vbase[t] = v_pages + head * D * page_size + slot0;
+        }
+#pragma unroll
+        for (int rep = 0; rep < KREP; ++rep)
+            st.k[rep] = *reinterpret_cast<const uint4*>((k_tile[rep] ? kbase[1] : kbase[0]) + k_off[rep]);
+#pragma unroll
+        for (int rep = 0; rep < VREP; ++rep)
+            st.v[rep] = *reinterpret_cast<const uint4*>((v_tile[rep] ? vbase[1] : vbase[0]) + v_off[rep]);
+        if (gone[0] || gone[1]) {
+#pragma unroll
+            for (int rep = 0; rep < KREP; ++rep)
+                if (gone[k_tile[rep]]) st.k[rep] = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int rep = 0; rep < VREP; ++rep)
+                if (gone[v_tile[rep]]) st.v[rep] = uint4{0u, 0u, 0u, 0u};
+        }
+    };
+    auto stash = [&](int b, const Staged& st) {
+        const int buf = (b - b0) & 1;
+#pragma unroll
+        for (int rep = 0; rep < KREP; ++rep) sK[buf][k_lds[rep]] = st.k[rep];
+        const bool tail = 32 * b + 31 > hi_g;  // slots above the newest key were never written
+#pragma unroll
+        for (int rep = 0; rep < VREP; ++rep) {
+            Frag f;
+            f.u = st.v[rep];
+            if (tail) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f.s[e] = (32 * b + v_key[rep] + e > hi_g) ? (uint16_t)0 : f.s[e];
+            }
+            sV[buf][v_lds[rep]] = f.h[0];
+            sV[buf][v_lds[rep] + 32] = f.h[1];
+        }
+    };
+
+    // keys at or below `full_hi` and at or above `full_lo` are visible to every column of the wave:
+    // blocks inside need no mask
+    int full_hi = 0x7fffffff, full_lo = 0;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
+        const int ph = col_ok[ct] ? col_pos[ct] : 0x7fffffff;
+        const int pl = col_ok[ct] ? col_lo[ct] : 0;
+        full_hi = ph < full_hi ? ph : full_hi;
+        full_lo = pl > full_lo ? pl : full_lo;
+    }
+#pragma unroll
+    for (int o = MV_WAVE / 2; o > 0; o >>= 1) {
+        const int a = __shfl_xor(full_hi, o, MV_WAVE), c = __shfl_xor(full_lo, o, MV_WAVE);
+        full_hi = a < full_hi ? a : full_hi;
+        full_lo = c > full_lo ? c : full_lo;
+    }
+    bool all_cols = true;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) all_cols = all_cols && col_ok[ct];
+    const bool wave_full = __all(all_cols);
+
+    auto compute = [&](int b) {
+        const int cur = (b - b0) & 1;
+        const int base = 32 * b;
+        if (!(base <= hi_w && base + 31 >= lo_w)) return;
+        const bool masked = !(wave_full && base + 31 <= full_hi && base >= full_lo);
+        // scores^T for the two 16-key tiles
+        float p[NT][2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            Frag kop[DS];
+#pragma unroll
+            for (int s = 0; s < DS; ++s) kop[s].u = sK[cur][(t * DS + s) * 64 + lane];
+#pragma unroll
+            for (int ct = 0; ct < NT; ++ct) {
+                floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < DS; ++s)
+                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[s].v, qop[ct][s].v, sacc, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) p[ct][t][r] = sacc[r];
+            }
+        }
+        if (masked) {
+#pragma unroll
+            for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = base + 16 * t + 4 * g + r;
+                        const bool ok = col_ok[ct] && key <= col_pos[ct] && key >= col_lo[ct];
+                        p[ct][t][r] = ok ? p[ct][t][r] : -INFINITY;
+                    }
+        }
+        // online softmax per column
+        Frag pop[NT];
+#pragma unroll
+        for (int ct = 0; ct < NT; ++ct) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, p[ct][t][r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
+            // The reference point of the exponentials (kept in the scaled, base-2 domain; the scale
+            // is positive) only follows the maximum when it has been overtaken by more than 2^8:
+            // until then the terms stay below 2^8, and the accumulators need no rescaling, which
+            // would move them between the accumulation and the vector registers.
+            const float mx_s = mx * sc_mul;
+            const bool stale = mx_s > m_run[ct] + 8.f;
+            if (__any(stale)) {
+                const float m_new = fmaxf(m_run[ct], mx_s);
+                const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;
+                const float corr = __builtin_amdgcn_exp2f(m_run[ct] - m_ref);   // exp2(-inf) = 0
+                l_run[ct] *= corr;
+                m_run[ct] = m_new;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) acc_o[ct][dt] *= corr;
+            }
+            const float m_safe = (m_run[ct] == -INFINITY) ? 0.f : m_run[ct];
+            float psum = 0.f;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float e = __builtin_amdgcn_exp2f(fmaf(p[ct][t][r], sc_mul, -m_safe));
+                    psum += e;
+                    pop[ct].v[t * 4 + r] = (__bf16)e;
+                }
+            l_run[ct] += psum;
+        }
+        // out^T += V^T P^T
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            Frag vop;
+            vop.h[0] = sV[cur][(dt * 64 + lane) * 2];
+            vop.h[1] = sV[cur][(dt * 64 + lane) * 2 + 1];
+#pragma unroll
+            for (int ct = 0; ct < NT; ++ct)
+                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
+        }
+    };
+
+    Staged sa, sb;
+    fetch(b0, sa);
+    fetch(b0 + 1, sb);
+    stash(b0, sa);
+    __syncthreads();
+    // invariant at the top: LDS holds block b, `sb` holds block b+1 (or zeros past the end)
+    for (int b = b0; b <= b1; b += 2) {
+        fetch(b + 2, sa);
+        compute(b);
+        if (b + 1 <= b1) stash(b + 1, sb);
+        __syncthreads();
+        if (b + 1 > b1) break;
+        fetch(b + 3, sb);
+        compute(b + 1);
+        if (b + 2 <= b1) stash(b + 2, sa);
+        __syncthreads();
+    }
+
+    // the sum of a column is spread over the four lane groups
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
+        l_run[ct] += __shfl_xor(l_run[ct], 16, MV_WAVE);
+        l_run[ct] += __shfl_xor(l_run[ct], 32, MV_WAVE);
+        if (!col_ok[ct]) continue;
+        const float inv = 1.f / l_run[ct];
+        bf16* orow = out + (size_t)col_tok[ct] * out_stride + (size_t)col_head[ct] * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            uint2 packed;
+            packed.x = (uint32_t)f32_to_bf16_bits(acc_o[ct][dt][0] * inv) |
+                       ((uint32_t)f32_to_bf16_bits(acc_o[ct][dt][1] * inv) << 16);
+            packed.y = (uint32_t)f32_to_bf16_bits(acc_o[ct][dt][2] * inv) |
+                       ((uint32_t)f32_to_bf16_bits(acc_o[ct][dt][3] * inv) << 16);
+            *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = packed;
+        }
+    }
+}
+
+// How many query tokens one workgroup serves with `nt` (1 or 2) column tiles per wave, for `group`
+// query heads per key/value head; 0 if the kernel does not take this combination.
+extern "C" int mv_attention_prefill_unit_tokens(int group, int nt) {
+    if (nt != 1 && nt != 2) return 0;
+    const int cols = 16 * AP_WAVES * nt;
+    return group > 0 && group <= cols ? cols / group : 0;
+}
+
+template <int D, int NT>
+static void launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
+                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
+                           int page_size, int page_shift, const int* positions, const int* cu_seqlens, int n_seqs,
+                           int H, int Hkv, float scale, int window) {
+    hipLaunchKernelGGL((attention_prefill_kernel<D, NT>), grid, dim3(AP_THREADS), 0, stream, (const bf16*)q, q_stride,
+                       (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,
+                       page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window);
+}
+
+// nt: column tiles per wave (2 = 128 columns per workgroup, for long prompts; 1 = 64 columns, twice
+// the workgroups, for steps too small to fill the chip otherwise).
+// n_units = sum over sequences of ceil(q_len / unit tokens(group, nt)). grid = (kv heads, units).
+extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
+                                    const void* v_pages, const int* block_table, int bt_width, int page_size,
+                                    const int* positions, const int* cu_seqlens, int n_seqs, int n_units, int nt,
+                                    int H, int Hkv, int D, float scale, int window, hipStream_t stream) {
+    MV_REQUIRE(H > 0 && Hkv > 0 && H % Hkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", H,
+               Hkv);
+    MV_REQUIRE(D == 64 || D == 128, "attention_prefill: head_dim %d is not served by the MFMA kernel (64 or 128)", D);
+    MV_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
+               "attention_prefill: page size %d must be a power of two, at least 16", page_size);
+    MV_REQUIRE(bt_width > 0, "attention_prefill: empty block table");
+    MV_REQUIRE(q_stride >= (long)H * D && q_stride % 8 == 0 && out_stride >= (long)H * D && out_stride % 4 == 0,
+               "attention_prefill: row strides %ld / %ld do not fit %d heads of %d", q_stride, out_stride, H, D);
+    MV_REQUIRE(n_units <= 65535, "attention_prefill: %d units exceed one launch", n_units);
+    MV_REQUIRE(mv_attention_prefill_unit_tokens(H / Hkv, nt) > 0, "attention_prefill: %d query heads per kv head "
+               "with %d column tiles per wave are not served", H / Hkv, nt);
+    if (n_seqs <= 0 || n_units <= 0) return 0;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    dim3 grid(Hkv, n_units, 1);
+#define AP_LAUNCH(DD, NN)                                                                                          \
+    launch_prefill<DD, NN>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,      \
+                           page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window)
+    if (D == 128 && nt == 2) AP_LAUNCH(128, 2);
+    else if (D == 128) AP_LAUNCH(128, 1);
+    else if (nt == 2) AP_LAUNCH(64, 2);
+    else AP_LAUNCH(64, 1);
+#undef AP_LAUNCH
+    return mv_check_launch("attention_prefill");
+}

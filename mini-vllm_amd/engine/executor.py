@@ -414,9 +414,9 @@ class Executor:
         self.ops.use_library_gemm = False          # only the engine's own kernels inside a graph
         try:
             if self._graph_workspace is None:
-                # one scratch area for all graphs, sized once for the largest bucket and then
-                # never reallocated: captured graphs keep its addresses
-                self._graph_workspace = Workspace(self.device)
+                # one scratch area for all graphs, sized for the largest bucket; should a later
+                # graph need a larger buffer, the old one stays alive for the graphs that hold it
+                self._graph_workspace = Workspace(self.device, retain=True)
                 self.rt.workspace = self._graph_workspace
                 largest = next(b for b in GRAPH_BUCKETS
                                if b >= min(self.config.max_num_batched_seqs, GRAPH_BUCKETS[-1]))
@@ -424,7 +424,6 @@ class Executor:
                 pad_ctx.attention_plan.max_context_len = self.config.max_model_len
                 self.model.forward(pad_ctx)
                 torch.cuda.synchronize()
-                self._graph_workspace.frozen = True
             self.rt.workspace = self._graph_workspace
             meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
             self._upload(arr, dst=meta)
@@ -433,11 +432,13 @@ class Executor:
             ctx.attention_plan.max_context_len = cap
             self.model.forward(ctx)                # loads every kernel before the capture
             torch.cuda.synchronize()
+            self._graph_workspace.frozen = True    # the eager run above sized everything: nothing is allocated now
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):
                 logits = self.model.forward(ctx)
             self._graph_pool = graph.pool()
         finally:
+            self._graph_workspace.frozen = False
             self.rt.workspace = eager_workspace
             self.ops.use_library_gemm = library_gemm
         torch.cuda.synchronize()

@@ -331,13 +331,21 @@ class Ops:
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
                           _ptr(partials), nsplit, token_seq.data_ptr(), self._stream())
             return True
-        unit = self.lib.dll.mv_attention_prefill_unit_tokens(group)
-        if unit <= 0:
+        if page_size & (page_size - 1):
             return False
-        n_units = sum(-(-ql // unit) for ql in plan.q_lens)
+        # 64 columns per workgroup (two workgroups fit a CU and hide each other's waits; measured
+        # faster than 128 columns at every prompt length); 128 only for groups of more than 64 heads
+        nt, n_units = 0, 0
+        for cand in (1, 2):
+            u = self.lib.dll.mv_attention_prefill_unit_tokens(group, cand)
+            if u > 0:
+                nt, n_units = cand, sum(-(-ql // u) for ql in plan.q_lens)
+                break
+        if nt == 0:
+            return False
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
-                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, H, Hkv, D, float(scale),
+                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, nt, H, Hkv, D, float(scale),
                       window, self._stream())
         return True
 

@@ -118,9 +118,13 @@ class Workspace:
     more. While a graph is being captured nothing may be allocated, so the buffers have to be
     grown (``reserve``) before."""
 
-    def __init__(self, device: torch.device):
+    def __init__(self, device: torch.device, retain: bool = False):
+        """``retain`` keeps a buffer alive after a larger one has replaced it: captured graphs that
+        hold its address go on working."""
         self.device = device
         self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self._retired: List[torch.Tensor] = []
+        self.retain = retain
         self.frozen = False
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
@@ -132,12 +136,14 @@ class Workspace:
         if buf is None or buf.numel() < n:
             if self.frozen:
                 raise RuntimeError(f"workspace buffer {name!r} would have to grow to {n} elements while frozen")
+            if buf is not None and self.retain:
+                self._retired.append(buf)
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
         return buf[:n].view(*shape)
 
     def bytes(self) -> int:
-        return sum(b.numel() * b.element_size() for b in self._buffers.values())
+        return sum(b.numel() * b.element_size() for b in list(self._buffers.values()) + self._retired)
 
 
 @dataclass
