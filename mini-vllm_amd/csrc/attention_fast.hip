@@ -1,8 +1,8 @@
-// Paged causal attention on the MFMA units of gfx950, bf16 in and out, float inside.
+// Paged attention for decode steps (one query token per sequence) on the MFMA units of gfx950,
+// bf16 in and out, float inside.
 //
-// A workgroup serves one key/value head of one "unit": a run of consecutive query tokens of one
-// sequence. The unit's (token, query head of the group) pairs are the columns of the problem;
-// with grouped heads the keys and values are read once for the whole group.
+// A workgroup serves one key/value head of one sequence; the query heads of the group are the
+// columns of the problem (at most 16), so the keys and values are read once for the whole group.
 //
 //   scores^T = K Q^T     A operand: 16 keys x 32 d of the key page (one 16-byte load per lane),
 //                        B operand: 32 d x 16 columns of the queries (kept in registers);
@@ -14,14 +14,13 @@
 // tiles (g = l/16), and the value operand is loaded for the same keys, so nothing is shuffled.
 // Each column keeps its own running maximum and sum (online softmax, base 2).
 //
-// Two ways to share the work inside a workgroup of four waves:
-//   SPLIT_KEYS   (decode: at most 16*NT columns) the waves take the 32-key blocks in turn and
-//                their partial results are merged through LDS; with nsplit > 1 several
-//                workgroups split the keys further and a second kernel merges their partials.
-//   otherwise    (prompt portions) each wave owns 16*NT columns and walks all their keys.
+// The W waves of a workgroup (4 or 8) take the 32-key blocks in turn, each with the K operands
+// of its next block already in flight, and their partial results are merged through LDS. With
+// nsplit > 1 several workgroups split a sequence's keys further and a second kernel merges
+// their partial results.
 //
 // Layouts: K[page][kv_head][slot][d], V[page][kv_head][d][slot]; the page size is a multiple of
-// 16. Keys outside a column's range (above its position, or more than `window` below it) get
+// 16. Keys outside the range (above the query's position, or more than `window` below it) get
 // probability zero; value slots that were never written are read as zero.
 #include "common.h"
 
@@ -35,8 +34,8 @@ union Frag {
     bf16x8_t v;
 };
 
-#define AF_WAVES 4
 #define LOG2E 1.4426950408889634f
+#define AF_MAX_CACHED_PAGES 1024
 
 __device__ __forceinline__ int wave_max_i(int v) {
 #pragma unroll
@@ -56,17 +55,18 @@ __device__ __forceinline__ int wave_min_i(int v) {
     return v;
 }
 
-template <int D, int NT, bool SPLIT_KEYS>
-__global__ void __launch_bounds__(64 * AF_WAVES)
-attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
+template <int D, int W>
+__global__ void __launch_bounds__(64 * W)
+attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                       const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                       const int* __restrict__ block_table, int bt_width, int page_size,
                       const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
-                      int decode_only, int H, int Hkv, float scale, int window, float* __restrict__ partials,
+                      int H, int Hkv, float scale, int window, float* __restrict__ partials,
                       int nsplit) {
     constexpr int DS = D / 32;
     constexpr int DT = D / 16;
-    constexpr int COLS = (SPLIT_KEYS ? 16 : 16 * AF_WAVES) * NT;  // columns of a workgroup
+    constexpr int NT = 1;      // column tiles of a wave (the group's heads fit one tile)
+    constexpr int COLS = 16;   // columns of a workgroup
     const int G = H / Hkv;
     const int kvh = blockIdx.y;
     const int split = blockIdx.z;
@@ -79,26 +79,10 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
     __shared__ int sh_unit[3];
     if (threadIdx.x == 0) {
         int seq = -1, t0 = 0, nt = 0;
-        if (decode_only) {
-            seq = blockIdx.x;
-            t0 = cu_seqlens[seq];
-            nt = cu_seqlens[seq + 1] - t0;
-            if (nt > tpu) nt = tpu;
-        } else {
-            int u = blockIdx.x;
-            for (int s = 0; s < n_seqs; ++s) {
-                const int ql = cu_seqlens[s + 1] - cu_seqlens[s];
-                const int nu = (ql + tpu - 1) / tpu;
-                if (u < nu) {
-                    seq = s;
-                    t0 = cu_seqlens[s] + u * tpu;
-                    nt = ql - u * tpu;
-                    if (nt > tpu) nt = tpu;
-                    break;
-                }
-                u -= nu;
-            }
-        }
+        seq = blockIdx.x;
+        t0 = cu_seqlens[seq];
+        nt = cu_seqlens[seq + 1] - t0;
+        if (nt > tpu) nt = tpu;
         sh_unit[0] = seq;
         sh_unit[1] = t0;
         sh_unit[2] = nt;
@@ -116,7 +100,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
     int hi_w = -1, lo_w = 0x7fffffff;
 #pragma unroll
     for (int ct = 0; ct < NT; ++ct) {
-        const int col = ((SPLIT_KEYS ? 0 : wave * NT) + ct) * 16 + i;
+        const int col = ct * 16 + i;
         col_ok[ct] = col < ncols;
         col_tok[ct] = t0 + (col_ok[ct] ? col / G : 0);
         col_head[ct] = kvh * G + (col_ok[ct] ? col % G : 0);
@@ -148,124 +132,108 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
     int b_begin = 0, b_end = 0, b_step = 1;
     if (hi_w >= 0) {
         const int b0 = lo_w / 32, b1 = hi_w / 32;
-        if (SPLIT_KEYS) {
-            const int nblocks = b1 - b0 + 1;
-            const int per = (nblocks + nsplit - 1) / nsplit;
-            b_begin = b0 + split * per + wave;
-            b_end = b0 + (split + 1) * per;
-            if (b_end > b1 + 1) b_end = b1 + 1;
-            b_step = AF_WAVES;
-        } else {
-            b_begin = b0;
-            b_end = b1 + 1;
-        }
+        const int nblocks = b1 - b0 + 1;
+        const int per = (nblocks + nsplit - 1) / nsplit;
+        b_begin = b0 + split * per + wave;
+        b_end = b0 + (split + 1) * per;
+        if (b_end > b1 + 1) b_end = b1 + 1;
+        b_step = W;
     }
     const float sc_mul = scale * LOG2E;
 
-    // Pages and operands of a block. K operands are fetched one block ahead and V operands
-    // before the scores are computed, so that their latency hides behind the MFMA work.
-    auto block_pages = [&](int b, int* page, int* slot0) {
+    // The page ids of this workgroup's key range go to LDS first (one round trip instead of one
+    // per block); K and V operands are fetched one block ahead of their use.
+    __shared__ int sh_pages[AF_MAX_CACHED_PAGES];
+    const int first_block = hi_w >= 0 ? lo_w / 32 : 0;
+    const int p_first = (32 * first_block) / page_size;
+    {
+        const int p_last = hi_w >= 0 ? hi_w / page_size : -1;
+        for (int p = p_first + (int)threadIdx.x; p <= p_last && p - p_first < AF_MAX_CACHED_PAGES; p += blockDim.x)
+            sh_pages[p - p_first] = p < bt_width ? bt[p] : -1;
+    }
+    __syncthreads();
+    auto page_of = [&](int pidx) -> int {
+        if (pidx >= bt_width) return -1;
+        const int rel = pidx - p_first;
+        return rel < AF_MAX_CACHED_PAGES ? sh_pages[rel] : bt[pidx];
+    };
+    struct Operands {
+        int page[2];
+        Frag k[2][DS];
+        Frag v[DT];
+    };
+    auto fetch = [&](int b, Operands& op) {
+        int slot0[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int key0 = 32 * b + 16 * t;
             const int pidx = key0 / page_size;
-            page[t] = (b < b_end && key0 <= hi_w && pidx < bt_width) ? bt[pidx] : -1;
-            slot0[t] = key0 % page_size;
+            op.page[t] = (b < b_end && key0 <= hi_w) ? page_of(pidx) : -1;
+            slot0[t] = key0 - pidx * page_size;
         }
-    };
-    auto load_k = [&](const int* page, const int* slot0, Frag (*kop)[DS]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            if (page[t] >= 0) {
-                const bf16* kptr =
-                    k_pages + (((size_t)page[t] * Hkv + kvh) * page_size + slot0[t] + i) * D + 8 * g;
+            if (op.page[t] >= 0) {
+                const size_t head = (size_t)op.page[t] * Hkv + kvh;
+                const bf16* kptr = k_pages + ((head * page_size + slot0[t] + i) * D + 8 * g);
 #pragma unroll
-                for (int s = 0; s < DS; ++s) kop[t][s].u = *reinterpret_cast<const uint4*>(kptr + 32 * s);
+                for (int s = 0; s < DS; ++s) op.k[t][s].u = *reinterpret_cast<const uint4*>(kptr + 32 * s);
+                const bf16* vptr = v_pages + (head * D + i) * page_size + slot0[t] + 4 * g;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    op.v[dt].h[t] = *reinterpret_cast<const uint2*>(vptr + (size_t)16 * dt * page_size);
             } else {
 #pragma unroll
-                for (int s = 0; s < DS; ++s) kop[t][s].u = uint4{0u, 0u, 0u, 0u};
+                for (int s = 0; s < DS; ++s) op.k[t][s].u = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) op.v[dt].h[t] = uint2{0u, 0u};
             }
         }
     };
-
-    int page[2], slot0[2];
-    Frag kop[2][DS];
-    block_pages(b_begin, page, slot0);
-    load_k(page, slot0, kop);
-
-    for (int b = b_begin; b < b_end; b += b_step) {
+    auto compute = [&](int b, Operands& op) {
         const int base = 32 * b;
-        // V^T operands of this block
-        Frag vop[DT];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (page[t] >= 0) {
-                    const bf16* vptr = v_pages + (((size_t)page[t] * Hkv + kvh) * D + 16 * dt + i) * page_size +
-                                       slot0[t] + 4 * g;
-                    vop[dt].h[t] = *reinterpret_cast<const uint2*>(vptr);
-                } else {
-                    vop[dt].h[t] = uint2{0u, 0u};
-                }
-            }
-        }
-        // K operands of the next block
-        int npage[2], nslot0[2];
-        Frag knext[2][DS];
-        block_pages(b + b_step, npage, nslot0);
-        load_k(npage, nslot0, knext);
-
         // scores^T for two tiles of 16 keys
-        float p[NT][2][4];
+        float p[2][4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            floatx4_t sacc[NT];
+            floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+            if (op.page[t] >= 0) {
 #pragma unroll
-            for (int ct = 0; ct < NT; ++ct) sacc[ct] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-            if (page[t] >= 0) {
-#pragma unroll
-                for (int ct = 0; ct < NT; ++ct)
-#pragma unroll
-                    for (int s = 0; s < DS; ++s)
-                        sacc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[t][s].v, qop[ct][s].v, sacc[ct], 0, 0, 0);
+                for (int s = 0; s < DS; ++s)
+                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.k[t][s].v, qop[0][s].v, sacc, 0, 0, 0);
             }
 #pragma unroll
-            for (int ct = 0; ct < NT; ++ct)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int key = base + 16 * t + 4 * g + r;
-                    const bool ok = page[t] >= 0 && col_ok[ct] && key <= col_pos[ct] && key >= col_lo[ct];
-                    p[ct][t][r] = ok ? sacc[ct][r] * sc_mul : -INFINITY;
-                }
+            for (int r = 0; r < 4; ++r) {
+                const int key = base + 16 * t + 4 * g + r;
+                const bool ok = op.page[t] >= 0 && col_ok[0] && key <= col_pos[0] && key >= col_lo[0];
+                p[t][r] = ok ? sacc[r] * sc_mul : -INFINITY;
+            }
         }
         // online softmax per column
-        Frag pop[NT];
+        Frag pop;
+        float mx = -INFINITY;
 #pragma unroll
-        for (int ct = 0; ct < NT; ++ct) {
-            float mx = -INFINITY;
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int r = 0; r < 4; ++r) mx = fmaxf(mx, p[t][r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
+        const float m_new = fmaxf(m_run[0], mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m_run[0] - m_safe);   // exp2(-inf) = 0
+        float psum = 0.f;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, p[ct][t][r]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
-            const float m_new = fmaxf(m_run[ct], mx);
-            const float corr = (m_new == -INFINITY) ? 1.f : exp2f(m_run[ct] - m_new);
-            float psum = 0.f;
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int r = 0; r < 4; ++r) {
+                const float e = __builtin_amdgcn_exp2f(p[t][r] - m_safe);
+                psum += e;
+                pop.v[t * 4 + r] = (__bf16)e;
+            }
+        l_run[0] = l_run[0] * corr + psum;
+        m_run[0] = m_new;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float e = (p[ct][t][r] == -INFINITY) ? 0.f : exp2f(p[ct][t][r] - m_new);
-                    psum += e;
-                    pop[ct].v[t * 4 + r] = (__bf16)e;
-                }
-            l_run[ct] = l_run[ct] * corr + psum;
-            m_run[ct] = m_new;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) acc_o[ct][dt] *= corr;
-        }
+        for (int dt = 0; dt < DT; ++dt) acc_o[0][dt] *= corr;
         // out^T += V^T P^T
         if (base + 31 > hi_w) {  // slots above the newest key were never written
 #pragma unroll
@@ -274,21 +242,21 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (base + 16 * t + 4 * g + r > hi_w) vop[dt].s[t * 4 + r] = 0;
+                        if (base + 16 * t + 4 * g + r > hi_w) op.v[dt].s[t * 4 + r] = 0;
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int ct = 0; ct < NT; ++ct)
-                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
-        // the prefetched block becomes the current one
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            page[t] = npage[t];
-            slot0[t] = nslot0[t];
-#pragma unroll
-            for (int s = 0; s < DS; ++s) kop[t][s] = knext[t][s];
-        }
+            acc_o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.v[dt].v, pop.v, acc_o[0][dt], 0, 0, 0);
+    };
+
+    Operands oa, ob;
+    fetch(b_begin, oa);
+    for (int b = b_begin; b < b_end; b += 2 * b_step) {
+        fetch(b + b_step, ob);
+        compute(b, oa);
+        if (b + b_step >= b_end) break;
+        fetch(b + 2 * b_step, oa);
+        compute(b + b_step, ob);
     }
 
     // the sum of a column is spread over the four lane groups
@@ -298,82 +266,69 @@ attention_mfma_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restric
         l_run[ct] += __shfl_xor(l_run[ct], 32, MV_WAVE);
     }
 
-    if (!SPLIT_KEYS) {
-#pragma unroll
-        for (int ct = 0; ct < NT; ++ct) {
-            if (!col_ok[ct]) continue;
-            const float inv = 1.f / l_run[ct];
-            bf16* orow = out + (size_t)col_tok[ct] * out_stride + (size_t)col_head[ct] * D;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                uint2 packed;
-                packed.x = (uint32_t)f32_to_bf16_bits(acc_o[ct][dt][0] * inv) |
-                           ((uint32_t)f32_to_bf16_bits(acc_o[ct][dt][1] * inv) << 16);
-                packed.y = (uint32_t)f32_to_bf16_bits(acc_o[ct][dt][2] * inv) |
-                           ((uint32_t)f32_to_bf16_bits(acc_o[ct][dt][3] * inv) << 16);
-                *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = packed;
-            }
-        }
-        return;
-    }
-
-    // ---- merge the four waves' partial results (same columns, disjoint keys)
-    __shared__ float sm_m[AF_WAVES][NT][16];
-    __shared__ float sm_l[AF_WAVES][NT][16];
-    __shared__ float sm_o[AF_WAVES][NT][DT][4][MV_WAVE];
-#pragma unroll
-    for (int ct = 0; ct < NT; ++ct) {
-        if (g == 0) {
-            sm_m[wave][ct][i] = m_run[ct];
-            sm_l[wave][ct][i] = l_run[ct];
-        }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sm_o[wave][ct][dt][r][lane] = acc_o[ct][dt][r];
+    // ---- merge the waves' partial results (same columns, disjoint keys) through LDS, half of the
+    // d tiles at a time
+    constexpr int HALF = DT / 2;
+    __shared__ float sm_m[W][16];
+    __shared__ float sm_l[W][16];
+    __shared__ float sm_o[W][HALF][4][MV_WAVE];
+    if (g == 0) {
+        sm_m[wave][i] = m_run[0];
+        sm_l[wave][i] = l_run[0];
     }
     __syncthreads();
+    float m_fin = -INFINITY;
 #pragma unroll
-    for (int ct = 0; ct < NT; ++ct) {
-        float m_fin = -INFINITY;
+    for (int w = 0; w < W; ++w) m_fin = fmaxf(m_fin, sm_m[w][i]);
+    float f[W], l_fin = 0.f;
 #pragma unroll
-        for (int w = 0; w < AF_WAVES; ++w) m_fin = fmaxf(m_fin, sm_m[w][ct][i]);
-        float f[AF_WAVES], l_fin = 0.f;
+    for (int w = 0; w < W; ++w) {
+        const float mw = sm_m[w][i];
+        f[w] = (mw == -INFINITY) ? 0.f : exp2f(mw - m_fin);
+        l_fin += f[w] * sm_l[w][i];
+    }
+    float* prow = nullptr;
+    bf16* orow = nullptr;
+    if (col_ok[0]) {
+        prow = partials ? partials + (((size_t)col_tok[0] * H + col_head[0]) * nsplit + split) * (D + 2) : nullptr;
+        orow = out + (size_t)col_tok[0] * out_stride + (size_t)col_head[0] * D;
+    }
 #pragma unroll
-        for (int w = 0; w < AF_WAVES; ++w) {
-            const float mw = sm_m[w][ct][i];
-            f[w] = (mw == -INFINITY) ? 0.f : exp2f(mw - m_fin);
-            l_fin += f[w] * sm_l[w][ct][i];
-        }
-        if (!col_ok[ct]) continue;
-        // the d tiles are dealt out to the waves
-        for (int dt = wave; dt < DT; dt += AF_WAVES) {
-            float o[4];
+    for (int half = 0; half < 2; ++half) {
+        if (half) __syncthreads();
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float a = 0.f;
+        for (int dt = 0; dt < HALF; ++dt)
 #pragma unroll
-                for (int w = 0; w < AF_WAVES; ++w) a += f[w] * sm_o[w][ct][dt][r][lane];
-                o[r] = a;
+            for (int r = 0; r < 4; ++r) sm_o[wave][dt][r][lane] = acc_o[0][half * HALF + dt][r];
+        __syncthreads();
+        if (col_ok[0]) {
+            // the d tiles of this half are dealt out to the waves
+            for (int dt = wave; dt < HALF; dt += W) {
+                float o[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float a = 0.f;
+#pragma unroll
+                    for (int w = 0; w < W; ++w) a += f[w] * sm_o[w][dt][r][lane];
+                    o[r] = a;
+                }
+                const int d0 = 16 * (half * HALF + dt) + 4 * g;
+                if (nsplit == 1) {
+                    const float inv = 1.f / l_fin;
+                    uint2 packed;
+                    packed.x = (uint32_t)f32_to_bf16_bits(o[0] * inv) | ((uint32_t)f32_to_bf16_bits(o[1] * inv) << 16);
+                    packed.y = (uint32_t)f32_to_bf16_bits(o[2] * inv) | ((uint32_t)f32_to_bf16_bits(o[3] * inv) << 16);
+                    *reinterpret_cast<uint2*>(orow + d0) = packed;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) prow[d0 + r] = o[r];
+                }
             }
-            if (nsplit == 1) {
-                const float inv = 1.f / l_fin;
-                bf16* orow = out + (size_t)col_tok[ct] * out_stride + (size_t)col_head[ct] * D;
-                uint2 packed;
-                packed.x = (uint32_t)f32_to_bf16_bits(o[0] * inv) | ((uint32_t)f32_to_bf16_bits(o[1] * inv) << 16);
-                packed.y = (uint32_t)f32_to_bf16_bits(o[2] * inv) | ((uint32_t)f32_to_bf16_bits(o[3] * inv) << 16);
-                *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = packed;
-            } else {
-                float* prow = partials + (((size_t)col_tok[ct] * H + col_head[ct]) * nsplit + split) * (D + 2);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) prow[16 * dt + 4 * g + r] = o[r];
-            }
         }
-        if (nsplit > 1 && wave == 0 && g == 0) {
-            float* prow = partials + (((size_t)col_tok[ct] * H + col_head[ct]) * nsplit + split) * (D + 2);
-            prow[D] = m_fin;
-            prow[D + 1] = l_fin;
-        }
+    }
+    if (nsplit > 1 && wave == 0 && g == 0 && col_ok[0]) {
+        prow[D] = m_fin;
+        prow[D + 1] = l_fin;
     }
 }
 
@@ -411,15 +366,14 @@ __global__ void attention_merge_kernel(const float* __restrict__ partials, bf16*
     }
 }
 
-template <int D, int NT, bool SPLIT_KEYS>
-static void launch_attention(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
-                             const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
-                             int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int decode_only,
-                             int H, int Hkv, float scale, int window, float* partials, int nsplit) {
-    hipLaunchKernelGGL((attention_mfma_kernel<D, NT, SPLIT_KEYS>), grid, dim3(64 * AF_WAVES), 0, stream,
-                       (const bf16*)q, q_stride, (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages,
-                       block_table, bt_width, page_size, positions, cu_seqlens, n_seqs, decode_only, H, Hkv, scale,
-                       window, partials, nsplit);
+template <int D, int W>
+static void launch_decode(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
+                          const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
+                          int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv,
+                          float scale, int window, float* partials, int nsplit) {
+    hipLaunchKernelGGL((attention_decode_kernel<D, W>), grid, dim3(64 * W), 0, stream, (const bf16*)q, q_stride,
+                       (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,
+                       page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit);
 }
 
 static int check_common(const char* what, long q_stride, long out_stride, int page_size, int bt_width, int H, int Hkv,
@@ -434,27 +388,29 @@ static int check_common(const char* what, long q_stride, long out_stride, int pa
     return 0;
 }
 
-// Decode steps: every sequence brings one token. grid = (sequences, kv heads, nsplit).
-// partials: float [n_seqs * H * nsplit * (D + 2)], needed when nsplit > 1.
+// Decode steps: every sequence brings one token. grid = (sequences, kv heads, nsplit); `waves` (4
+// or 8) per workgroup. partials: float [n_seqs * H * nsplit * (D + 2)], needed when nsplit > 1.
 extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
                                    const void* v_pages, const int* block_table, int bt_width, int page_size,
                                    const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
-                                   float scale, int window, float* partials, int nsplit, const int* token_seq,
-                                   hipStream_t stream) {
+                                   float scale, int window, float* partials, int nsplit, int waves,
+                                   const int* token_seq, hipStream_t stream) {
     if (int rc = check_common("attention_decode", q_stride, out_stride, page_size, bt_width, H, Hkv, D)) return rc;
     MV_REQUIRE(H / Hkv <= 16, "attention_decode: %d query heads per kv head exceed 16", H / Hkv);
     MV_REQUIRE(nsplit >= 1 && nsplit <= AF_MAX_SPLITS && (nsplit == 1 || partials != nullptr),
                "attention_decode: bad split count %d or missing work area", nsplit);
+    MV_REQUIRE(waves == 4 || waves == 8, "attention_decode: %d waves per workgroup (4 or 8)", waves);
     if (n_seqs <= 0) return 0;
     dim3 grid(n_seqs, Hkv, nsplit);
-    if (D == 128)
-        launch_attention<128, 1, true>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,
-                                       bt_width, page_size, positions, cu_seqlens, n_seqs, 1, H, Hkv, scale, window,
-                                       partials, nsplit);
-    else
-        launch_attention<64, 1, true>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,
-                                      bt_width, page_size, positions, cu_seqlens, n_seqs, 1, H, Hkv, scale, window,
-                                      partials, nsplit);
+    float* part = nsplit > 1 ? partials : nullptr;
+#define AF_LAUNCH(DD, WW)                                                                                         \
+    launch_decode<DD, WW>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,      \
+                          page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, part, nsplit)
+    if (D == 128 && waves == 8) AF_LAUNCH(128, 8);
+    else if (D == 128) AF_LAUNCH(128, 4);
+    else if (waves == 8) AF_LAUNCH(64, 8);
+    else AF_LAUNCH(64, 4);
+#undef AF_LAUNCH
     if (int rc = mv_check_launch("attention_decode")) return rc;
     if (nsplit > 1) {
         hipLaunchKernelGGL(attention_merge_kernel, dim3(n_seqs, H), dim3(D >= 128 ? 128 : 64), 0, stream, partials,
@@ -463,4 +419,3 @@ extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long
     }
     return 0;
 }
-

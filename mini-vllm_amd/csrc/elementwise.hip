@@ -171,7 +171,7 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, long row_stride, 
     const int wave = threadIdx.x / MV_WAVE;
     const int lane = threadIdx.x % MV_WAVE;
     const int head = blockIdx.y * 4 + wave;
-    const int total = H + (store_kv ? 2 * Hkv : 0);
+    const int total = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
     const int seq = token_seq[tok];
     const int pos = positions[tok];
     const bool active = head < total && seq >= 0;
@@ -256,7 +256,7 @@ extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int 
     MV_REQUIRE(!has_norm || eps > 0.f, "qk_norm_rope_store: eps must be positive");
     MV_REQUIRE(mv_valid_dtype(weight_dtype), "qk_norm_rope_store: bad weight dtype %d", weight_dtype);
     if (n == 0) return 0;
-    const int heads = H + (store_kv ? 2 * Hkv : 0);
+    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
     WeightPtr qw{q_weight, weight_dtype}, kw{k_weight, weight_dtype};
     dim3 grid(n, (heads + 3) / 4);
     MV_DISPATCH_T(dtype, "qk_norm_rope_store",
@@ -265,6 +265,64 @@ extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int 
                                      (T*)k_pages, (T*)v_pages, H, Hkv, D, qw, kw, has_norm, eps, unit_offset, table,
                                      rot_dim, interleaved, store_kv));
     return mv_check_launch("qk_norm_rope_store");
+}
+
+// ---------------------------------------------------------------------------------------
+// Value rows of many tokens into the transposed value pages V[page][kv_head][d][slot].
+// A workgroup takes 16 consecutive tokens of the step and one kv head, stages their value rows in
+// LDS, and writes with the token index running fastest over the lanes: tokens that follow each
+// other in a sequence fill neighbouring slots, so the two-byte stores of a wave merge into
+// 32-byte segments (the per-token kernel above scatters them 2 bytes at a time).
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+store_v_pages_kernel(const T* __restrict__ qkv, long row_stride, int v_off, const int* __restrict__ positions,
+                     const int* __restrict__ token_seq, const int* __restrict__ block_table, int bt_width,
+                     int page_size, T* __restrict__ v_pages, int n, int Hkv, int D) {
+    __shared__ float tile[16][MV_MAX_HEAD_DIM + 1];
+    __shared__ long dst_base[16];
+    const int tok0 = blockIdx.x * 16;
+    const int kvh = blockIdx.y;
+    const int tid = threadIdx.x;
+    if (tid < 16) {
+        const int tok = tok0 + tid;
+        long base = -1;
+        if (tok < n) {
+            const int seq = token_seq[tok];
+            if (seq >= 0) {
+                const int pos = positions[tok];
+                const int page = block_table[(size_t)seq * bt_width + pos / page_size];
+                if (page >= 0) base = ((long)page * Hkv + kvh) * D * page_size + pos % page_size;
+            }
+        }
+        dst_base[tid] = base;
+    }
+    for (int idx = tid; idx < 16 * D; idx += 256) {
+        const int j = idx / D, d = idx % D;
+        const int tok = tok0 + j;
+        tile[j][d] = tok < n ? to_f(qkv[(size_t)tok * row_stride + v_off + (size_t)kvh * D + d]) : 0.f;
+    }
+    __syncthreads();
+    const int j = tid % 16;
+    const long base = dst_base[j];
+    if (base < 0) return;
+    for (int d = tid / 16; d < D; d += 16) v_pages[base + (long)d * page_size] = from_f<T>(tile[j][d]);
+}
+
+extern "C" int mv_store_v_pages(const void* qkv, long row_stride, int v_off, const int* positions,
+                                const int* token_seq, const int* block_table, int bt_width, int page_size,
+                                void* v_pages, int n, int Hkv, int D, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && Hkv > 0 && D > 0 && D <= MV_MAX_HEAD_DIM, "store_v_pages: bad sizes n=%d Hkv=%d D=%d", n, Hkv,
+               D);
+    MV_REQUIRE(block_table && v_pages && page_size > 0 && bt_width > 0, "store_v_pages: missing pages or block table");
+    MV_REQUIRE(Hkv <= 65535, "store_v_pages: too many kv heads");
+    if (n == 0) return 0;
+    dim3 grid((n + 15) / 16, Hkv);
+    MV_DISPATCH_T(dtype, "store_v_pages",
+                  hipLaunchKernelGGL(store_v_pages_kernel<T>, grid, dim3(256), 0, stream, (const T*)qkv, row_stride,
+                                     v_off, positions, token_seq, block_table, bt_width, page_size, (T*)v_pages, n,
+                                     Hkv, D));
+    return mv_check_launch("store_v_pages");
 }
 
 // ---------------------------------------------------------------------------------------

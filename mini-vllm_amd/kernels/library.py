@@ -35,6 +35,8 @@ _SIGNATURES = {
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int,  # k, v pages, n, H, Hkv, D
                                       c_void_p, c_void_p, c_int, c_float, c_int,       # qw, kw, wdtype, eps, unit
                                       c_void_p, c_int, c_int, c_int, c_int, c_void_p]),  # table, rot, inter, store, dtype
+    "mv_store_v_pages": (c_int, [c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                 c_int, c_int, c_int, c_int, c_void_p]),
     "mv_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_ref": (c_int, [c_void_p, c_long, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_int,
                             c_int, c_int, c_int, c_void_p]),
@@ -51,7 +53,7 @@ _OPTIONAL_SIGNATURES = {
     "mv_gemm_skinny_swiglu": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),
     "mv_attention_decode": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
-                                    c_void_p, c_int, c_void_p, c_void_p]),
+                                    c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "mv_attention_prefill": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                      c_void_p]),

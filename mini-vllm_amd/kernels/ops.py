@@ -17,6 +17,10 @@ _NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
 
 # largest number of rows the weight-streaming product takes in one launch
 SKINNY_MAX_M = 64
+# waves per workgroup of the decode attention
+DECODE_ATTENTION_WAVES = 4
+# from this many tokens on, value rows are written to their pages by a kernel of their own
+STORE_V_SPLIT_TOKENS = 64
 
 
 def dtype_from_name(name: str) -> torch.dtype:
@@ -52,11 +56,21 @@ class Ops:
         self.lib = library.load(library.variant_of(_NAMES[dtype]))
         self.use_fast_kernels = dtype == torch.bfloat16
         self.use_library_gemm = dtype == torch.bfloat16
+        self.stream_handle: Optional[int] = None
+        self._transposed = {}
 
     # ------------------------------------------------------------------------------------
-    @staticmethod
-    def _stream() -> int:
-        return torch.cuda.current_stream().cuda_stream
+    def bind_stream(self) -> None:
+        """Looks the current stream up once; until ``unbind_stream`` every launch goes there.
+        (Asking for the current stream costs more than a launch; a step asks once.)"""
+        self.stream_handle = torch.cuda.current_stream().cuda_stream
+
+    def unbind_stream(self) -> None:
+        self.stream_handle = None
+
+    def _stream(self) -> int:
+        h = self.stream_handle
+        return h if h is not None else torch.cuda.current_stream().cuda_stream
 
     def _act(self, t: torch.Tensor, what: str) -> None:
         _dev(t, what)
@@ -180,11 +194,20 @@ class Ops:
             bt_width = block_table.shape[1]
         q_dim = num_heads * head_dim
         kv_dim = num_kv_heads * head_dim
-        self.lib.call("mv_qk_norm_rope_store", qkv.data_ptr(), qkv.stride(0) if n > 1 else width, 0, q_dim,
+        stride = qkv.stride(0) if n > 1 else width
+        # with many tokens the values go to their transposed pages in a pass of their own, in
+        # which neighbouring tokens write neighbouring slots; with few, one launch does everything
+        split_v = store and n >= STORE_V_SPLIT_TOKENS
+        mode = 0 if not store else (2 if split_v else 1)
+        self.lib.call("mv_qk_norm_rope_store", qkv.data_ptr(), stride, 0, q_dim,
                       q_dim + kv_dim, positions.data_ptr(), token_seq.data_ptr(), _ptr(block_table), bt_width,
                       page_size, _ptr(k_pages), _ptr(v_pages), n, num_heads, num_kv_heads, head_dim,
                       _ptr(q_weight), _ptr(k_weight), wcode, float(eps), int(unit_offset), _ptr(rope_table), rot,
-                      int(interleaved), int(store), self.code, self._stream())
+                      int(interleaved), mode, self.code, self._stream())
+        if split_v:
+            self.lib.call("mv_store_v_pages", qkv.data_ptr(), stride, q_dim + kv_dim, positions.data_ptr(),
+                          token_seq.data_ptr(), block_table.data_ptr(), bt_width, page_size, v_pages.data_ptr(), n,
+                          num_kv_heads, head_dim, self.code, self._stream())
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
         """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
@@ -233,10 +256,13 @@ class Ops:
                                   self._stream())
                 return
         if fast and self.use_library_gemm and out.dtype == self.dtype and M > SKINNY_MAX_M:
+            wt = self._transposed.get(w.data_ptr())
+            if wt is None or wt.shape != (K, N):
+                wt = self._transposed[w.data_ptr()] = w.t()      # the view is made once per weight
             if bias is None:
-                torch.mm(a, w.t(), out=out)
+                torch.mm(a, wt, out=out)
             else:
-                torch.addmm(bias, a, w.t(), out=out)
+                torch.addmm(bias, a, wt, out=out)
             return
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
@@ -315,13 +341,13 @@ class Ops:
         group = H // Hkv
         n_seqs = plan.n_seqs
         if plan.decode_only and group <= 16:
-            # Split the keys of a sequence over several workgroups until about 512 workgroups are
-            # in flight, but never below 128 keys per split (measured on MI355X: batch 1 and 8 are
-            # fastest at 8 splits for 1K contexts, batch 64 without a split). The count is a
-            # property of the plan (a captured graph keeps it); each split takes its share of the
-            # keys a sequence actually has.
+            # Split the keys of a sequence over several workgroups until about 256 workgroups are
+            # in flight, but never below 128 keys per split (measured on MI355X with 8 kv heads:
+            # batch 1 is fastest at 8 to 16 splits, batch 8 at 4, batch 64 without a split). The
+            # count is a property of the plan (a captured graph keeps it); each split takes its
+            # share of the keys a sequence actually has.
             ctx = max(1, plan.max_context_len)
-            nsplit = max(1, min(512 // max(1, n_seqs * Hkv), max(1, ctx // 128), 64))
+            nsplit = max(1, min(256 // max(1, n_seqs * Hkv), max(1, ctx // 128), 64))
             partials = None
             if nsplit > 1:
                 rows = max(n_seqs * nsplit, 2048 // Hkv, 256)      # one size serves every batch of a graph set
@@ -329,7 +355,7 @@ class Ops:
             self.lib.call("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
-                          _ptr(partials), nsplit, token_seq.data_ptr(), self._stream())
+                          _ptr(partials), nsplit, DECODE_ATTENTION_WAVES, token_seq.data_ptr(), self._stream())
             return True
         if page_size & (page_size - 1):
             return False

@@ -126,6 +126,14 @@ class CausalLM:
     def forward(self, ctx) -> torch.Tensor:
         """Runs the step described by ``ctx`` and returns float32 logits [len(logit_rows), vocab]."""
         rt, plan = self.rt, self.plan
+        rt.ops.bind_stream()
+        try:
+            return self._forward(ctx)
+        finally:
+            rt.ops.unbind_stream()
+
+    def _forward(self, ctx) -> torch.Tensor:
+        rt, plan = self.rt, self.plan
         n = ctx.n_tokens
         resid = rt.workspace.get("resid", (n, plan.hidden_size), torch.float32)
         rt.ops.embedding(ctx.token_ids, self.embedding_table, resid, self.embedding_scale)

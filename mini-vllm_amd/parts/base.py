@@ -123,11 +123,16 @@ class Workspace:
         hold its address go on working."""
         self.device = device
         self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self._views: Dict[Tuple, torch.Tensor] = {}
         self._retired: List[torch.Tensor] = []
         self.retain = retain
         self.frozen = False
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        vkey = (name, dtype, tuple(shape))
+        view = self._views.get(vkey)          # making a view costs as much as a launch: keep them
+        if view is not None:
+            return view
         n = 1
         for s in shape:
             n *= int(s)
@@ -140,7 +145,13 @@ class Workspace:
                 self._retired.append(buf)
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-        return buf[:n].view(*shape)
+            for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[k]             # views of the replaced buffer
+        view = buf[:n].view(*shape)
+        if len(self._views) > 4096:
+            self._views.clear()
+        self._views[vkey] = view
+        return view
 
     def bytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in list(self._buffers.values()) + self._retired)

@@ -166,6 +166,50 @@ def test_qk_norm_rope_store(dtype, H, Hkv, D, rot, inter):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,D,ps", [(4, 2, 128, 16), (3, 3, 48, 8)])
+def test_qk_norm_rope_store_many_tokens(dtype, H, Hkv, D, ps):
+    """Enough tokens for the separate value pass: three sequences (one starting mid-page, one
+    padding row), pages in scrambled order, untouched slots must stay untouched."""
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(33)
+    spans = [(0, 50), (21, 40), (5, 7)]                       # (start position, tokens)
+    positions, token_seq = [], []
+    for s_, (start, cnt) in enumerate(spans):
+        positions += list(range(start, start + cnt)); token_seq += [s_] * cnt
+    n = len(positions)
+    token_seq[60] = -1
+    pages_per = [-(-(start + cnt) // ps) for start, cnt in spans]
+    num_pages = sum(pages_per) + 2
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    bt = torch.full((3, max(pages_per)), -1, dtype=torch.int32)
+    cur = 0
+    for s_, n_p in enumerate(pages_per):
+        bt[s_, :n_p] = torch.tensor(perm[cur:cur + n_p], dtype=torch.int32); cur += n_p
+    positions = torch.tensor(positions, dtype=torch.int32); token_seq = torch.tensor(token_seq, dtype=torch.int32)
+    qkv = torch.randn(n, (H + 2 * Hkv) * D, generator=g).to(dtype)
+    kp, vp = paged_cache(num_pages, Hkv, ps, D, dtype)
+    kp.fill_(9.0); vp.fill_(9.0)
+    qd = dev(qkv).clone()
+    ops.qk_norm_rope_store(qd, H, Hkv, D, dev(positions), dev(token_seq), None, None, 1e-6, None, False, kp, vp, dev(bt), ps)
+    kc, vc = kp.float().cpu(), vp.float().cpu()
+    k = qkv[:, H * D:(H + Hkv) * D].float().view(n, Hkv, D)
+    v = qkv[:, (H + Hkv) * D:].float().view(n, Hkv, D)
+    written = set()
+    for i in range(n):
+        if token_seq[i] < 0:
+            continue
+        page = int(bt[token_seq[i], positions[i] // ps]); slot = int(positions[i] % ps)
+        written.add((page, slot))
+        assert torch.equal(kc[page, :, slot, :], k[i]) and torch.equal(vc[page, :, :, slot], v[i]), i
+    for page in range(num_pages):
+        for slot in range(ps):
+            if (page, slot) not in written:
+                assert float((kc[page, :, slot, :] - 9.0).abs().max()) == 0.0
+                assert float((vc[page, :, :, slot] - 9.0).abs().max()) == 0.0
+    assert torch.equal(qd.cpu(), qkv)                         # no norm, no rotation: q is unchanged
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_swiglu(dtype):
     ops = ops_for(dtype)
     g = torch.Generator().manual_seed(4)
