@@ -12,13 +12,14 @@
 //
 // A fused variant computes the gated activation of a feed-forward in the same pass:
 //     out[M, I] = silu(A Wg^T) * (A Wu^T)  with Wg = W[0:I], Wu = W[I:2I].
-#include "common.h"
+#include "dispatch.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
 union Frag {
     uint4 u;
+    uint16_t s[8];
     bf16x8_t v;
 };
 
@@ -28,13 +29,28 @@ template <typename TC> __device__ __forceinline__ void store_c(TC* p, float v);
 template <> __device__ __forceinline__ void store_c<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void store_c<bf16>(bf16* p, float v) { *p = from_f<bf16>(v); }
 
+// What the NORM variant computes in front of the product (see below).
+struct NormInput {
+    const float* resid_in;   // [M, K] float
+    const bf16* delta;       // [M, K] or null
+    float* resid_out;        // [M, K] float, or null when delta is null
+    WeightPtr weight;        // [K]
+    float eps;
+    int unit_offset;
+};
+
 // R: 16-row weight tiles per workgroup; TM: 16-token tiles (M <= 16 * TM); SWIGLU: R == 2 and
 // the two tiles are the gate rows and the up rows of the same output columns.
-template <int R, int TM, bool SWIGLU, typename TC>
+// NORM (TM == 1): the activations are not read from A but made here:
+//     x = resid_in + delta;  A[m][k] = bf16(x[m][k] * rsqrt(mean_k x[m]^2 + eps) * weight[k])
+// Every workgroup normalises the (few) rows for itself into LDS, which costs less than a kernel
+// launch; workgroup 0 also writes x to resid_out (a buffer other than resid_in: the other
+// workgroups still read that one).
+template <int R, int TM, bool SWIGLU, bool NORM, typename TC>
 __global__ void __launch_bounds__(64 * SK_MAX_WAVES)
 gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W, const bf16* __restrict__ bias,
-                   TC* __restrict__ C, long ldc, int M, int N, int K) {
-    extern __shared__ float red[];  // [S - 1][R * TM][64][4]
+                   TC* __restrict__ C, long ldc, int M, int N, int K, NormInput norm) {
+    extern __shared__ float red[];  // [S - 1][R * TM][64][4], then (NORM) bf16 [M][K + 8]
     const int S = blockDim.x / MV_WAVE;
     const int wave = threadIdx.x / MV_WAVE;
     const int lane = threadIdx.x % MV_WAVE;
@@ -64,11 +80,71 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     }
     const uint4* arow[TM];
     bool avalid[TM];
+    if (NORM) {
+        bf16* sA = reinterpret_cast<bf16*>(red + (size_t)(S - 1) * R * TM * 256);
+        const int lds_ld = K + 8;  // row pitch in elements: the 16 rows an operand load touches fall into different banks
+        for (int m = wave; m < M; m += S) {
+            const float* xr = norm.resid_in + (size_t)m * K;
+            const bf16* dr = norm.delta ? norm.delta + (size_t)m * K : nullptr;
+            float ss = 0.f;
+            for (int c = lane * 8; c < K; c += 64 * 8) {
+                float x[8];
+                const float4 r0 = *reinterpret_cast<const float4*>(xr + c);
+                const float4 r1 = *reinterpret_cast<const float4*>(xr + c + 4);
+                x[0] = r0.x; x[1] = r0.y; x[2] = r0.z; x[3] = r0.w;
+                x[4] = r1.x; x[5] = r1.y; x[6] = r1.z; x[7] = r1.w;
+                if (dr) {
+                    Frag d;
+                    d.u = *reinterpret_cast<const uint4*>(dr + c);
 #pragma unroll
-    for (int t = 0; t < TM; ++t) {
-        const int tok = 16 * t + i;
-        avalid[t] = tok < M;
-        arow[t] = reinterpret_cast<const uint4*>(A + (size_t)(avalid[t] ? tok : 0) * lda) + g;
+                    for (int e = 0; e < 8; ++e) x[e] += (float)d.v[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+            }
+            ss = wave_sum(ss);
+            const float rinv = rsqrtf(ss / (float)K + norm.eps);
+            for (int c = lane * 8; c < K; c += 64 * 8) {
+                float x[8];
+                const float4 r0 = *reinterpret_cast<const float4*>(xr + c);
+                const float4 r1 = *reinterpret_cast<const float4*>(xr + c + 4);
+                x[0] = r0.x; x[1] = r0.y; x[2] = r0.z; x[3] = r0.w;
+                x[4] = r1.x; x[5] = r1.y; x[6] = r1.z; x[7] = r1.w;
+                if (dr) {
+                    Frag d;
+                    d.u = *reinterpret_cast<const uint4*>(dr + c);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[e] += (float)d.v[e];
+                    if (blockIdx.x == 0) {
+                        float* yr = norm.resid_out + (size_t)m * K + c;
+                        *reinterpret_cast<float4*>(yr) = float4{x[0], x[1], x[2], x[3]};
+                        *reinterpret_cast<float4*>(yr + 4) = float4{x[4], x[5], x[6], x[7]};
+                    }
+                }
+                Frag o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float wt = norm.weight.at(c + e);
+                    if (norm.unit_offset) wt += 1.f;
+                    o.s[e] = f32_to_bf16_bits(x[e] * rinv * wt);
+                }
+                *reinterpret_cast<uint4*>(sA + (size_t)m * lds_ld + c) = o.u;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < TM; ++t) {
+            const int tok = 16 * t + i;
+            avalid[t] = tok < M;
+            arow[t] = reinterpret_cast<const uint4*>(sA + (size_t)(avalid[t] ? tok : 0) * lds_ld) + g;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < TM; ++t) {
+            const int tok = 16 * t + i;
+            avalid[t] = tok < M;
+            arow[t] = reinterpret_cast<const uint4*>(A + (size_t)(avalid[t] ? tok : 0) * lda) + g;
+        }
     }
 
     floatx4_t acc[R][TM];
@@ -165,14 +241,30 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     }
 }
 
+static size_t skinny_lds_bytes(int S, int R, int TM, bool with_norm, int M, int K) {
+    size_t lds = (size_t)(S - 1) * R * TM * 256 * sizeof(float);
+    if (with_norm) lds += (size_t)M * (K + 8) * sizeof(uint16_t);
+    return lds;
+}
+
 template <int R, int TM, bool SWIGLU, typename TC>
 static void launch_skinny(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N,
                           int K, int S, hipStream_t stream) {
     const int tiles = (N + 15) / 16;
     const int blocks = SWIGLU ? tiles : (tiles + R - 1) / R;
-    const size_t lds = (size_t)(S - 1) * R * TM * 256 * sizeof(float);
-    hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, TC>), dim3(blocks), dim3(64 * S), lds, stream,
-                       (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K);
+    const size_t lds = skinny_lds_bytes(S, R, TM, false, M, K);
+    hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC>), dim3(blocks), dim3(64 * S), lds, stream,
+                       (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, NormInput{});
+}
+
+template <int R, bool SWIGLU, typename TC>
+static void launch_skinny_norm(const NormInput& norm, const void* W, const void* bias, void* C, long ldc, int M, int N,
+                               int K, int S, hipStream_t stream) {
+    const int tiles = (N + 15) / 16;
+    const int blocks = SWIGLU ? tiles : (tiles + R - 1) / R;
+    const size_t lds = skinny_lds_bytes(S, R, 1, true, M, K);
+    hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC>), dim3(blocks), dim3(64 * S), lds, stream,
+                       (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, norm);
 }
 
 static int pick_waves(int K) {
@@ -238,4 +330,35 @@ extern "C" int mv_gemm_skinny_swiglu(const void* A, long lda, const void* Wgu, v
     int rc = dispatch_tm<2, true, bf16>(A, lda, Wgu, nullptr, out, ldo, M, I, K, S, stream);
     if (rc) return rc;
     return mv_check_launch("gemm_skinny_swiglu");
+}
+
+// The product (or the gated pair with `swiglu`) with the residual add and RMSNorm in front:
+//     x = resid_in + delta (delta may be null); resid_out = x (written when delta is given);
+//     A = bf16(rmsnorm(x) * weight);  C = A W^T (+ bias)   or   C = silu(A Wg^T) * (A Wu^T).
+// At most 16 rows, K a multiple of 64, and the rows must fit LDS beside the partial tiles; returns
+// 2 (and sets the error text) when the shape is not taken, so that the caller can run the two
+// steps separately.
+extern "C" int mv_gemm_skinny_norm(const float* resid_in, const void* delta, float* resid_out, const void* norm_weight,
+                                   int norm_weight_dtype, float eps, int unit_offset, const void* W, const void* bias,
+                                   void* C, long ldc, int c_dtype, int M, int N, int K, int swiglu,
+                                   hipStream_t stream) {
+    MV_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny_norm: bad sizes M=%d N=%d K=%d", M, N, K);
+    MV_REQUIRE(mv_valid_dtype(norm_weight_dtype) && norm_weight != nullptr, "gemm_skinny_norm: bad norm weight");
+    MV_REQUIRE(delta == nullptr || (resid_out != nullptr && resid_out != resid_in),
+               "gemm_skinny_norm: the updated residual needs a buffer of its own");
+    MV_REQUIRE(eps > 0.f, "gemm_skinny_norm: eps must be positive");
+    MV_REQUIRE(ldc >= N, "gemm_skinny_norm: ldc=%ld smaller than N=%d", ldc, N);
+    MV_REQUIRE(c_dtype == MV_BF16 || (c_dtype == MV_F32 && !swiglu), "gemm_skinny_norm: bad output dtype %d", c_dtype);
+    if (M == 0) return 0;
+    const int S = pick_waves(K);
+    const int R = swiglu ? 2 : 1;
+    if (M > 16 || K % 64 != 0 || skinny_lds_bytes(S, R, 1, true, M, K) > 60 * 1024) {
+        mv_fail("gemm_skinny_norm: M=%d K=%d is not taken by the fused kernel", M, K);
+        return 2;
+    }
+    NormInput norm{resid_in, (const bf16*)delta, resid_out, WeightPtr{norm_weight, norm_weight_dtype}, eps, unit_offset};
+    if (swiglu) launch_skinny_norm<2, true, bf16>(norm, W, nullptr, C, ldc, M, N, K, S, stream);
+    else if (c_dtype == MV_F32) launch_skinny_norm<1, false, float>(norm, W, bias, C, ldc, M, N, K, S, stream);
+    else launch_skinny_norm<1, false, bf16>(norm, W, bias, C, ldc, M, N, K, S, stream);
+    return mv_check_launch("gemm_skinny_norm");
 }

@@ -17,6 +17,8 @@ _NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
 
 # largest number of rows the weight-streaming product takes in one launch
 SKINNY_MAX_M = 64
+# most rows for which residual add and norm are fused into the following product
+FUSED_NORM_MAX_M = 16
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
 # from this many tokens on, value rows are written to their pages by a kernel of their own
@@ -225,7 +227,14 @@ class Ops:
         float32 compute always takes the exact kernel. bfloat16 compute takes the
         weight-streaming MFMA kernel for up to SKINNY_MAX_M rows, the library's matrix product
         for more rows, and the exact kernel when the weight is stored in float32, when
-        ``exact`` is set or when no other kernel takes the shape."""
+        ``exact`` is set or when no other kernel takes the shape.
+
+        ``a`` may be a pending norm (parts.base.PendingNorm): then the residual add, the norm and
+        the product run as one kernel when the step has at most 16 rows, else the norm runs first."""
+        if not isinstance(a, torch.Tensor):
+            if not exact and self._gemm_fused_norm(a, w, out, bias, swiglu=False):
+                return
+            a = a.materialize()
         self._act(a, "gemm input"); _dev(w, "gemm weight"); _dev(out, "gemm output")
         if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
             raise KernelLibraryError("gemm: operands must be matrices")
@@ -267,10 +276,44 @@ class Ops:
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
 
+    def can_fuse_norm(self, rows: int, width: int) -> bool:
+        """Whether a norm over ``rows`` x ``width`` may be deferred into the next product."""
+        return (self.use_fast_kernels and self.lib.has("mv_gemm_skinny_norm") and 0 < rows <= FUSED_NORM_MAX_M
+                and width % 64 == 0 and rows * (width + 8) * 2 <= 44 * 1024)
+
+    def _gemm_fused_norm(self, pending, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor],
+                         swiglu: bool) -> bool:
+        """add + RMSNorm + product (or gated pair) in one kernel; False if the shape is not taken
+        (nothing has been done then)."""
+        M, K = pending.shape
+        norm = pending.norm
+        weight = getattr(norm, "weight", None)
+        spec = getattr(norm, "spec", None)
+        if (weight is None or spec is None or getattr(spec, "kind", "") != "rmsnorm" or not self.can_fuse_norm(M, K)
+                or w.dtype != torch.bfloat16 or not w.is_contiguous() or w.shape[1] != K
+                or out.stride(1) != 1 or (swiglu and (w.shape[0] % 2 or out.dtype != torch.bfloat16))):
+            return False
+        N = w.shape[0] // 2 if swiglu else w.shape[0]
+        if out.shape != (M, N) or out.dtype not in (torch.bfloat16, torch.float32):
+            return False
+        if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N):
+            return False
+        resid_in, delta, resid_out = pending.fused()
+        self.lib.call("mv_gemm_skinny_norm", resid_in.data_ptr(), _ptr(delta), _ptr(resid_out), weight.data_ptr(),
+                      _weight_code(weight, "norm weight"), float(spec.eps), int(spec.unit_offset), w.data_ptr(),
+                      _ptr(bias), out.data_ptr(), out.stride(0) if M > 1 else N, _CODES[out.dtype], M, N, K,
+                      int(swiglu), self._stream())
+        return True
+
     def gemm_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> bool:
         """out[M, I] = silu(a Wg^T) * (a Wu^T) for the packed weight [2I, K] in one pass over the
         weight, when the weight-streaming kernel takes the shape. Returns False (and does nothing)
-        otherwise; the caller then runs the product and the activation separately."""
+        otherwise; the caller then runs the product and the activation separately. ``a`` may be a
+        pending norm, as in ``gemm``."""
+        if not isinstance(a, torch.Tensor):
+            if self._gemm_fused_norm(a, w_gate_up, out, None, swiglu=True):
+                return True
+            a = a.materialize()
         if not (self.use_fast_kernels and self.lib.has("mv_gemm_skinny_swiglu")):
             return False
         M, K = a.shape

@@ -137,7 +137,7 @@ class CausalLM:
         n = ctx.n_tokens
         resid = rt.workspace.get("resid", (n, plan.hidden_size), torch.float32)
         rt.ops.embedding(ctx.token_ids, self.embedding_table, resid, self.embedding_scale)
-        stream = HiddenStream(resid)
+        stream = HiddenStream(resid, rt.workspace.get("resid.spare", (n, plan.hidden_size), torch.float32))
         for call_index, call in enumerate(plan.calls):
             self.blocks[call.layer].forward(stream, ctx, call_index)
         m = ctx.n_logit_rows

@@ -46,6 +46,7 @@ class AttentionSpec(PartSpec):
 @register_mixer(AttentionSpec.kind)
 class Attention(Mixer):
     spec_class = AttentionSpec
+    accepts_pending_norm = True      # the input is used by one packed product only
 
     @classmethod
     def tensors(cls, spec: AttentionSpec) -> Dict[str, TensorDecl]:

@@ -172,11 +172,53 @@ class HiddenStream:
     ``delta`` that has not been added yet. A norm consumes the pending delta (one fused
     kernel adds it and normalises the sum)."""
 
-    __slots__ = ("resid", "delta")
+    __slots__ = ("resid", "delta", "spare")
 
-    def __init__(self, resid: torch.Tensor):
+    def __init__(self, resid: torch.Tensor, spare: Optional[torch.Tensor] = None):
         self.resid = resid
         self.delta: Optional[torch.Tensor] = None
+        # a second buffer of the same shape: a kernel that adds the delta while other workgroups
+        # still read the old sum writes the new sum here, and the two change places
+        self.spare = spare
+
+
+class PendingNorm:
+    """A norm that has not run yet: the stream whose pending delta it will add, and its weight
+    and constants. A part whose first operation is one matrix product over its input may take
+    this instead of a tensor (it declares ``accepts_pending_norm = True``) and hand it to
+    ``ops.gemm`` / ``ops.gemm_swiglu``, which fuse add, norm and product into one kernel when the
+    step is small enough, and otherwise call ``materialize`` and go on as usual. It must be used
+    exactly once."""
+
+    def __init__(self, norm, stream: HiddenStream, ctx):
+        self.norm, self.stream, self.ctx = norm, stream, ctx
+        self.shape = stream.resid.shape
+        self.used = False
+        self._tensor: Optional[torch.Tensor] = None
+
+    def materialize(self) -> torch.Tensor:
+        """Runs the norm (once) and returns the normalised activations."""
+        if self._tensor is None:
+            if self.used:
+                raise RuntimeError("a pending norm was already consumed by a fused kernel")
+            self.used = True
+            self._tensor = self.norm.forward(self.stream, self.ctx)
+        return self._tensor
+
+    def fused(self) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+        """For a kernel that does the add and the norm itself: (residual in, delta or None,
+        residual out or None). The stream is updated as if the norm had run."""
+        if self.used:
+            raise RuntimeError("a pending norm was used twice")
+        self.used = True
+        st = self.stream
+        resid_in, delta = st.resid, st.delta
+        resid_out = None
+        if delta is not None:
+            resid_out = st.spare
+            st.resid, st.spare = resid_out, resid_in
+            st.delta = None
+        return resid_in, delta, resid_out
 
 
 # ---------------------------------------------------------------------------------------
@@ -194,7 +236,11 @@ class Part:
 class Norm(Part):
     """forward(stream, rows=None) -> normalised activations [n or len(rows), h]; adds the
     stream's pending delta first (and keeps the sum in the stream unless ``rows`` is given).
-    apply(x, out) normalises a plain tensor."""
+    apply(x, out) normalises a plain tensor. ``pending(stream, ctx)`` may return a PendingNorm
+    (see there) instead of running; the default runs at once."""
+
+    def pending(self, stream: HiddenStream, ctx):
+        return self.forward(stream, ctx)
 
     def forward(self, stream: HiddenStream, ctx, rows: Optional[torch.Tensor] = None,
                 tag: str = "normed") -> torch.Tensor:

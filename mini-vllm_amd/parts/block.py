@@ -29,7 +29,11 @@ class PreNormBlock(Block):
         self.ffn = ffn
 
     def forward(self, stream: HiddenStream, ctx, call: int) -> None:
-        h = self.norm_mixer.forward(stream, ctx)
+        # a part that starts with one matrix product over its input may get the norm unrun, to
+        # fuse it into that product
+        defer = getattr(self.mixer, "accepts_pending_norm", False)
+        h = self.norm_mixer.pending(stream, ctx) if defer else self.norm_mixer.forward(stream, ctx)
         stream.delta = self.mixer.forward(h, ctx, call)
-        h = self.norm_ffn.forward(stream, ctx)
+        defer = getattr(self.ffn, "accepts_pending_norm", False)
+        h = self.norm_ffn.pending(stream, ctx) if defer else self.norm_ffn.forward(stream, ctx)
         stream.delta = self.ffn.forward(h, ctx)

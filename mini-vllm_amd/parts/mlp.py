@@ -24,6 +24,7 @@ class SwiGLUSpec(PartSpec):
 @register_feed_forward(SwiGLUSpec.kind)
 class SwiGLU(FeedForward):
     spec_class = SwiGLUSpec
+    accepts_pending_norm = True      # the input is used by one packed product only
 
     @classmethod
     def tensors(cls, spec: SwiGLUSpec) -> Dict[str, TensorDecl]:
@@ -45,6 +46,8 @@ class SwiGLU(FeedForward):
         act = rt.workspace.get("ffn.act", (n, spec.intermediate_size), rt.dtype)
         if not ops.gemm_swiglu(x, self.w_gate_up, act):      # one pass over the weight for few rows
             gu = rt.workspace.get("ffn.gate_up", (n, 2 * spec.intermediate_size), rt.dtype)
+            if not isinstance(x, torch.Tensor):
+                x = x.materialize()
             ops.gemm(x, self.w_gate_up, gu)
             ops.swiglu(gu, act)
         y = rt.workspace.get("ffn.out", (n, spec.hidden_size), rt.dtype)

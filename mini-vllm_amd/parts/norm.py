@@ -13,7 +13,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import HiddenStream, Norm, PartSpec, Runtime, TensorDecl, register_norm
+from .base import HiddenStream, Norm, PartSpec, PendingNorm, Runtime, TensorDecl, register_norm
 
 
 @dataclass(frozen=True)
@@ -46,6 +46,12 @@ class RMSNorm(Norm):
         if rows is None:
             stream.delta = None
         return out
+
+    def pending(self, stream: HiddenStream, ctx):
+        """Deferred when the step is small enough for the fused add + norm + product kernel."""
+        if stream.spare is not None and self.rt.ops.can_fuse_norm(stream.resid.shape[0], self.spec.size):
+            return PendingNorm(self, stream, ctx)
+        return self.forward(stream, ctx)
 
     def apply(self, x: torch.Tensor, out: torch.Tensor) -> None:
         self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, out, unit_offset=self.spec.unit_offset)

@@ -483,3 +483,64 @@ def test_sampling_frequencies():
     freq = np.bincount(out.cpu().numpy(), minlength=V) / draws
     p = torch.softmax(logits[0].double() / T, dim=0).numpy()
     assert np.abs(freq - p).max() < 4 * np.sqrt(p.max() / draws)
+
+
+@pytest.mark.parametrize("M,N,K,swiglu", [(1, 4096, 1024, False), (8, 1000, 1024, False), (16, 96, 64, False),
+                                          (8, 3072, 1024, True), (3, 200, 128, True), (5, 333, 2048, False)])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_gemm_with_fused_add_and_norm(M, N, K, swiglu, with_delta):
+    """Residual add + RMSNorm + product (or gated pair) as one kernel, through the deferred-norm
+    interface of the parts."""
+    from minivllm_amd.parts import NORMS, HiddenStream, RMSNormSpec, Runtime, Workspace
+    from minivllm_amd.parts.base import PendingNorm
+    ops = ops_for(torch.bfloat16)
+    rt = Runtime(device=torch.device("cuda:0"), dtype=torch.bfloat16, ops=ops,
+                 workspace=Workspace(torch.device("cuda:0")), max_positions=16)
+    g = torch.Generator().manual_seed(44)
+    spec = RMSNormSpec(size=K, eps=1e-5)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16)
+    norm = NORMS.get(spec.kind)(spec, {"weight": dev(nw)}, rt)
+    resid = torch.randn(M, K, generator=g)
+    delta = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn((2 * N if swiglu else N), K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    bias = None if swiglu else torch.randn(N, generator=g).to(torch.bfloat16)
+    assert ops.can_fuse_norm(M, K)
+    stream = HiddenStream(dev(resid).clone(), torch.full((M, K), float("nan"), device="cuda"))
+    if with_delta:
+        stream.delta = dev(delta)
+    first = stream.resid
+    pending = norm.pending(stream, None)
+    assert isinstance(pending, PendingNorm)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    if swiglu:
+        assert ops.gemm_swiglu(pending, dev(w), out)
+    else:
+        ops.gemm(pending, dev(w), out, dev(bias))
+    x = resid.double() + (delta.double() if with_delta else 0)
+    a = (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double()).to(torch.bfloat16).double()
+    if swiglu:
+        gu = a @ w.double().T
+        want = torch.nn.functional.silu(gu[:, :N]) * gu[:, N:]
+    else:
+        want = a @ w.double().T + bias.double()
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[torch.bfloat16]
+    # the stream moved on as if the norm had run: the sum sits in the other buffer, nothing pending
+    assert stream.delta is None
+    if with_delta:
+        assert stream.resid is not first and stream.spare is first
+        assert rel_err(stream.resid.cpu().numpy(), x.float().numpy()) <= 1e-7
+        assert torch.equal(first.cpu(), resid)                   # the old sum was only read
+    else:
+        assert stream.resid is first
+
+
+def test_norm_is_not_deferred_for_many_rows():
+    from minivllm_amd.parts import NORMS, HiddenStream, RMSNormSpec, Runtime, Workspace
+    ops = ops_for(torch.bfloat16)
+    rt = Runtime(device=torch.device("cuda:0"), dtype=torch.bfloat16, ops=ops,
+                 workspace=Workspace(torch.device("cuda:0")), max_positions=16)
+    spec = RMSNormSpec(size=128, eps=1e-5)
+    norm = NORMS.get(spec.kind)(spec, {"weight": torch.ones(128, device="cuda")}, rt)
+    stream = HiddenStream(torch.randn(17, 128, device="cuda"), torch.empty(17, 128, device="cuda"))
+    assert isinstance(norm.pending(stream, None), torch.Tensor)
+    assert not ops_for(torch.float32).can_fuse_norm(4, 128)
