@@ -83,52 +83,93 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     if (NORM) {
         bf16* sA = reinterpret_cast<bf16*>(red + (size_t)(S - 1) * R * TM * 256);
         const int lds_ld = K + 8;  // row pitch in elements: the 16 rows an operand load touches fall into different banks
+        // A row is held in registers between the sum of squares and the scaling (up to 2048
+        // columns: 4 chunks of 8 per lane), so that the kernel waits for memory once.
+        constexpr int MAXJ = 4;
+        const int nj = (K + 511) / 512;
         for (int m = wave; m < M; m += S) {
             const float* xr = norm.resid_in + (size_t)m * K;
             const bf16* dr = norm.delta ? norm.delta + (size_t)m * K : nullptr;
+            float x[MAXJ][8];
             float ss = 0.f;
-            for (int c = lane * 8; c < K; c += 64 * 8) {
-                float x[8];
-                const float4 r0 = *reinterpret_cast<const float4*>(xr + c);
-                const float4 r1 = *reinterpret_cast<const float4*>(xr + c + 4);
-                x[0] = r0.x; x[1] = r0.y; x[2] = r0.z; x[3] = r0.w;
-                x[4] = r1.x; x[5] = r1.y; x[6] = r1.z; x[7] = r1.w;
-                if (dr) {
-                    Frag d;
-                    d.u = *reinterpret_cast<const uint4*>(dr + c);
+            if (nj <= MAXJ) {
+                float4 r0[MAXJ], r1[MAXJ];
+                Frag d[MAXJ];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) x[e] += (float)d.v[e];
+                for (int j = 0; j < MAXJ; ++j) {
+                    const int c = lane * 8 + 512 * j;
+                    if (j < nj && c < K) {
+                        r0[j] = *reinterpret_cast<const float4*>(xr + c);
+                        r1[j] = *reinterpret_cast<const float4*>(xr + c + 4);
+                        d[j].u = dr ? *reinterpret_cast<const uint4*>(dr + c) : uint4{0u, 0u, 0u, 0u};
+                    }
                 }
 #pragma unroll
-                for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+                for (int j = 0; j < MAXJ; ++j) {
+                    const int c = lane * 8 + 512 * j;
+                    if (j < nj && c < K) {
+                        x[j][0] = r0[j].x; x[j][1] = r0[j].y; x[j][2] = r0[j].z; x[j][3] = r0[j].w;
+                        x[j][4] = r1[j].x; x[j][5] = r1[j].y; x[j][6] = r1[j].z; x[j][7] = r1[j].w;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            x[j][e] += (float)d[j].v[e];      // a missing delta was loaded as zeros
+                            ss += x[j][e] * x[j][e];
+                        }
+                    }
+                }
+            } else {
+                for (int c = lane * 8; c < K; c += 512) {
+                    const float4 q0 = *reinterpret_cast<const float4*>(xr + c);
+                    const float4 q1 = *reinterpret_cast<const float4*>(xr + c + 4);
+                    float y[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+                    if (dr) {
+                        Frag dd;
+                        dd.u = *reinterpret_cast<const uint4*>(dr + c);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) y[e] += (float)dd.v[e];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ss += y[e] * y[e];
+                }
             }
             ss = wave_sum(ss);
             const float rinv = rsqrtf(ss / (float)K + norm.eps);
-            for (int c = lane * 8; c < K; c += 64 * 8) {
-                float x[8];
-                const float4 r0 = *reinterpret_cast<const float4*>(xr + c);
-                const float4 r1 = *reinterpret_cast<const float4*>(xr + c + 4);
-                x[0] = r0.x; x[1] = r0.y; x[2] = r0.z; x[3] = r0.w;
-                x[4] = r1.x; x[5] = r1.y; x[6] = r1.z; x[7] = r1.w;
-                if (dr) {
-                    Frag d;
-                    d.u = *reinterpret_cast<const uint4*>(dr + c);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) x[e] += (float)d.v[e];
-                    if (blockIdx.x == 0) {
-                        float* yr = norm.resid_out + (size_t)m * K + c;
-                        *reinterpret_cast<float4*>(yr) = float4{x[0], x[1], x[2], x[3]};
-                        *reinterpret_cast<float4*>(yr + 4) = float4{x[4], x[5], x[6], x[7]};
-                    }
+            // scales eight values, rounds them, and puts them where the MFMA operand loads expect
+            // them; workgroup 0 also stores the new residual sum
+            auto emit = [&](int c, const float* y) {
+                if (dr && blockIdx.x == 0) {
+                    float* yr = norm.resid_out + (size_t)m * K + c;
+                    *reinterpret_cast<float4*>(yr) = float4{y[0], y[1], y[2], y[3]};
+                    *reinterpret_cast<float4*>(yr + 4) = float4{y[4], y[5], y[6], y[7]};
                 }
                 Frag o;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     float wt = norm.weight.at(c + e);
                     if (norm.unit_offset) wt += 1.f;
-                    o.s[e] = f32_to_bf16_bits(x[e] * rinv * wt);
+                    o.s[e] = f32_to_bf16_bits(y[e] * rinv * wt);
                 }
                 *reinterpret_cast<uint4*>(sA + (size_t)m * lds_ld + c) = o.u;
+            };
+            if (nj <= MAXJ) {
+#pragma unroll
+                for (int j = 0; j < MAXJ; ++j) {
+                    const int c = lane * 8 + 512 * j;
+                    if (j < nj && c < K) emit(c, x[j]);
+                }
+            } else {
+                for (int c = lane * 8; c < K; c += 512) {
+                    const float4 q0 = *reinterpret_cast<const float4*>(xr + c);
+                    const float4 q1 = *reinterpret_cast<const float4*>(xr + c + 4);
+                    float y[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+                    if (dr) {
+                        Frag dd;
+                        dd.u = *reinterpret_cast<const uint4*>(dr + c);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) y[e] += (float)dd.v[e];
+                    }
+                    emit(c, y);
+                }
             }
         }
         __syncthreads();
