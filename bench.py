@@ -140,6 +140,8 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
+                    help="measure one phase alone (for profiling); the line then lacks the other's fields")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -156,22 +158,26 @@ def main() -> int:
     nums = model_numbers(shape, layers)
     item = 2 if args.dtype == "bfloat16" else 4
 
-    prefill_s = measure_prefill(llm, cfg.vocab_size, args.prefill_tokens, repeats=3, seed=args.seed)
-    T = args.prefill_tokens
-    attn_flops = layers * 2 * cfg.num_attention_heads * cfg.head_dim * T * T       # causal half of 4 H D T^2
-    prefill_flops = 2 * T * nums["matrix_params"] + attn_flops + 2 * cfg.vocab_size * cfg.hidden_size
-    prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
-               "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    prefill = None
+    if args.only in ("all", "prefill"):
+        prefill_s = measure_prefill(llm, cfg.vocab_size, args.prefill_tokens, repeats=3, seed=args.seed)
+        T = args.prefill_tokens
+        attn_flops = layers * 2 * cfg.num_attention_heads * cfg.head_dim * T * T   # causal half of 4 H D T^2
+        prefill_flops = 2 * T * nums["matrix_params"] + attn_flops + 2 * cfg.vocab_size * cfg.hidden_size
+        prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
 
-    tok_s, ms_step, mean_ctx = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len, args.steps,
-                                              args.warmup, args.seed)
-    step_bytes = nums["step_params"] * item + args.batch * mean_ctx * nums["kv_bytes_per_token"] * item
-    achieved = step_bytes / (ms_step * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    tok_s = ms_step = roofline = None
+    if args.only in ("all", "decode"):
+        tok_s, ms_step, mean_ctx = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len, args.steps,
+                                                  args.warmup, args.seed)
+        step_bytes = nums["step_params"] * item + args.batch * mean_ctx * nums["kv_bytes_per_token"] * item
+        achieved = step_bytes / (ms_step * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBS, 4)}
 
     points = {}
-    if not args.no_points:
+    if not args.no_points and args.only == "all":
         for b, key in ((1, "decode_b1"), (64, "decode_b64")):
             n = min(args.steps, 128)
             v, _, _ = measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8), args.seed + b)
@@ -184,8 +190,8 @@ def main() -> int:
               "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
               "parallelism": "single-gpu"}
     line = {"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
-            "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms_step, 4) if ms_step is not None else None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic", "config": config,
             "prefill": prefill, "roofline": roofline, "points": points}
     print(json.dumps(line))
