@@ -22,7 +22,7 @@
 // Layouts: K[page][kv_head][slot][d], V[page][kv_head][d][slot]; the page size is a multiple of
 // 16. Keys outside the range (above the query's position, or more than `window` below it) get
 // probability zero; value slots that were never written are read as zero.
-#include "common.h"
+#include "dispatch.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
@@ -55,14 +55,86 @@ __device__ __forceinline__ int wave_min_i(int v) {
     return v;
 }
 
-template <int D, int W>
+// What the FUSED variant does itself instead of reading finished queries and a finished cache:
+// the rows of the step's [q | k | v] product are normalised per head (RMSNorm, when weights are
+// given) and rotated (half-split pairs, table row = cat(cos, sin) of the position, when a table
+// is given) on the way into the registers; with `store` the new key and value also go to their
+// page slot, and the wave that meets that slot among its keys uses the registers, not the page.
+struct FusedInput {
+    const bf16* qkv;        // [tokens, stride]
+    long stride;
+    int q_off, k_off, v_off;
+    WeightPtr qw, kw;       // [D] each
+    int has_norm;
+    float eps;
+    int unit_offset;
+    const float* table;     // [positions, D] or null
+    int store;
+    const int* token_seq;   // rows that belong to no sequence (< 0) are left alone
+};
+
+// A head's raw elements (DS groups of eight a lane, d = 32 s + 8 g + e; the four lane groups g
+// hold a head between them) are normalised (weights w[D], or null), rotated (cs = cat(cos, sin) of
+// the position, or null; element d pairs with d + D/2: the same lane, DS/2 groups further) and
+// rounded to the operand type. w and cs lie in LDS.
+template <int DS>
+__device__ __forceinline__ void norm_rotate(const Frag (&raw)[DS], int g, const float* w, float eps, const float* cs,
+                                            int D, Frag (&dst)[DS]) {
+    float x[DS][8];
+#pragma unroll
+    for (int s = 0; s < DS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[s][e] = (float)raw[s].v[e];
+    if (w != nullptr) {
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < DS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += x[s][e] * x[s][e];
+        ss += __shfl_xor(ss, 16, MV_WAVE);
+        ss += __shfl_xor(ss, 32, MV_WAVE);
+        const float rinv = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int s = 0; s < DS; ++s) {
+            const float4 w0 = *reinterpret_cast<const float4*>(w + 32 * s + 8 * g);
+            const float4 w1 = *reinterpret_cast<const float4*>(w + 32 * s + 8 * g + 4);
+            const float wt[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[s][e] = x[s][e] * rinv * wt[e];
+        }
+    }
+    if (cs != nullptr) {
+        constexpr int HS = DS / 2;
+#pragma unroll
+        for (int s = 0; s < HS; ++s) {
+            const float4 c0 = *reinterpret_cast<const float4*>(cs + 32 * s + 8 * g);
+            const float4 c1 = *reinterpret_cast<const float4*>(cs + 32 * s + 8 * g + 4);
+            const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2 + 32 * s + 8 * g);
+            const float4 s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 32 * s + 8 * g + 4);
+            const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float a = x[s][e], b = x[s + HS][e];
+                x[s][e] = a * c[e] - b * sn[e];
+                x[s + HS][e] = b * c[e] + a * sn[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < DS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[s].s[e] = f32_to_bf16_bits(x[s][e]);
+}
+
+template <int D, int W, bool FUSED>
 __global__ void __launch_bounds__(64 * W)
 attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                       const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                       const int* __restrict__ block_table, int bt_width, int page_size,
                       const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
                       int H, int Hkv, float scale, int window, float* __restrict__ partials,
-                      int nsplit) {
+                      int nsplit, FusedInput fz) {
     constexpr int DS = D / 32;
     constexpr int DT = D / 16;
     constexpr int NT = 1;      // column tiles of a wave (the group's heads fit one tile)
@@ -83,6 +155,8 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         t0 = cu_seqlens[seq];
         nt = cu_seqlens[seq + 1] - t0;
         if (nt > tpu) nt = tpu;
+        if (FUSED && nt > 1) nt = 1;   // decode steps: one token a sequence
+        if (FUSED && nt == 1 && fz.token_seq[t0] < 0) nt = 0;
         sh_unit[0] = seq;
         sh_unit[1] = t0;
         sh_unit[2] = nt;
@@ -110,7 +184,10 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
             hi_w = col_pos[ct] > hi_w ? col_pos[ct] : hi_w;
             lo_w = col_lo[ct] < lo_w ? col_lo[ct] : lo_w;
         }
-        const bf16* qrow = q + (size_t)col_tok[ct] * q_stride + (size_t)col_head[ct] * D + 8 * g;
+        // the query rows: finished, or (FUSED) raw, to be normalised and rotated further down while
+        // the first keys are on their way
+        const bf16* qrow = FUSED ? fz.qkv + (size_t)col_tok[ct] * fz.stride + fz.q_off + (size_t)col_head[ct] * D + 8 * g
+                                 : q + (size_t)col_tok[ct] * q_stride + (size_t)col_head[ct] * D + 8 * g;
 #pragma unroll
         for (int s = 0; s < DS; ++s)
             qop[ct][s].u = col_ok[ct] ? *reinterpret_cast<const uint4*>(qrow + 32 * s) : uint4{0u, 0u, 0u, 0u};
@@ -140,6 +217,36 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         b_step = W;
     }
     const float sc_mul = scale * LOG2E;
+
+    // (FUSED) the norm weights and the table row of the position go to LDS with the page ids; the
+    // wave that will meet the newest position among its keys asks for the raw key and value now
+    __shared__ __attribute__((aligned(16))) float sh_const[FUSED ? 3 : 1][FUSED ? D : 1];
+    const int b_new = hi_w >= 0 ? hi_w / 32 : -1;
+    const bool owns_new = FUSED && fz.store && b_new >= b_begin && b_new < b_end && (b_new - b_begin) % b_step == 0;
+    Frag knew[DS], kraw[DS];
+    uint16_t vnew[DT];
+    if (FUSED) {
+        for (int d = threadIdx.x; d < D; d += blockDim.x) {
+            if (fz.has_norm) {
+                sh_const[0][d] = fz.qw.at(d) + (fz.unit_offset ? 1.f : 0.f);
+                if (fz.kw.p != nullptr) sh_const[1][d] = fz.kw.at(d) + (fz.unit_offset ? 1.f : 0.f);
+            }
+            if (fz.table != nullptr) sh_const[2][d] = fz.table[(size_t)(hi_w >= 0 ? hi_w : 0) * D + d];
+        }
+#pragma unroll
+        for (int s = 0; s < DS; ++s) knew[s].u = kraw[s].u = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vnew[dt] = 0;
+        if (owns_new) {
+            const bf16* row = fz.qkv + (size_t)t0 * fz.stride;
+            const bf16* krow = row + fz.k_off + (size_t)kvh * D + 8 * g;
+#pragma unroll
+            for (int s = 0; s < DS; ++s) kraw[s].u = *reinterpret_cast<const uint4*>(krow + 32 * s);
+            const uint16_t* vrow = reinterpret_cast<const uint16_t*>(row + fz.v_off + (size_t)kvh * D);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vnew[dt] = vrow[16 * dt + i];
+        }
+    }
 
     // The page ids of this workgroup's key range go to LDS first (one round trip instead of one
     // per block); K and V operands are fetched one block ahead of their use.
@@ -192,6 +299,21 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     };
     auto compute = [&](int b, Operands& op) {
         const int base = 32 * b;
+        if (FUSED && owns_new && b == b_new) {   // the newest key and value come from the registers
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (base + 16 * t + i == hi_w) {
+#pragma unroll
+                    for (int s = 0; s < DS; ++s) op.k[t][s] = knew[s];
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (base + 16 * t + 4 * g + r == hi_w) {
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) op.v[dt].s[t * 4 + r] = vnew[dt];
+                    }
+            }
+        }
         // scores^T for two tiles of 16 keys
         float p[2][4];
 #pragma unroll
@@ -251,6 +373,28 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
 
     Operands oa, ob;
     fetch(b_begin, oa);
+    if (FUSED) {   // while those loads are in flight
+        const float* cs = fz.table != nullptr ? sh_const[2] : nullptr;
+        norm_rotate<DS>(qop[0], g, fz.has_norm ? sh_const[0] : nullptr, fz.eps, cs, D, qop[0]);
+        if (owns_new) {
+            norm_rotate<DS>(kraw, g, fz.has_norm ? sh_const[1] : nullptr, fz.eps, cs, D, knew);
+            const int page = page_of(hi_w / page_size);
+            if (page >= 0) {
+                const int slot = hi_w % page_size;
+                const size_t head = (size_t)page * Hkv + kvh;
+                if (i == 0) {
+                    bf16* kdst = const_cast<bf16*>(k_pages) + ((head * page_size + slot) * D + 8 * g);
+#pragma unroll
+                    for (int s = 0; s < DS; ++s) *reinterpret_cast<uint4*>(kdst + 32 * s) = knew[s].u;
+                }
+                if (g == 0) {
+                    uint16_t* vdst = reinterpret_cast<uint16_t*>(const_cast<bf16*>(v_pages)) + (head * D + i) * page_size + slot;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) vdst[(size_t)16 * dt * page_size] = vnew[dt];
+                }
+            }
+        }
+    }
     for (int b = b_begin; b < b_end; b += 2 * b_step) {
         fetch(b + b_step, ob);
         compute(b, oa);
@@ -366,14 +510,14 @@ __global__ void attention_merge_kernel(const float* __restrict__ partials, bf16*
     }
 }
 
-template <int D, int W>
+template <int D, int W, bool FUSED>
 static void launch_decode(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                           int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv,
-                          float scale, int window, float* partials, int nsplit) {
-    hipLaunchKernelGGL((attention_decode_kernel<D, W>), grid, dim3(64 * W), 0, stream, (const bf16*)q, q_stride,
+                          float scale, int window, float* partials, int nsplit, const FusedInput& fz) {
+    hipLaunchKernelGGL((attention_decode_kernel<D, W, FUSED>), grid, dim3(64 * W), 0, stream, (const bf16*)q, q_stride,
                        (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,
-                       page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit);
+                       page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit, fz);
 }
 
 static int check_common(const char* what, long q_stride, long out_stride, int page_size, int bt_width, int H, int Hkv,
@@ -388,14 +532,11 @@ static int check_common(const char* what, long q_stride, long out_stride, int pa
     return 0;
 }
 
-// Decode steps: every sequence brings one token. grid = (sequences, kv heads, nsplit); `waves` (4
-// or 8) per workgroup. partials: float [n_seqs * H * nsplit * (D + 2)], needed when nsplit > 1.
-extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
-                                   const void* v_pages, const int* block_table, int bt_width, int page_size,
-                                   const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
-                                   float scale, int window, float* partials, int nsplit, int waves,
-                                   const int* token_seq, hipStream_t stream) {
-    if (int rc = check_common("attention_decode", q_stride, out_stride, page_size, bt_width, H, Hkv, D)) return rc;
+static int decode_common(bool fused, const FusedInput& fz, const void* q, long q_stride, void* out, long out_stride,
+                         const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
+                         int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
+                         float scale, int window, float* partials, int nsplit, int waves, const int* token_seq,
+                         hipStream_t stream) {
     MV_REQUIRE(H / Hkv <= 16, "attention_decode: %d query heads per kv head exceed 16", H / Hkv);
     MV_REQUIRE(nsplit >= 1 && nsplit <= AF_MAX_SPLITS && (nsplit == 1 || partials != nullptr),
                "attention_decode: bad split count %d or missing work area", nsplit);
@@ -403,13 +544,19 @@ extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long
     if (n_seqs <= 0) return 0;
     dim3 grid(n_seqs, Hkv, nsplit);
     float* part = nsplit > 1 ? partials : nullptr;
-#define AF_LAUNCH(DD, WW)                                                                                         \
-    launch_decode<DD, WW>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,      \
-                          page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, part, nsplit)
-    if (D == 128 && waves == 8) AF_LAUNCH(128, 8);
-    else if (D == 128) AF_LAUNCH(128, 4);
-    else if (waves == 8) AF_LAUNCH(64, 8);
-    else AF_LAUNCH(64, 4);
+#define AF_LAUNCH(DD, WW, FF)                                                                                     \
+    launch_decode<DD, WW, FF>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,  \
+                              page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, part, nsplit, fz)
+    if (fused) {
+        MV_REQUIRE(waves == 4, "attention_decode_fused: %d waves per workgroup (4 only)", waves);
+        if (D == 128) AF_LAUNCH(128, 4, true);
+        else AF_LAUNCH(64, 4, true);
+    } else {
+        if (D == 128 && waves == 8) AF_LAUNCH(128, 8, false);
+        else if (D == 128) AF_LAUNCH(128, 4, false);
+        else if (waves == 8) AF_LAUNCH(64, 8, false);
+        else AF_LAUNCH(64, 4, false);
+    }
 #undef AF_LAUNCH
     if (int rc = mv_check_launch("attention_decode")) return rc;
     if (nsplit > 1) {
@@ -418,4 +565,49 @@ extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long
         return mv_check_launch("attention_merge");
     }
     return 0;
+}
+
+// Decode steps: every sequence brings one token. grid = (sequences, kv heads, nsplit); `waves` (4
+// or 8) per workgroup. partials: float [n_seqs * H * nsplit * (D + 2)], needed when nsplit > 1.
+extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
+                                   const void* v_pages, const int* block_table, int bt_width, int page_size,
+                                   const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
+                                   float scale, int window, float* partials, int nsplit, int waves,
+                                   const int* token_seq, hipStream_t stream) {
+    if (int rc = check_common("attention_decode", q_stride, out_stride, page_size, bt_width, H, Hkv, D)) return rc;
+    return decode_common(false, FusedInput{}, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,
+                         page_size, positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, partials, nsplit, waves,
+                         token_seq, stream);
+}
+
+// The same for a decode step whose queries, keys and values are still the raw rows of the
+// [q | k | v] product (one token a sequence; row t of qkv belongs to sequence t): per-head RMSNorm
+// (q_weight / k_weight, or null for none) and rotation by the table row of the position
+// (half-split pairs over the whole head, or null for none) happen on the way into the kernel;
+// with store_kv the new key and value are written to their page slot as well.
+extern "C" int mv_attention_decode_fused(const void* qkv, long qkv_stride, int q_off, int k_off, int v_off, void* out,
+                                         long out_stride, void* k_pages, void* v_pages, const int* block_table,
+                                         int bt_width, int page_size, const int* positions, const int* cu_seqlens,
+                                         int n_seqs, int H, int Hkv, int D, float scale, int window,
+                                         const void* q_weight, const void* k_weight, int weight_dtype, float eps,
+                                         int unit_offset, const float* table, int store_kv, float* partials,
+                                         int nsplit, int waves, const int* token_seq, hipStream_t stream) {
+    if (int rc = check_common("attention_decode_fused", qkv_stride, out_stride, page_size, bt_width, H, Hkv, D))
+        return rc;
+    MV_REQUIRE(qkv != nullptr && ((uintptr_t)qkv % 16) == 0 && q_off % 8 == 0 && k_off % 8 == 0 && v_off >= 0,
+               "attention_decode_fused: the qkv rows must be 16-byte aligned (offsets %d / %d / %d)", q_off, k_off, v_off);
+    MV_REQUIRE(qkv_stride >= (long)q_off + (long)H * D, "attention_decode_fused: row stride %ld too small", qkv_stride);
+    MV_REQUIRE(token_seq != nullptr, "attention_decode_fused: token_seq is missing");
+    MV_REQUIRE(!store_kv || qkv_stride >= (long)(k_off > v_off ? k_off : v_off) + (long)Hkv * D,
+               "attention_decode_fused: row stride %ld does not hold the key and value heads", qkv_stride);
+    const int has_norm = q_weight != nullptr;
+    MV_REQUIRE(!has_norm || ((k_weight != nullptr || !store_kv) && eps > 0.f && mv_valid_dtype(weight_dtype) &&
+                             ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0),
+               "attention_decode_fused: bad norm weights (missing, unknown type or not 16-byte aligned) or eps");
+    MV_REQUIRE(table == nullptr || ((uintptr_t)table % 16) == 0, "attention_decode_fused: the table is not 16-byte aligned");
+    FusedInput fz{(const bf16*)qkv, qkv_stride, q_off, k_off, v_off, WeightPtr{q_weight, weight_dtype},
+                  WeightPtr{k_weight, weight_dtype}, has_norm, eps, unit_offset, table, store_kv ? 1 : 0, token_seq};
+    return decode_common(true, fz, nullptr, 0, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size,
+                         positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, partials, nsplit, waves, token_seq,
+                         stream);
 }

@@ -45,6 +45,23 @@ struct WeightPtr {
         if (dtype == MV_F32) return ((const float*)p)[i];
         return to_f(((const bf16*)p)[i]);
     }
+    // eight consecutive elements from i (i a multiple of 8, the tensor 16-byte aligned)
+    __device__ __forceinline__ void at8(size_t i, float (&out)[8]) const {
+        if (dtype == MV_F32) {
+            const float4 a = *reinterpret_cast<const float4*>((const float*)p + i);
+            const float4 b = *reinterpret_cast<const float4*>((const float*)p + i + 4);
+            out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+            out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+        } else {
+            const uint4 u = *reinterpret_cast<const uint4*>((const bf16*)p + i);
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                out[2 * e] = __uint_as_float(w[e] << 16);
+                out[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+            }
+        }
+    }
 };
 
 // ---------------------------------------------------------------------------------------

@@ -24,6 +24,10 @@ union Frag {
 };
 
 #define SK_MAX_WAVES 8
+#ifndef SK_STAGE_FRAGS
+#define SK_STAGE_FRAGS 8    // 16-byte operand loads per lane in one register stage of the main loop
+#endif
+#define SK_NORM_CHUNKS 4   // chunks of 512 columns a wave holds in the fused norm's prologue
 
 template <typename TC> __device__ __forceinline__ void store_c(TC* p, float v);
 template <> __device__ __forceinline__ void store_c<float>(float* p, float v) { *p = v; }
@@ -83,94 +87,79 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     if (NORM) {
         bf16* sA = reinterpret_cast<bf16*>(red + (size_t)(S - 1) * R * TM * 256);
         const int lds_ld = K + 8;  // row pitch in elements: the 16 rows an operand load touches fall into different banks
-        // A row is held in registers between the sum of squares and the scaling (up to 2048
-        // columns: 4 chunks of 8 per lane), so that the kernel waits for memory once.
-        constexpr int MAXJ = 4;
-        const int nj = (K + 511) / 512;
-        for (int m = wave; m < M; m += S) {
-            const float* xr = norm.resid_in + (size_t)m * K;
-            const bf16* dr = norm.delta ? norm.delta + (size_t)m * K : nullptr;
-            float x[MAXJ][8];
-            float ss = 0.f;
-            if (nj <= MAXJ) {
-                float4 r0[MAXJ], r1[MAXJ];
-                Frag d[MAXJ];
+        // The rows are cut into chunks of 512 columns (8 per lane); wave w takes the chunks
+        // w * cpw .. (w + 1) * cpw - 1 and holds them in registers between the sum of squares and
+        // the scaling, so the kernel waits for memory once. Where a wave's chunks are whole rows
+        // the sums stay in the wave; otherwise they are exchanged through LDS. The launcher takes
+        // only shapes with at most SK_NORM_CHUNKS chunks a wave.
+        float* part = reinterpret_cast<float*>(sA + (size_t)M * lds_ld);   // [chunks] sums of squares
+        const int cpr = (K + 511) / 512;       // chunks per row
+        const int nq = M * cpr;
+        const int cpw = (nq + S - 1) / S;      // chunks per wave
+        const bool whole = cpw % cpr == 0;
+        float x[SK_NORM_CHUNKS][8], ss[SK_NORM_CHUNKS];
+        {
+            float4 r0[SK_NORM_CHUNKS], r1[SK_NORM_CHUNKS];
+            Frag d[SK_NORM_CHUNKS];
 #pragma unroll
-                for (int j = 0; j < MAXJ; ++j) {
-                    const int c = lane * 8 + 512 * j;
-                    if (j < nj && c < K) {
-                        r0[j] = *reinterpret_cast<const float4*>(xr + c);
-                        r1[j] = *reinterpret_cast<const float4*>(xr + c + 4);
-                        d[j].u = dr ? *reinterpret_cast<const uint4*>(dr + c) : uint4{0u, 0u, 0u, 0u};
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < MAXJ; ++j) {
-                    const int c = lane * 8 + 512 * j;
-                    if (j < nj && c < K) {
-                        x[j][0] = r0[j].x; x[j][1] = r0[j].y; x[j][2] = r0[j].z; x[j][3] = r0[j].w;
-                        x[j][4] = r1[j].x; x[j][5] = r1[j].y; x[j][6] = r1[j].z; x[j][7] = r1[j].w;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            x[j][e] += (float)d[j].v[e];      // a missing delta was loaded as zeros
-                            ss += x[j][e] * x[j][e];
-                        }
-                    }
-                }
-            } else {
-                for (int c = lane * 8; c < K; c += 512) {
-                    const float4 q0 = *reinterpret_cast<const float4*>(xr + c);
-                    const float4 q1 = *reinterpret_cast<const float4*>(xr + c + 4);
-                    float y[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-                    if (dr) {
-                        Frag dd;
-                        dd.u = *reinterpret_cast<const uint4*>(dr + c);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) y[e] += (float)dd.v[e];
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) ss += y[e] * y[e];
+            for (int qi = 0; qi < SK_NORM_CHUNKS; ++qi) {
+                const int q = wave * cpw + qi;
+                const int m = q / cpr, c = (q % cpr) * 512 + lane * 8;
+                r0[qi] = r1[qi] = float4{0.f, 0.f, 0.f, 0.f};
+                d[qi].u = uint4{0u, 0u, 0u, 0u};
+                if (qi < cpw && q < nq && c < K) {
+                    const float* xr = norm.resid_in + (size_t)m * K + c;
+                    r0[qi] = *reinterpret_cast<const float4*>(xr);
+                    r1[qi] = *reinterpret_cast<const float4*>(xr + 4);
+                    if (norm.delta) d[qi].u = *reinterpret_cast<const uint4*>(norm.delta + (size_t)m * K + c);
                 }
             }
-            ss = wave_sum(ss);
-            const float rinv = rsqrtf(ss / (float)K + norm.eps);
-            // scales eight values, rounds them, and puts them where the MFMA operand loads expect
-            // them; workgroup 0 also stores the new residual sum
-            auto emit = [&](int c, const float* y) {
-                if (dr && blockIdx.x == 0) {
-                    float* yr = norm.resid_out + (size_t)m * K + c;
-                    *reinterpret_cast<float4*>(yr) = float4{y[0], y[1], y[2], y[3]};
-                    *reinterpret_cast<float4*>(yr + 4) = float4{y[4], y[5], y[6], y[7]};
-                }
-                Frag o;
+#pragma unroll
+            for (int qi = 0; qi < SK_NORM_CHUNKS; ++qi) {
+                x[qi][0] = r0[qi].x; x[qi][1] = r0[qi].y; x[qi][2] = r0[qi].z; x[qi][3] = r0[qi].w;
+                x[qi][4] = r1[qi].x; x[qi][5] = r1[qi].y; x[qi][6] = r1[qi].z; x[qi][7] = r1[qi].w;
+                float t = 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    float wt = norm.weight.at(c + e);
-                    if (norm.unit_offset) wt += 1.f;
-                    o.s[e] = f32_to_bf16_bits(y[e] * rinv * wt);
+                    x[qi][e] += (float)d[qi].v[e];      // a missing delta was loaded as zeros
+                    t += x[qi][e] * x[qi][e];
                 }
-                *reinterpret_cast<uint4*>(sA + (size_t)m * lds_ld + c) = o.u;
-            };
-            if (nj <= MAXJ) {
-#pragma unroll
-                for (int j = 0; j < MAXJ; ++j) {
-                    const int c = lane * 8 + 512 * j;
-                    if (j < nj && c < K) emit(c, x[j]);
-                }
-            } else {
-                for (int c = lane * 8; c < K; c += 512) {
-                    const float4 q0 = *reinterpret_cast<const float4*>(xr + c);
-                    const float4 q1 = *reinterpret_cast<const float4*>(xr + c + 4);
-                    float y[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-                    if (dr) {
-                        Frag dd;
-                        dd.u = *reinterpret_cast<const uint4*>(dr + c);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) y[e] += (float)dd.v[e];
-                    }
-                    emit(c, y);
-                }
+                ss[qi] = wave_sum(t);
             }
+        }
+        if (!whole) {
+#pragma unroll
+            for (int qi = 0; qi < SK_NORM_CHUNKS; ++qi) {
+                const int q = wave * cpw + qi;
+                if (qi < cpw && q < nq && lane == 0) part[q] = ss[qi];
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int qi = 0; qi < SK_NORM_CHUNKS; ++qi) {
+            const int q = wave * cpw + qi;
+            const int m = q / cpr, c = (q % cpr) * 512 + lane * 8;
+            if (qi >= cpw || q >= nq || c >= K) continue;
+            float tot = 0.f;
+            if (whole) {
+#pragma unroll
+                for (int qj = 0; qj < SK_NORM_CHUNKS; ++qj)
+                    if (qj < cpw && qj / cpr == qi / cpr) tot += ss[qj];   // the chunks of this row, in order
+            } else {
+                for (int j = 0; j < cpr; ++j) tot += part[m * cpr + j];    // the same order in every workgroup
+            }
+            const float rinv = rsqrtf(tot / (float)K + norm.eps);
+            if (norm.delta && blockIdx.x == 0) {   // workgroup 0 stores the new residual sum
+                float* yr = norm.resid_out + (size_t)m * K + c;
+                *reinterpret_cast<float4*>(yr) = float4{x[qi][0], x[qi][1], x[qi][2], x[qi][3]};
+                *reinterpret_cast<float4*>(yr + 4) = float4{x[qi][4], x[qi][5], x[qi][6], x[qi][7]};
+            }
+            float wt[8];
+            norm.weight.at8(c, wt);
+            Frag o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o.s[e] = f32_to_bf16_bits(x[qi][e] * rinv * (norm.unit_offset ? wt[e] + 1.f : wt[e]));
+            *reinterpret_cast<uint4*>(sA + (size_t)m * lds_ld + c) = o.u;
         }
         __syncthreads();
 #pragma unroll
@@ -194,26 +183,44 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 #pragma unroll
         for (int t = 0; t < TM; ++t) acc[r][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    // four k-steps per iteration: all loads are issued before the first MFMA needs its operands
-    constexpr int U = 4;
-    int ks = ks0;
-    for (; ks + U <= ks1; ks += U) {
-        Frag a[U][TM], w[U][R];
+    // Two register stages of U k-steps each: while the MFMAs of one stage run, the loads of the
+    // next are in flight, so a wave always has a stage's worth of weight bytes on the way.
+    constexpr int U = SK_STAGE_FRAGS / (R + TM) >= 8 ? 8 : (SK_STAGE_FRAGS / (R + TM) >= 4 ? 4 : (SK_STAGE_FRAGS / (R + TM) >= 2 ? 2 : 1));
+    struct Stage {
+        Frag w[U][R], a[U][TM];
+    };
+    auto fetch = [&](Stage& st, int k0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) w[u][r].u = wrow[r][(size_t)(ks + u) * 4];
+            for (int r = 0; r < R; ++r) st.w[u][r].u = wrow[r][(size_t)(k0 + u) * 4];
 #pragma unroll
             for (int t = 0; t < TM; ++t)
-                a[u][t].u = avalid[t] ? arow[t][(size_t)(ks + u) * 4] : uint4{0u, 0u, 0u, 0u};
+                st.a[u][t].u = avalid[t] ? arow[t][(size_t)(k0 + u) * 4] : uint4{0u, 0u, 0u, 0u};
         }
+    };
+    auto multiply = [&](const Stage& st) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int t = 0; t < TM; ++t)
-                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][r].v, a[u][t].v, acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.w[u][r].v, st.a[u][t].v, acc[r][t], 0, 0, 0);
+    };
+    const int nfull = (ks1 - ks0) / U;
+    int ks = ks0 + nfull * U;
+    if (nfull > 0) {
+        Stage s0, s1;
+        fetch(s0, ks0);
+        int it = 0;
+        for (; it + 2 <= nfull; it += 2) {
+            fetch(s1, ks0 + (it + 1) * U);
+            multiply(s0);
+            if (it + 2 < nfull) fetch(s0, ks0 + (it + 2) * U);
+            multiply(s1);
+        }
+        if (it < nfull) multiply(s0);
     }
     for (; ks < ks1; ++ks) {
         Frag a[TM], w[R];
@@ -284,7 +291,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 
 static size_t skinny_lds_bytes(int S, int R, int TM, bool with_norm, int M, int K) {
     size_t lds = (size_t)(S - 1) * R * TM * 256 * sizeof(float);
-    if (with_norm) lds += (size_t)M * (K + 8) * sizeof(uint16_t);
+    if (with_norm) lds += (size_t)M * (K + 8) * sizeof(uint16_t) + (size_t)M * ((K + 511) / 512) * sizeof(float);
     return lds;
 }
 
@@ -384,16 +391,20 @@ extern "C" int mv_gemm_skinny_norm(const float* resid_in, const void* delta, flo
                                    void* C, long ldc, int c_dtype, int M, int N, int K, int swiglu,
                                    hipStream_t stream) {
     MV_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny_norm: bad sizes M=%d N=%d K=%d", M, N, K);
-    MV_REQUIRE(mv_valid_dtype(norm_weight_dtype) && norm_weight != nullptr, "gemm_skinny_norm: bad norm weight");
+    MV_REQUIRE(mv_valid_dtype(norm_weight_dtype) && norm_weight != nullptr && ((uintptr_t)norm_weight % 16) == 0,
+               "gemm_skinny_norm: the norm weight is missing, of an unknown type or not 16-byte aligned");
     MV_REQUIRE(delta == nullptr || (resid_out != nullptr && resid_out != resid_in),
                "gemm_skinny_norm: the updated residual needs a buffer of its own");
     MV_REQUIRE(eps > 0.f, "gemm_skinny_norm: eps must be positive");
     MV_REQUIRE(ldc >= N, "gemm_skinny_norm: ldc=%ld smaller than N=%d", ldc, N);
     MV_REQUIRE(c_dtype == MV_BF16 || (c_dtype == MV_F32 && !swiglu), "gemm_skinny_norm: bad output dtype %d", c_dtype);
     if (M == 0) return 0;
-    const int S = pick_waves(K);
+    // enough waves to hold the rows in registers during the prologue, also where K alone asks for fewer
+    const int chunks = M * ((K + 511) / 512);
+    int S = pick_waves(K);
+    if (S * SK_NORM_CHUNKS < chunks) S = (chunks + SK_NORM_CHUNKS - 1) / SK_NORM_CHUNKS;
     const int R = swiglu ? 2 : 1;
-    if (M > 16 || K % 64 != 0 || skinny_lds_bytes(S, R, 1, true, M, K) > 60 * 1024) {
+    if (M > 16 || K % 64 != 0 || S > SK_MAX_WAVES || skinny_lds_bytes(S, R, 1, true, M, K) > 60 * 1024) {
         mv_fail("gemm_skinny_norm: M=%d K=%d is not taken by the fused kernel", M, K);
         return 2;
     }

@@ -403,6 +403,8 @@ class Executor:
         arr[o:o + size] = -1
         o, size = off["logit_rows"]
         arr[o:o + size] = -1
+        o, size = off["cu_seqlens"]
+        arr[o:o + size] = 0                        # no sequence has a token
         meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
         self._upload(arr, dst=meta)
         return self._context(meta, off, facts, dummy)

@@ -19,6 +19,8 @@ _NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
 SKINNY_MAX_M = 64
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
+# the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
+FUSED_NORM_MAX_CHUNKS = 32
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
 # from this many tokens on, value rows are written to their pages by a kernel of their own
@@ -279,7 +281,8 @@ class Ops:
     def can_fuse_norm(self, rows: int, width: int) -> bool:
         """Whether a norm over ``rows`` x ``width`` may be deferred into the next product."""
         return (self.use_fast_kernels and self.lib.has("mv_gemm_skinny_norm") and 0 < rows <= FUSED_NORM_MAX_M
-                and width % 64 == 0 and rows * (width + 8) * 2 <= 44 * 1024)
+                and width % 64 == 0 and rows * ((width + 511) // 512) <= FUSED_NORM_MAX_CHUNKS
+                and rows * (width + 8) * 2 <= 44 * 1024)
 
     def _gemm_fused_norm(self, pending, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor],
                          swiglu: bool) -> bool:
@@ -290,6 +293,7 @@ class Ops:
         weight = getattr(norm, "weight", None)
         spec = getattr(norm, "spec", None)
         if (weight is None or spec is None or getattr(spec, "kind", "") != "rmsnorm" or not self.can_fuse_norm(M, K)
+                or weight.data_ptr() % 16
                 or w.dtype != torch.bfloat16 or not w.is_contiguous() or w.shape[1] != K
                 or out.stride(1) != 1 or (swiglu and (w.shape[0] % 2 or out.dtype != torch.bfloat16))):
             return False
@@ -374,6 +378,77 @@ class Ops:
                       positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim,
                       float(scale), w, self.code, self._stream())
 
+    def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int):
+        """How many workgroups share a sequence's keys in a decode step, and their work area.
+
+        The keys are split until about 256 workgroups are in flight, but never below 128 keys per
+        split (measured on MI355X with 8 kv heads: batch 1 is fastest at 8 to 16 splits, batch 8 at
+        4, batch 64 without a split). The count is a property of the plan (a captured graph keeps
+        it); each split takes its share of the keys a sequence actually has."""
+        ctx = max(1, plan.max_context_len)
+        nsplit = max(1, min(256 // max(1, n_seqs * Hkv), max(1, ctx // 128), 64))
+        partials = None
+        if nsplit > 1:
+            rows = max(n_seqs * nsplit, 2048 // Hkv, 256)      # one size serves every batch of a graph set
+            partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
+        return nsplit, partials
+
+    def attention_decode_fused(self, qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor,
+                               v_pages: torch.Tensor, block_table: torch.Tensor, page_size: int,
+                               positions: torch.Tensor, token_seq: torch.Tensor, num_heads: int, num_kv_heads: int,
+                               head_dim: int, scale: float, window: Optional[int], plan,
+                               q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                               rope_table: Optional[torch.Tensor], interleaved: bool, store_kv: bool,
+                               unit_offset: bool = False) -> bool:
+        """A decode step's attention straight from the raw rows ``qkv`` = [q | k | v] (or [q] alone
+        without ``store_kv``): per-head norm, rotation, cache write and attention in one kernel.
+        Returns False, having done nothing, when the step or the sizes are not taken; the caller
+        then runs ``qk_norm_rope_store`` and ``attention``."""
+        if (not self.use_fast_kernels or plan is None or not plan.decode_only
+                or not self.lib.has("mv_attention_decode_fused")):
+            return False
+        H, Hkv, D = num_heads, num_kv_heads, head_dim
+        n = qkv.shape[0]
+        width = (H + (2 * Hkv if store_kv else 0)) * D
+        stride = qkv.stride(0) if n > 1 else qkv.shape[1]
+        os_ = out.stride(0) if n > 1 else H * D
+        if (D not in (64, 128) or page_size % 16 or H % Hkv or H // Hkv > 16 or n != plan.n_seqs or n == 0
+                or qkv.dim() != 2 or qkv.shape[1] < width or qkv.stride(1) != 1 or stride % 8 or qkv.data_ptr() % 16
+                or out.shape != (n, H * D) or out.stride(1) != 1 or os_ % 4 or out.data_ptr() % 8
+                or interleaved or (rope_table is not None and (rope_table.dim() != 2 or rope_table.shape[1] != D
+                                                               or rope_table.dtype != torch.float32
+                                                               or not rope_table.is_contiguous()))
+                or (q_weight is None and k_weight is not None)):
+            return False
+        wcode = DTYPE_F32
+        if q_weight is not None:
+            if q_weight.numel() != D or q_weight.data_ptr() % 16 or (
+                    store_kv and (k_weight is None or k_weight.numel() != D or k_weight.dtype != q_weight.dtype
+                                  or k_weight.data_ptr() % 16)):
+                return False
+            wcode = _weight_code(q_weight, "q_norm weight")
+        self._act(qkv, "qkv"); self._act(out, "attention output")
+        self._act(k_pages, "key pages"); self._act(v_pages, "value pages")
+        if tuple(k_pages.shape[1:]) != (Hkv, page_size, D) or tuple(v_pages.shape[1:]) != (Hkv, D, page_size) or \
+                not k_pages.is_contiguous() or not v_pages.is_contiguous():
+            raise KernelLibraryError(f"attention: pages {tuple(k_pages.shape)} / {tuple(v_pages.shape)} have the "
+                                     f"wrong layout for {Hkv} heads of {D}, page {page_size}")
+        for t, what in ((positions, "positions"), (token_seq, "token_seq")):
+            _dev(t, what)
+            if t.dtype != torch.int32 or t.numel() < n:
+                raise KernelLibraryError(f"attention: {what} must be int32 with at least {n} elements")
+        _dev(block_table, "block table")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+            raise KernelLibraryError("attention: the block table must be a contiguous int32 matrix")
+        nsplit, partials = self._decode_split(plan, n, H, Hkv, D)
+        self.lib.call("mv_attention_decode_fused", qkv.data_ptr(), stride, 0, H * D, (H + Hkv) * D, out.data_ptr(), os_,
+                      k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n, H, Hkv, D, float(scale),
+                      -1 if window is None else int(window), _ptr(q_weight), _ptr(k_weight), wcode, float(eps),
+                      int(unit_offset), _ptr(rope_table), int(store_kv), _ptr(partials), nsplit,
+                      DECODE_ATTENTION_WAVES, token_seq.data_ptr(), self._stream())
+        return True
+
     def _attention_fast(self, q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
                         H, Hkv, D, scale, window, plan) -> bool:
         """The MFMA kernels, when the step and the sizes allow them."""
@@ -384,17 +459,7 @@ class Ops:
         group = H // Hkv
         n_seqs = plan.n_seqs
         if plan.decode_only and group <= 16:
-            # Split the keys of a sequence over several workgroups until about 256 workgroups are
-            # in flight, but never below 128 keys per split (measured on MI355X with 8 kv heads:
-            # batch 1 is fastest at 8 to 16 splits, batch 8 at 4, batch 64 without a split). The
-            # count is a property of the plan (a captured graph keeps it); each split takes its
-            # share of the keys a sequence actually has.
-            ctx = max(1, plan.max_context_len)
-            nsplit = max(1, min(256 // max(1, n_seqs * Hkv), max(1, ctx // 128), 64))
-            partials = None
-            if nsplit > 1:
-                rows = max(n_seqs * nsplit, 2048 // Hkv, 256)      # one size serves every batch of a graph set
-                partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
+            nsplit, partials = self._decode_split(plan, n_seqs, H, Hkv, D)
             self.lib.call("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,

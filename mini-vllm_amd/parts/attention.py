@@ -115,12 +115,22 @@ class Attention(Mixer):
                 raise NotImplementedError("a position encoding without a rotary table cannot follow the fused "
                                           "q/k norm; give it a table or leave qk_norm off")
             self.position.apply(q3, k3, ctx)
+        attn = ws.get("attn.out", (n, spec.q_dim), rt.dtype)
+        plan = ctx.attention_plan
+        if plan is not None and plan.decode_only:
+            # a decode step: norm, rotation, cache write and attention in one kernel where it is taken
+            if ops.attention_decode_fused(qkv, attn, kv.k_pages, kv.v_pages, kv.block_table, kv.page_size,
+                                          ctx.positions, ctx.token_seq, spec.num_heads, spec.num_kv_heads,
+                                          spec.head_dim, spec.scale, spec.window, plan, self.q_norm, self.k_norm,
+                                          spec.qk_norm_eps, table, interleaved, not spec.shares_kv):
+                y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
+                ops.gemm(attn, self.w_o, y, self.b_o)
+                return y
         ops.qk_norm_rope_store(
             qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, ctx.positions, ctx.token_seq,
             self.q_norm, self.k_norm, spec.qk_norm_eps, table, interleaved,
             None if spec.shares_kv else kv.k_pages, None if spec.shares_kv else kv.v_pages,
             None if spec.shares_kv else kv.block_table, kv.page_size)
-        attn = ws.get("attn.out", (n, spec.q_dim), rt.dtype)
         ops.attention(qkv[:, :spec.q_dim] if self.width != spec.q_dim else qkv, attn, kv.k_pages, kv.v_pages,
                       kv.block_table, kv.page_size, ctx.positions, ctx.token_seq, spec.num_heads,
                       spec.num_kv_heads, spec.head_dim, spec.scale, spec.window, plan=ctx.attention_plan)

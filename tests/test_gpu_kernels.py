@@ -277,11 +277,13 @@ def fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype):
     return kp, vp
 
 
-def make_plan(q_lens, ctx_lens, max_context_len=None):
+def make_plan(q_lens, ctx_lens, max_context_len=None, decode_only=None):
     from minivllm_amd.engine.step import AttentionPlan
     from minivllm_amd.parts import Workspace
     cu = torch.tensor([0] + list(np.cumsum(q_lens)), dtype=torch.int32, device="cuda")
-    return AttentionPlan(decode_only=all(q == 1 for q in q_lens), max_q_len=max(q_lens),
+    if decode_only is None:
+        decode_only = all(q == 1 for q in q_lens)
+    return AttentionPlan(decode_only=decode_only, max_q_len=max(q_lens),
                          max_context_len=max_context_len or max(ctx_lens), n_seqs=len(q_lens), q_lens=list(q_lens),
                          cu_seqlens=cu, workspace=Workspace(torch.device("cuda:0")))
 
@@ -384,6 +386,107 @@ def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
                   window, plan=plan)
     want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
     assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+
+
+@pytest.mark.parametrize("H,Hkv,D,ps,window", [(16, 8, 128, 16, None), (8, 1, 128, 32, None), (6, 2, 64, 16, 50),
+                                                (16, 1, 64, 64, None)])
+@pytest.mark.parametrize("with_norm,with_rope,store", [(True, True, True), (False, True, True), (True, False, True),
+                                                       (True, True, False)])
+@pytest.mark.parametrize("max_context", [None, 40000])
+def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_rope, store, max_context):
+    """A decode step from the raw [q | k | v] rows: per-head norm, rotation, cache write and attention
+    in one kernel. The slot of the new position holds NaN before (unless the cache is another
+    layer's and already complete), the finished key and value afterwards."""
+    ops = ops_for(torch.bfloat16)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(21)
+    ctx_lens = [1, 17, 300, 1200, 33, 64, 16]
+    q_lens = [1, 1, 1, 0, 1, 1, 1]                  # sequence 3 is padding: no token
+    live = [s for s, ql in enumerate(q_lens) if ql]
+    n = len(live)
+    eps = 1e-5
+    qw = (1 + 0.2 * torch.randn(D, generator=g)).to(dtype) if with_norm else None
+    kw = (1 + 0.2 * torch.randn(D, generator=g)).to(dtype) if with_norm else None
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)))
+    table = ops.rope_table(dev(inv_freq), 1300) if with_rope else None
+
+    def finish(x, w, pos):                      # x [heads, D] raw (bf16 values), float64 math
+        x = x.double()
+        if w is not None:
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+        if with_rope:
+            ang = pos * inv_freq.double()
+            c, sn = torch.cos(ang), torch.sin(ang)
+            a, b = x[:, :D // 2], x[:, D // 2:]
+            x = torch.cat([a * c - b * sn, b * c + a * sn], dim=-1)
+        return x.to(dtype).double()
+
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    raw = torch.randn(n, (H + 2 * Hkv) * D, generator=g).to(dtype)
+    far = 5 if window is None else 300 - 1 - window
+    raw[2, :H * D] = (6.0 * k_all[2][far].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)).reshape(-1).to(dtype)
+    q_fin = torch.zeros(n, H, D, dtype=torch.float64)
+    for t, s in enumerate(live):
+        pos = ctx_lens[s] - 1
+        q_fin[t] = finish(raw[t, :H * D].view(H, D), qw, pos)
+        if store:
+            k_all[s][pos] = finish(raw[t, H * D:(H + Hkv) * D].view(Hkv, D), kw, pos)
+            v_all[s][pos] = raw[t, (H + Hkv) * D:].view(Hkv, D).double()
+    pages_per = [-(-c // ps) for c in ctx_lens]
+    num_pages = sum(pages_per) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, cur = [], 0
+    for n_p in pages_per:
+        tables.append(perm[cur:cur + n_p]); cur += n_p
+    if window is not None:
+        for s, c in enumerate(ctx_lens):
+            for i in range(max(0, (c - 1) - window) // ps):
+                tables[s][i] = -1
+    kp, vp = fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype)
+    want_k, want_v = kp.clone(), vp.clone()
+    if store:                                        # the new slots are not written yet
+        for s in live:
+            pos = ctx_lens[s] - 1
+            kp[tables[s][pos // ps], :, pos % ps, :] = float("nan")
+            vp[tables[s][pos // ps], :, :, pos % ps] = float("nan")
+    bt = torch.full((len(tables), max(pages_per)), -1, dtype=torch.int32)
+    for s, t in enumerate(tables):
+        bt[s, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    positions = torch.tensor([ctx_lens[s] - 1 for s in live], dtype=torch.int32)
+    token_seq = torch.tensor(live, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(D)
+    # as in the engine's padded decode steps: one row per sequence of the plan, padding at the end
+    # (a sequence without a token, a row that belongs to no sequence)
+    out = torch.full((n + 1, H * D), float("nan"), dtype=dtype, device="cuda")
+    plan = make_plan([1] * n + [0], [ctx_lens[s] for s in live], max_context_len=max_context, decode_only=True)
+    rows = raw if store else raw[:, :H * D].contiguous()
+    qkv = dev(torch.cat([rows, torch.full((1, rows.shape[1]), float("nan"), dtype=dtype)]))
+    bt_rows = torch.cat([bt[live], torch.full((1, bt.shape[1]), -1, dtype=torch.int32)]).contiguous()
+    took = ops.attention_decode_fused(qkv, out, kp, vp, dev(bt_rows), ps,
+                                      dev(torch.cat([positions, torch.zeros(1, dtype=torch.int32)])),
+                                      dev(torch.tensor(list(range(n)) + [-1], dtype=torch.int32)), H, Hkv, D, scale,
+                                      window, plan, dev(qw) if with_norm else None, dev(kw) if with_norm else None,
+                                      eps, table, False, store)
+    assert took
+    out = out[:n]
+    seqs = torch.arange(n, dtype=torch.int32)
+    want = reference_attention(q_fin, [k_all[s] for s in live], [v_all[s] for s in live], positions, seqs, H, Hkv,
+                               scale, window)
+    assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+    # the cache: the new slots hold the finished key and the value, everything else is untouched
+    def same(a, b):
+        a, b = a.float().cpu(), b.float().cpu()
+        return bool(torch.all((a == b) | (torch.isnan(a) & torch.isnan(b))))
+    if store:
+        for s in live:
+            pos = ctx_lens[s] - 1
+            page, slot = tables[s][pos // ps], pos % ps
+            got_k = kp[page, :, slot, :].float().cpu().double()
+            assert rel_err(got_k.numpy(), k_all[s][pos].numpy()) <= OP_TOL[dtype]
+            assert torch.equal(vp[page, :, :, slot].float().cpu().double(), v_all[s][pos])
+            want_k[page, :, slot, :] = kp[page, :, slot, :]
+    assert same(kp, want_k) and same(vp, want_v)
 
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
