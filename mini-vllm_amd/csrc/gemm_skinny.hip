@@ -24,6 +24,7 @@ union Frag {
 };
 
 #define SK_MAX_WAVES 8
+#define SK_COMPUTE_UNITS 256
 #ifndef SK_STAGE_FRAGS
 #define SK_STAGE_FRAGS 8    // 16-byte operand loads per lane in one register stage of the main loop
 #endif
@@ -53,15 +54,31 @@ struct NormInput {
 template <int R, int TM, bool SWIGLU, bool NORM, typename TC>
 __global__ void __launch_bounds__(64 * SK_MAX_WAVES)
 gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W, const bf16* __restrict__ bias,
-                   TC* __restrict__ C, long ldc, int M, int N, int K, NormInput norm) {
+                   TC* __restrict__ C, long ldc, int M, int N, int K, int groups, int blocks, NormInput norm) {
     extern __shared__ float red[];  // [S - 1][R * TM][64][4], then (NORM) bf16 [M][K + 8]
+    // The tokens may be dealt out to `groups` workgroups per weight tile (16 * TM tokens each): with
+    // few weight tiles that fills more compute units, and each unit pulls fewer activation rows.
+    // Workgroups go to the chip's eight dies in turn, so the groups of one tile are given ids that
+    // are 8 apart: they share a die's L2 and the tile's weights are fetched from memory once.
+    int block = blockIdx.x;
+    if (groups > 1) {
+        const int within = blockIdx.x % (8 * groups);
+        const int tg = within / 8;
+        block = (blockIdx.x / (8 * groups)) * 8 + within % 8;
+        if (block >= blocks) return;
+        A += (size_t)tg * 16 * TM * lda;
+        C += (size_t)tg * 16 * TM * ldc;
+        M -= tg * 16 * TM;
+        if (M <= 0) return;
+        if (M > 16 * TM) M = 16 * TM;
+    }
     const int S = blockDim.x / MV_WAVE;
     const int wave = threadIdx.x / MV_WAVE;
     const int lane = threadIdx.x % MV_WAVE;
     const int i = lane % 16;
     const int g = lane / 16;
     // output columns of this workgroup: SWIGLU -> 16 columns of I = N; else 16 * R columns of N
-    const int n_base = SWIGLU ? blockIdx.x * 16 : blockIdx.x * 16 * R;
+    const int n_base = SWIGLU ? block * 16 : block * 16 * R;
 
     const int ksteps = K / 32;
     const int per = ksteps / S, rem = ksteps % S;
@@ -295,14 +312,21 @@ static size_t skinny_lds_bytes(int S, int R, int TM, bool with_norm, int M, int 
     return lds;
 }
 
+static int skinny_blocks(int N, int R, bool swiglu) {
+    const int tiles = (N + 15) / 16;
+    return swiglu ? tiles : (tiles + R - 1) / R;
+}
+
 template <int R, int TM, bool SWIGLU, typename TC>
 static void launch_skinny(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N,
                           int K, int S, hipStream_t stream) {
-    const int tiles = (N + 15) / 16;
-    const int blocks = SWIGLU ? tiles : (tiles + R - 1) / R;
+    const int blocks = skinny_blocks(N, R, SWIGLU);
+    const int groups = (M + 16 * TM - 1) / (16 * TM);
+    const int grid = groups > 1 ? (blocks + 7) / 8 * 8 * groups : blocks;
     const size_t lds = skinny_lds_bytes(S, R, TM, false, M, K);
-    hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC>), dim3(blocks), dim3(64 * S), lds, stream,
-                       (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, NormInput{});
+    hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC>), dim3(grid), dim3(64 * S), lds, stream,
+                       (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, groups, blocks,
+                       NormInput{});
 }
 
 template <int R, bool SWIGLU, typename TC>
@@ -312,7 +336,8 @@ static void launch_skinny_norm(const NormInput& norm, const void* W, const void*
     const int blocks = SWIGLU ? tiles : (tiles + R - 1) / R;
     const size_t lds = skinny_lds_bytes(S, R, 1, true, M, K);
     hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC>), dim3(blocks), dim3(64 * S), lds, stream,
-                       (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, norm);
+                       (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, 1, blocks,
+                       norm);
 }
 
 static int pick_waves(int K) {
@@ -325,9 +350,25 @@ static int pick_waves(int K) {
 template <int R, bool SWIGLU, typename TC>
 static int dispatch_tm(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N, int K,
                        int S, hipStream_t stream) {
-    if (M <= 16) launch_skinny<R, 1, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-    else if (M <= 32) launch_skinny<R, 2, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-    else if (M <= 48) launch_skinny<R, 3, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
+    // Token tiles per workgroup: all of them (the weights pass each compute unit once), or fewer
+    // with the tokens dealt out to several workgroups per weight tile. A compute unit pulls
+    // R + TM operand rows of 16 per workgroup it runs; the choice with the least per unit wins.
+    const int tiles_m = (M + 15) / 16;
+    const int blocks = skinny_blocks(N, R, SWIGLU);
+    int best_tm = tiles_m;
+    long best_cost = -1;
+    for (int tm = tiles_m; tm >= 1; --tm) {
+        if (tm == 3 && tiles_m == 4) continue;   // 3 + 1 wastes a workgroup
+        const int groups = (tiles_m + tm - 1) / tm;
+        const long cost = (((long)blocks * groups + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS) * (R + tm);
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best_tm = tm;
+        }
+    }
+    if (best_tm == 1) launch_skinny<R, 1, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
+    else if (best_tm == 2) launch_skinny<R, 2, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
+    else if (best_tm == 3) launch_skinny<R, 3, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
     else launch_skinny<R, 4, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
     return 0;
 }
