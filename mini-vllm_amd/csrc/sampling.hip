@@ -65,10 +65,74 @@ __device__ Best block_argmax(Best b, Best* sh) {
     return sh[16];
 }
 
+// A row needs no threshold when nothing is cut away: its token is one arg-max over the row (of the
+// logits, or of z + Gumbel noise), which many workgroups can share.
+__device__ __forceinline__ bool row_is_simple(int row, int V, float T, const int* top_k, const float* top_p) {
+    if (!(T > 0.f)) return true;
+    const int k = top_k ? top_k[row] : 0;
+    const float p = top_p ? top_p[row] : 1.f;
+    return !(k > 0 && k < V) && !(p < 1.f);
+}
+
+#define SP_PART_THREADS 256
+
+// First of two passes for simple rows: workgroup (row, chunk) finds the best of its chunk of the
+// vocabulary and leaves it in partial[row][chunk]. Rows that need thresholds are left to the
+// second pass alone.
+__global__ void __launch_bounds__(SP_PART_THREADS)
+sample_partial_kernel(const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
+                      const int* __restrict__ top_k, const float* __restrict__ top_p,
+                      const unsigned long long* __restrict__ rng, Best* __restrict__ partial, int chunks) {
+    __shared__ Best sh[SP_PART_THREADS / MV_WAVE];
+    const int row = blockIdx.x, chunk = blockIdx.y;
+    const float T = temperature ? temperature[row] : 0.f;
+    if (!row_is_simple(row, V, T, top_k, top_p)) return;
+    const float* x = logits + (size_t)row * ld;
+    const int per = ((V + chunks - 1) / chunks + 3) & ~3;
+    const int lo = chunk * per, hi = lo + per < V ? lo + per : V;
+    const bool greedy = !(T > 0.f);
+    uint64_t seed = 0, counter = 0;
+    if (!greedy) {
+        seed = rng[2 * (size_t)row];
+        counter = rng[2 * (size_t)row + 1];
+    }
+    Best b{-INFINITY, 0x7fffffff};
+    auto take = [&](float v, int i) {
+        if (!greedy) v = v / T - logf(-logf(uniform23(seed, counter, (uint32_t)i)));
+        b = better(b, Best{v, i});
+    };
+    if ((ld & 3) == 0 && (((uintptr_t)logits) & 15) == 0) {
+        for (int i = lo + 4 * (int)threadIdx.x; i < hi; i += 4 * SP_PART_THREADS) {
+            if (i + 3 < hi) {
+                const float4 v = *reinterpret_cast<const float4*>(x + i);
+                take(v.x, i); take(v.y, i + 1); take(v.z, i + 2); take(v.w, i + 3);
+            } else {
+                for (int j = i; j < hi; ++j) take(x[j], j);
+            }
+        }
+    } else {
+        for (int i = lo + (int)threadIdx.x; i < hi; i += SP_PART_THREADS) take(x[i], i);
+    }
+#pragma unroll
+    for (int o = MV_WAVE / 2; o > 0; o >>= 1) {
+        Best other;
+        other.v = __shfl_xor(b.v, o, MV_WAVE);
+        other.i = __shfl_xor(b.i, o, MV_WAVE);
+        b = better(b, other);
+    }
+    if (threadIdx.x % MV_WAVE == 0) sh[threadIdx.x / MV_WAVE] = b;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < SP_PART_THREADS / MV_WAVE; ++w) b = better(b, sh[w]);
+        partial[(size_t)row * chunks + chunk] = b;
+    }
+}
+
 __global__ void __launch_bounds__(SP_THREADS)
 sample_kernel(const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
               const int* __restrict__ top_k, const float* __restrict__ top_p,
-              const unsigned long long* __restrict__ rng, int* __restrict__ out) {
+              const unsigned long long* __restrict__ rng, int* __restrict__ out,
+              const Best* __restrict__ partial, int chunks) {
     __shared__ Best shb[17];
     __shared__ float scratch[17];
     __shared__ int hcount[256];
@@ -83,6 +147,13 @@ sample_kernel(const float* __restrict__ logits, long ld, int V, const float* __r
     const float T = temperature ? temperature[row] : 0.f;
     const int NEG_I = 0x7fffffff;
 
+    if (partial != nullptr && row_is_simple(row, V, T, top_k, top_p)) {   // the first pass did the work
+        Best b{-INFINITY, NEG_I};
+        for (int c = tid; c < chunks; c += SP_THREADS) b = better(b, partial[(size_t)row * chunks + c]);
+        b = block_argmax(b, shb);
+        if (tid == 0) out[row] = b.i;
+        return;
+    }
     if (!(T > 0.f)) {
         Best b{-INFINITY, NEG_I};
         for (int i = tid; i < V; i += SP_THREADS) b = better(b, Best{x[i], i});
@@ -186,12 +257,22 @@ sample_kernel(const float* __restrict__ logits, long ld, int V, const float* __r
 }
 
 // temperature, top_k, top_p: per row, or null for 0 / off / off. rng: [M][2] = (seed, counter).
+// work: 8 * M * chunks bytes of scratch, or null. With it, rows that need no threshold (greedy
+// rows, and drawn rows without top-k and top-p) are served by two short launches in which
+// `chunks` workgroups share a row; the drawn token is the same either way.
 extern "C" int mv_sample(const float* logits, long ld, int M, int V, const float* temperature, const int* top_k,
-                         const float* top_p, const unsigned long long* rng, int* out, hipStream_t stream) {
+                         const float* top_p, const unsigned long long* rng, int* out, void* work, int chunks,
+                         hipStream_t stream) {
     MV_REQUIRE(M >= 0 && V > 0 && ld >= V, "sample: bad sizes M=%d V=%d ld=%ld", M, V, ld);
     MV_REQUIRE(temperature == nullptr || rng != nullptr, "sample: temperatures given without random keys");
+    MV_REQUIRE(work == nullptr || (chunks >= 1 && chunks <= 65535), "sample: bad chunk count %d", chunks);
     if (M == 0) return 0;
+    if (work != nullptr) {
+        hipLaunchKernelGGL(sample_partial_kernel, dim3(M, chunks), dim3(SP_PART_THREADS), 0, stream, logits, ld, V,
+                           temperature, top_k, top_p, rng, (Best*)work, chunks);
+        if (int rc = mv_check_launch("sample (first pass)")) return rc;
+    }
     hipLaunchKernelGGL(sample_kernel, dim3(M), dim3(SP_THREADS), 0, stream, logits, ld, V, temperature, top_k,
-                       top_p, rng, out);
+                       top_p, rng, out, (const Best*)work, chunks);
     return mv_check_launch("sample");
 }

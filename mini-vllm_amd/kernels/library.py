@@ -43,7 +43,7 @@ _SIGNATURES = {
     "mv_attention_ref": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                  c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
     "mv_sample": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_void_p]),
+                          c_void_p, c_int, c_void_p]),
 }
 
 # entry points that only the bfloat16 library has

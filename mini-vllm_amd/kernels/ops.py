@@ -21,6 +21,9 @@ SKINNY_MAX_M = 64
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
 FUSED_NORM_MAX_CHUNKS = 32
+# the sampler's first pass: workgroups that share a row, and the rows its scratch is made for
+SAMPLE_CHUNKS = 32
+SAMPLE_WORK_ROWS = 1024
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
 # from this many tokens on, value rows are written to their pages by a kernel of their own
@@ -62,6 +65,7 @@ class Ops:
         self.use_library_gemm = dtype == torch.bfloat16
         self.stream_handle: Optional[int] = None
         self._transposed = {}
+        self._sample_work: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------------------------
     def bind_stream(self) -> None:
@@ -509,8 +513,16 @@ class Ops:
             _dev(rng, "rng")
         if M == 0:
             return
+        # rows without thresholds are shared by SAMPLE_CHUNKS workgroups each (two short launches);
+        # the scratch for their partial results is made once
+        work = None
+        if M <= SAMPLE_WORK_ROWS and V >= 4096:
+            if self._sample_work is None:
+                self._sample_work = torch.empty(SAMPLE_WORK_ROWS * SAMPLE_CHUNKS * 2, dtype=torch.int32,
+                                                device=logits.device)
+            work = self._sample_work
         self.lib.call("mv_sample", logits.data_ptr(), logits.stride(0) if M > 1 else V, M, V, _ptr(temperature),
-                      _ptr(top_k), _ptr(top_p), _ptr(rng), out.data_ptr(), self._stream())
+                      _ptr(top_k), _ptr(top_p), _ptr(rng), out.data_ptr(), _ptr(work), SAMPLE_CHUNKS, self._stream())
 
 
 _OPS = {}

@@ -574,6 +574,36 @@ def test_sampling_greedy_and_draws():
             assert score[got[i]] >= score[tok] - 1e-4 * max(1.0, abs(float(score[tok]))), (i, got[i], tok)
 
 
+@pytest.mark.parametrize("V,pad", [(50021, 0), (50021, 3), (151936, 0)])
+def test_sampling_large_vocabulary_two_passes(V, pad):
+    """With a large vocabulary the rows that need no threshold are shared by many workgroups (two
+    launches); every row gets the token the one-launch path gives it."""
+    ops = ops_for(torch.float32)
+    g = torch.Generator().manual_seed(81)
+    M = 7
+    wide = (2.0 * torch.randn(M, V + pad, generator=g)).float()
+    logits = wide[:, :V]
+    logits[0, 11] = logits[0, V - 5] = logits[0].max() + 1       # a tie across chunks: the lowest id wins
+    temps = torch.tensor([0.0, 0.0, 0.9, 1.2, 0.8, 1.0, 0.0])
+    top_k = torch.tensor([0, 5, 0, 0, 50, 0, 0], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 0.5, 1.0, 1.0, 1.0, 0.9, 1.0])
+    rng = torch.tensor([[77 + i, 3] for i in range(M)], dtype=torch.int64)
+    x = dev(wide)[:, :V]
+    two = torch.empty(M, dtype=torch.int32, device="cuda")
+    one = torch.empty(M, dtype=torch.int32, device="cuda")
+    d_temps, d_k, d_p, d_rng = dev(temps), dev(top_k), dev(top_p), dev(rng)
+    ops.sample(x, two, d_temps, d_k, d_p, d_rng)
+    assert ops._sample_work is not None
+    ops.lib.call("mv_sample", x.data_ptr(), x.stride(0), M, V, d_temps.data_ptr(), d_k.data_ptr(), d_p.data_ptr(),
+                 d_rng.data_ptr(), one.data_ptr(), 0, 1, ops._stream())
+    torch.cuda.synchronize()
+    assert two.cpu().tolist() == one.cpu().tolist()
+    assert two[0].item() == 11 and two[1].item() == int(torch.argmax(logits[1])) \
+        and two[6].item() == int(torch.argmax(logits[6]))
+    ops.sample(x, two)                                            # all rows greedy
+    assert two.cpu().tolist() == [11] + [int(torch.argmax(logits[i])) for i in range(1, M)]
+
+
 def test_sampling_frequencies():
     """Draws follow softmax(logits / T) on a small vocabulary."""
     ops = ops_for(torch.float32)
