@@ -27,6 +27,37 @@ extern "C" int mv_embedding(const int* ids, const void* table, int table_dtype, 
     return mv_check_launch("embedding");
 }
 
+// Eight consecutive elements, read and written 16 bytes (bf16) or 32 bytes (float) at a time.
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16> {
+    static __device__ __forceinline__ void load(const bf16* p, float (&x)[8]) {
+        const uint4 u = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x[2 * e] = __uint_as_float(w[e] << 16);
+            x[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ void store(bf16* p, const float (&x)[8]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            w[e] = (uint32_t)f32_to_bf16_bits(x[2 * e]) | ((uint32_t)f32_to_bf16_bits(x[2 * e + 1]) << 16);
+        *reinterpret_cast<uint4*>(p) = uint4{w[0], w[1], w[2], w[3]};
+    }
+};
+template <> struct Vec8<float> {
+    static __device__ __forceinline__ void load(const float* p, float (&x)[8]) {
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&x)[8]) {
+        *reinterpret_cast<float4*>(p) = float4{x[0], x[1], x[2], x[3]};
+        *reinterpret_cast<float4*>(p + 4) = float4{x[4], x[5], x[6], x[7]};
+    }
+};
+
 // ---------------------------------------------------------------------------------------
 // Residual add + RMSNorm.
 //   rows == null : for every row r: v = resid[r] + delta[r]; resid[r] = v; out[r] = norm(v) * w
@@ -71,6 +102,75 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     }
 }
 
+// The same with rows of a multiple of 8 columns, at most 8192: TPR threads share a row (a block
+// of 256 serves 256 / TPR rows), each keeps its chunks of eight columns in registers between the
+// sum of squares and the scaling, so a row is read once.
+#define ARN_MAX_CHUNKS 4
+template <typename T>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta, WeightPtr w, float eps, int unit_offset,
+                       T* __restrict__ out, const int* __restrict__ rows, int n_out, int h, int tpr) {
+    __shared__ float part[256 / MV_WAVE];
+    const int rpb = 256 / tpr;                        // rows of this block
+    const int sub = threadIdx.x / tpr, t = threadIdx.x % tpr;
+    const int i = blockIdx.x * rpb + sub;
+    const bool live = i < n_out;
+    const int r = live ? (rows ? rows[i] : i) : -1;
+    float x[ARN_MAX_CHUNKS][8];
+    float ss = 0.f;
+    if (r >= 0) {
+        float* xr = resid + (size_t)r * h;
+        const T* dl = delta ? delta + (size_t)r * h : nullptr;
+#pragma unroll
+        for (int c = 0; c < ARN_MAX_CHUNKS; ++c) {
+            const int d = (c * tpr + t) * 8;
+            if (d < h) {
+                Vec8<float>::load(xr + d, x[c]);
+                if (dl) {
+                    float dv[8];
+                    Vec8<T>::load(dl + d, dv);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[c][e] += dv[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += x[c][e] * x[c][e];
+            }
+        }
+    }
+    ss = wave_sum(ss);
+    if (tpr > MV_WAVE) {                              // a row spans several waves
+        if (threadIdx.x % MV_WAVE == 0) part[threadIdx.x / MV_WAVE] = ss;
+        __syncthreads();
+        const int w0 = sub * (tpr / MV_WAVE);
+        ss = 0.f;
+        for (int k = 0; k < tpr / MV_WAVE; ++k) ss += part[w0 + k];
+    }
+    if (!live) return;
+    if (r < 0) {
+        if (out) {
+            const float zero[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int d = t * 8; d < h; d += tpr * 8) Vec8<T>::store(out + (size_t)i * h + d, zero);
+        }
+        return;
+    }
+    const float rinv = rsqrtf(ss / (float)h + eps);
+    const bool write_back = rows == nullptr && delta != nullptr;
+#pragma unroll
+    for (int c = 0; c < ARN_MAX_CHUNKS; ++c) {
+        const int d = (c * tpr + t) * 8;
+        if (d < h) {
+            if (write_back) Vec8<float>::store(resid + (size_t)r * h + d, x[c]);
+            if (out) {
+                float wt[8], y[8];
+                w.at8(d, wt);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) y[e] = x[c][e] * rinv * (unit_offset ? wt[e] + 1.f : wt[e]);
+                Vec8<T>::store(out + (size_t)i * h + d, y);
+            }
+        }
+    }
+}
+
 extern "C" int mv_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype, float eps,
                               int unit_offset, void* out, const int* rows, int n_out, int h, int dtype,
                               hipStream_t stream) {
@@ -80,6 +180,17 @@ extern "C" int mv_add_rmsnorm(float* resid, const void* delta, const void* weigh
     MV_REQUIRE(eps > 0.f || out == nullptr, "add_rmsnorm: eps must be positive");
     if (n_out == 0) return 0;
     WeightPtr w{weight, weight_dtype};
+    if (out != nullptr && h % 8 == 0 && h <= 8 * 256 * ARN_MAX_CHUNKS && ((uintptr_t)resid % 16) == 0 &&
+        ((uintptr_t)delta % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)weight % 16) == 0) {
+        // threads per row: a power of two of at least 64 that covers the row in ARN_MAX_CHUNKS chunks or fewer
+        int tpr = 64;
+        while (tpr < 256 && tpr * 8 * 2 <= h) tpr *= 2;
+        const int rpb = 256 / tpr;
+        MV_DISPATCH_T(dtype, "add_rmsnorm",
+                      hipLaunchKernelGGL(add_rmsnorm_vec_kernel<T>, dim3((n_out + rpb - 1) / rpb), dim3(256), 0, stream,
+                                         resid, (const T*)delta, w, eps, unit_offset, (T*)out, rows, n_out, h, tpr));
+        return mv_check_launch("add_rmsnorm");
+    }
     MV_DISPATCH_T(dtype, "add_rmsnorm",
                   hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(256), 0, stream, resid,
                                      (const T*)delta, w, eps, unit_offset, (T*)out, rows, h));
@@ -237,6 +348,105 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, long row_stride, 
     }
 }
 
+// The same for the common case (rotation over the whole head in half-split pairs, head size 64,
+// 128, 256 or 512): a head is spread over L = D / 8 neighbouring lanes, eight elements each, read
+// and written 16 bytes (bf16) at a time; sums and rotation partners travel by lane shuffles, so
+// nothing goes through LDS and a wave serves 64 / L heads.
+template <typename T, int L>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, int k_off, int v_off,
+                              const int* __restrict__ positions, const int* __restrict__ token_seq,
+                              const int* __restrict__ block_table, int bt_width, int page_size,
+                              T* __restrict__ k_pages, T* __restrict__ v_pages, int n, int H, int Hkv,
+                              WeightPtr qw, WeightPtr kw, int has_norm, float eps, int unit_offset,
+                              const float* __restrict__ table, int store_kv) {
+    constexpr int D = 8 * L;
+    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
+    const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long hidx = gid / L;
+    const int j = (int)(gid % L);            // this lane's eight elements start at d0 = 8 j
+    const int tok = (int)(hidx / heads), head = (int)(hidx % heads);
+    const int seq = tok < n ? token_seq[tok] : -1;
+    const bool active = tok < n && seq >= 0;
+    int kind = 0, hh = head;                 // 0 q, 1 k, 2 v
+    if (head >= H + Hkv) {
+        kind = 2;
+        hh = head - H - Hkv;
+    } else if (head >= H) {
+        kind = 1;
+        hh = head - H;
+    }
+    const int pos = active ? positions[tok] : 0;
+    T* src = qkv + (size_t)(active ? tok : 0) * row_stride + (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) +
+             (size_t)hh * D + 8 * j;
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (active) Vec8<T>::load(src, x);
+    if (kind != 2) {
+        if (has_norm) {
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+            for (int o = L / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, MV_WAVE);
+            const float rinv = rsqrtf(ss / (float)D + eps);
+            float wt[8];
+            (kind == 0 ? qw : kw).at8(8 * j, wt);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = x[e] * rinv * (unit_offset ? wt[e] + 1.f : wt[e]);
+        }
+        if (table != nullptr) {
+            const float* cs = table + (size_t)pos * D + 8 * (j % (L / 2));
+            const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
+            const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2);
+            const float4 s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
+            const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            const bool low = j < L / 2;      // holds d < D/2; its partner d + D/2 sits L/2 lanes on
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float other = __shfl_xor(x[e], L / 2, MV_WAVE);
+                x[e] = low ? x[e] * c[e] - other * sn[e] : x[e] * c[e] + other * sn[e];
+            }
+        }
+    }
+    if (!active) return;
+    if (kind == 0) {
+        Vec8<T>::store(src, x);
+        return;
+    }
+    const int page = block_table[(size_t)seq * bt_width + pos / page_size];
+    if (page < 0) return;
+    const int slot = pos % page_size;
+    if (kind == 1) {
+        Vec8<T>::store(k_pages + (((size_t)page * Hkv + hh) * page_size + slot) * D + 8 * j, x);
+    } else {
+        T* dst = v_pages + (((size_t)page * Hkv + hh) * D + 8 * j) * page_size + slot;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[(size_t)e * page_size] = from_f<T>(x[e]);
+    }
+}
+
+template <typename T>
+static bool launch_qk_vec(T* qkv, long row_stride, int q_off, int k_off, int v_off, const int* positions,
+                          const int* token_seq, const int* block_table, int bt_width, int page_size, T* k_pages,
+                          T* v_pages, int n, int H, int Hkv, int D, WeightPtr qw, WeightPtr kw, int has_norm, float eps,
+                          int unit_offset, const float* table, int store_kv, hipStream_t stream) {
+    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
+    const long lanes = (long)n * heads * (D / 8);
+    const dim3 grid((unsigned)((lanes + 255) / 256));
+#define QK_VEC(LL)                                                                                                 \
+    hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<T, LL>), grid, dim3(256), 0, stream, qkv, row_stride, q_off,   \
+                       k_off, v_off, positions, token_seq, block_table, bt_width, page_size, k_pages, v_pages, n, H, \
+                       Hkv, qw, kw, has_norm, eps, unit_offset, table, store_kv)
+    if (D == 64) QK_VEC(8);
+    else if (D == 128) QK_VEC(16);
+    else if (D == 256) QK_VEC(32);
+    else if (D == 512) QK_VEC(64);
+    else return false;
+#undef QK_VEC
+    return true;
+}
+
 extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int k_off, int v_off,
                                      const int* positions, const int* token_seq, const int* block_table,
                                      int bt_width, int page_size, void* k_pages, void* v_pages, int n, int H,
@@ -258,6 +468,21 @@ extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int 
     if (n == 0) return 0;
     const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
     WeightPtr qw{q_weight, weight_dtype}, kw{k_weight, weight_dtype};
+    // the vector kernel: rotation over the whole head in half-split pairs, everything 16-byte aligned
+    const size_t esz = dtype == MV_F32 ? 4 : 2;
+    const bool aligned = ((uintptr_t)qkv % 16) == 0 && (row_stride * esz) % 16 == 0 && (q_off * esz) % 16 == 0 &&
+                         (k_off * esz) % 16 == 0 && (v_off * esz) % 16 == 0 && ((uintptr_t)k_pages % 16) == 0 &&
+                         ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0 &&
+                         ((uintptr_t)table % 16) == 0;
+    if (aligned && (D == 64 || D == 128 || D == 256 || D == 512) && (table == nullptr || (rot_dim == D && !interleaved)) &&
+        (long)n * heads * (D / 8) < (1L << 31)) {
+        bool took = false;
+        MV_DISPATCH_T(dtype, "qk_norm_rope_store",
+                      took = launch_qk_vec<T>((T*)qkv, row_stride, q_off, k_off, v_off, positions, token_seq,
+                                              block_table, bt_width, page_size, (T*)k_pages, (T*)v_pages, n, H, Hkv, D,
+                                              qw, kw, has_norm, eps, unit_offset, table, store_kv, stream));
+        if (took) return mv_check_launch("qk_norm_rope_store");
+    }
     dim3 grid(n, (heads + 3) / 4);
     MV_DISPATCH_T(dtype, "qk_norm_rope_store",
                   hipLaunchKernelGGL(qk_norm_rope_store_kernel<T>, grid, dim3(256), 0, stream, (T*)qkv, row_stride,
@@ -339,9 +564,31 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, lon
     out[idx] = from_f<T>(g / (1.f + expf(-g)) * u);
 }
 
+template <typename T>
+__global__ void swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, long total8, int I8) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;   // eight columns each
+    if (idx >= total8) return;
+    const long row = idx / I8;
+    const int col = (int)(idx - row * I8) * 8;
+    const int I = I8 * 8;
+    float g[8], u[8], y[8];
+    Vec8<T>::load(gu + row * 2 * I + col, g);
+    Vec8<T>::load(gu + row * 2 * I + I + col, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+    Vec8<T>::store(out + row * I + col, y);
+}
+
 extern "C" int mv_swiglu(const void* gate_up, void* out, int n, int I, int dtype, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && I > 0, "swiglu: bad sizes n=%d I=%d", n, I);
     if (n == 0) return 0;
+    if (I % 8 == 0 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        const long total8 = (long)n * (I / 8);
+        MV_DISPATCH_T(dtype, "swiglu",
+                      hipLaunchKernelGGL(swiglu_vec_kernel<T>, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0,
+                                         stream, (const T*)gate_up, (T*)out, total8, I / 8));
+        return mv_check_launch("swiglu");
+    }
     const long total = (long)n * I;
     const unsigned blocks = (unsigned)((total + 255) / 256);
     MV_DISPATCH_T(dtype, "swiglu",
