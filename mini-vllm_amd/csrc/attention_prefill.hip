@@ -35,8 +35,11 @@ union Frag {
 #define AP_THREADS (64 * AP_WAVES)
 #define LOG2E 1.4426950408889634f
 
+// Two workgroups share a compute unit (LDS and latency hiding are sized for that), so a wave may
+// use half of a SIMD's registers: the accumulators stay in the vector registers and the operand
+// reads from LDS run ahead of the MFMAs.
 template <int D, int NT>
-__global__ void __launch_bounds__(AP_THREADS)
+__global__ void __launch_bounds__(AP_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                          const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                          const int* __restrict__ block_table, int bt_width, int page_size, int page_shift,
@@ -255,17 +258,26 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         const bool masked = !(wave_full && base + 31 <= full_hi && base >= full_lo);
         // scores^T for the two 16-key tiles
         float p[NT][2][4];
+        Frag kop[2][DS];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < DS; ++s) kop[t][s].u = sK[cur][(t * DS + s) * 64 + lane];
+        // the value operands are asked for now and arrive while the softmax is worked out
+        Frag vop[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            vop[dt].h[0] = sV[cur][(dt * 64 + lane) * 2];
+            vop[dt].h[1] = sV[cur][(dt * 64 + lane) * 2 + 1];
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            Frag kop[DS];
-#pragma unroll
-            for (int s = 0; s < DS; ++s) kop[s].u = sK[cur][(t * DS + s) * 64 + lane];
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct) {
                 floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s = 0; s < DS; ++s)
-                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[s].v, qop[ct][s].v, sacc, 0, 0, 0);
+                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[t][s].v, qop[ct][s].v, sacc, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) p[ct][t][r] = sacc[r];
             }
@@ -291,15 +303,16 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) mx = fmaxf(mx, p[ct][t][r]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
             // The reference point of the exponentials (kept in the scaled, base-2 domain; the scale
             // is positive) only follows the maximum when it has been overtaken by more than 2^8:
-            // until then the terms stay below 2^8, and the accumulators need no rescaling, which
-            // would move them between the accumulation and the vector registers.
-            const float mx_s = mx * sc_mul;
-            const bool stale = mx_s > m_run[ct] + 8.f;
+            // until then the terms stay below 2^8 and nothing is rescaled. A column's maximum is
+            // spread over four lanes, but it exceeds the bound exactly when one lane's share does,
+            // so the lanes are only brought together (two shuffles) when a vote says so.
+            const bool stale = mx * sc_mul > m_run[ct] + 8.f;
             if (__any(stale)) {
+                mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
+                const float mx_s = mx * sc_mul;
                 const float m_new = fmaxf(m_run[ct], mx_s);
                 const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;
                 const float corr = __builtin_amdgcn_exp2f(m_run[ct] - m_ref);   // exp2(-inf) = 0
@@ -322,14 +335,10 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         }
         // out^T += V^T P^T
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            Frag vop;
-            vop.h[0] = sV[cur][(dt * 64 + lane) * 2];
-            vop.h[1] = sV[cur][(dt * 64 + lane) * 2 + 1];
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct)
-                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
-        }
+                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
     };
 
     Staged sa, sb;

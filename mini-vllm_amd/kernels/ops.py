@@ -24,6 +24,8 @@ FUSED_NORM_MAX_CHUNKS = 32
 # the sampler's first pass: workgroups that share a row, and the rows its scratch is made for
 SAMPLE_CHUNKS = 32
 SAMPLE_WORK_ROWS = 1024
+# compute units of the device the launch heuristics are tuned for
+COMPUTE_UNITS = 256
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
 # from this many tokens on, value rows are written to their pages by a kernel of their own
@@ -471,13 +473,18 @@ class Ops:
             return True
         if page_size & (page_size - 1):
             return False
-        # 64 columns per workgroup (two workgroups fit a CU and hide each other's waits; measured
-        # faster than 128 columns at every prompt length); 128 only for groups of more than 64 heads
+        # 128 columns per workgroup (each operand read from LDS feeds two MFMAs) when that still leaves
+        # two workgroups for every compute unit, else 64 (measured on MI355X: 2048 tokens of one
+        # sequence with 8 kv heads are faster with 64, 4096 tokens or 8 x 512 with 128)
         nt, n_units = 0, 0
-        for cand in (1, 2):
+        for cand in (2, 1):
             u = self.lib.dll.mv_attention_prefill_unit_tokens(group, cand)
             if u > 0:
-                nt, n_units = cand, sum(-(-ql // u) for ql in plan.q_lens)
+                units = sum(-(-ql // u) for ql in plan.q_lens)
+                if cand == 2 and units * Hkv < 2 * COMPUTE_UNITS and \
+                        self.lib.dll.mv_attention_prefill_unit_tokens(group, 1) > 0:
+                    continue
+                nt, n_units = cand, units
                 break
         if nt == 0:
             return False
