@@ -74,7 +74,7 @@ def build_llm(args, shape, layers):
                       max_num_batched_tokens=max(args.prefill_tokens, 2048), max_num_batched_seqs=max(64, args.batch),
                       kv_cache_block_size=args.block_size,
                       kv_cache_num_blocks=max(64, args.batch) * pages_per_seq + 16,
-                      use_cuda_graph=not args.no_graph, seed=args.seed)
+                      use_cuda_graph=not args.no_graph, num_scheduler_steps=args.scheduler_steps, seed=args.seed)
     return LLM(config=ec, model_source=(arch, cfg, source)), cfg
 
 
@@ -84,28 +84,38 @@ def random_prompt(vocab, n, seed):
 
 
 def measure_decode(llm, vocab, batch, prompt_len, steps, warmup, seed):
-    """Tokens per second of ``steps`` decode steps at ``batch`` after the prompts are in the cache."""
+    """Tokens per second over ``steps`` decode steps (tokens per request) at ``batch`` after the
+    prompts are in the cache. One call of ``llm.step()`` may run several decode steps in a row on
+    the device; what is counted is what the requests received."""
     import torch
     from minivllm_amd import SamplingParams
-    sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8, ignore_eos=True)
+    # room for what the first requests decode while the last prompts are still being read
+    sp = SamplingParams(temperature=0.0, max_tokens=llm.config.max_model_len - prompt_len - 1, ignore_eos=True)
     reqs = [llm.submit(random_prompt(vocab, prompt_len, seed + i), sp) for i in range(batch)]
     while any(r.num_completion_tokens == 0 for r in reqs):          # prompts in, first token drawn
         llm.step()
-    for _ in range(warmup):
-        llm.step()
+    def run(n):
+        target = min(r.num_completion_tokens for r in reqs) + n
+        while min(r.num_completion_tokens for r in reqs) < target:
+            if llm.step() is None or any(r.finished for r in reqs):
+                raise RuntimeError("a request of the benchmark ended before the timed steps were over; "
+                                   "give it a longer --context")
+    run(warmup)
     torch.cuda.synchronize()
+    before = sum(r.num_completion_tokens for r in reqs)
     t0 = time.perf_counter()
-    for _ in range(steps):
-        llm.step()
+    run(steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    mean_ctx = prompt_len + 1 + warmup + steps / 2.0
+    tokens = sum(r.num_completion_tokens for r in reqs) - before
+    done_steps = tokens / batch
+    mean_ctx = prompt_len + 1 + warmup + done_steps / 2.0
     # finish and free
     for r in reqs:
         r.sampling_params.max_tokens = r.num_completion_tokens
     while llm.has_unfinished():
         llm.step()
-    return batch * steps / dt, dt / steps * 1e3, mean_ctx
+    return tokens / dt, dt / done_steps * 1e3, mean_ctx, int(round(done_steps))
 
 
 def measure_prefill(llm, vocab, tokens, repeats, seed):
@@ -138,6 +148,8 @@ def main() -> int:
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--scheduler-steps", type=int, default=4,
+                    help="decode steps run in a row on the device before the host looks at the tokens")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
@@ -168,9 +180,10 @@ def main() -> int:
                    "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
 
     tok_s = ms_step = roofline = None
+    ran = 0
     if args.only in ("all", "decode"):
-        tok_s, ms_step, mean_ctx = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len, args.steps,
-                                                  args.warmup, args.seed)
+        tok_s, ms_step, mean_ctx, ran = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len, args.steps,
+                                                       args.warmup, args.seed)
         step_bytes = nums["step_params"] * item + args.batch * mean_ctx * nums["kv_bytes_per_token"] * item
         achieved = step_bytes / (ms_step * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -180,7 +193,7 @@ def main() -> int:
     if not args.no_points and args.only == "all":
         for b, key in ((1, "decode_b1"), (64, "decode_b64")):
             n = min(args.steps, 128)
-            v, _, _ = measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8), args.seed + b)
+            v, _, _, _ = measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8), args.seed + b)
             points[key] = round(v, 1)
 
     config = {"model": f"qwen3-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
@@ -188,9 +201,10 @@ def main() -> int:
               "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
               "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch, "seq_len": args.context,
               "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
+              "scheduler_steps": args.scheduler_steps,
               "parallelism": "single-gpu"}
     line = {"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
-            "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1, "steps": ran if ran else args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms_step, 4) if ms_step is not None else None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic", "config": config,
             "prefill": prefill, "roofline": roofline, "points": points}

@@ -45,6 +45,9 @@ class EngineConfig:
 
     # ---- executor ----------------------------------------------------------------------
     use_cuda_graph: bool = True
+    # decode-only steps run this many times in a row on the device before the host looks at the
+    # tokens (1: every step comes back to the host)
+    num_scheduler_steps: int = 4
     seed: int = 0
 
     def __post_init__(self) -> None:
@@ -53,6 +56,8 @@ class EngineConfig:
     def validate(self) -> None:
         if self.dtype not in (None, "bfloat16", "float32"):
             raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
+        if self.num_scheduler_steps < 1:
+            raise ValueError(f"num_scheduler_steps must be >= 1, got {self.num_scheduler_steps}")
         if self.max_model_len < 1:
             raise ValueError(f"max_model_len must be >= 1, got {self.max_model_len}")
         if self.max_num_batched_tokens < 1:

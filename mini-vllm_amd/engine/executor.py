@@ -124,6 +124,7 @@ class Executor:
         self._meta_device: Optional[torch.Tensor] = None
         self._graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, StepContext, torch.Tensor, torch.Tensor]] = {}
         self._graph_pool = None
+        self._repeat_graphs: Dict[Tuple[int, int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
         self._graph_workspace: Optional[Workspace] = None
         self.kv_pages: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
         self.state_tensors: Dict[int, torch.Tensor] = {}
@@ -175,6 +176,7 @@ class Executor:
             v = torch.zeros((num_pages,) + v_shape, dtype=self.dtype, device=self.device)
             self.kv_pages[call] = (k, v)
         self._graphs.clear()
+        self._repeat_graphs.clear()
 
     def _warmup(self, num_tokens: int) -> None:
         """One dry step of ``num_tokens`` tokens against a throw-away cache, so that every scratch
@@ -204,10 +206,11 @@ class Executor:
     # ------------------------------------------------------------------------------------
     # building a step
     # ------------------------------------------------------------------------------------
-    def _validate(self, seqs: Sequence[SeqStep]) -> None:
+    def _validate(self, seqs: Sequence[SeqStep], lookahead: int = 0) -> None:
+        """``lookahead``: positions beyond the step's own that later runs of a repeated step write."""
         ps = self.page_size
         for i, s in enumerate(seqs):
-            n = len(s.tokens)
+            n = len(s.tokens) + lookahead
             if n < 1:
                 raise ValueError(f"sequence {i} of the step brings no token")
             if s.start < 0 or s.start + n > self.config.max_model_len:
@@ -219,7 +222,7 @@ class Executor:
             if not (0 <= s.state_slot < self.num_state_slots):
                 raise ValueError(f"sequence {i}: state slot {s.state_slot} out of range")
             for w in s.want:
-                if not (0 <= w < n):
+                if not (0 <= w < len(s.tokens)):
                     raise ValueError(f"sequence {i}: wanted index {w} outside its {n} tokens")
             last_page = (s.start + n - 1) // ps
             for g in range(len(self.groups)):
@@ -227,8 +230,11 @@ class Executor:
                     raise ValueError(f"sequence {i}: group {g} has {len(s.block_tables[g])} pages, position "
                                      f"{s.start + n - 1} needs {last_page + 1}")
 
-    def _fill(self, seqs: Sequence[SeqStep], pad_to: Optional[int] = None, bt_widths: Optional[List[int]] = None):
-        """Packs the step's integers into one int32 array. Returns (array, offsets dict, facts)."""
+    def _fill(self, seqs: Sequence[SeqStep], pad_to: Optional[int] = None, bt_widths: Optional[List[int]] = None,
+              lookahead: int = 0, extra_words: int = 0):
+        """Packs the step's integers into one int32 array. Returns (array, offsets dict, facts).
+        ``lookahead`` extends the check of the block tables to positions that later runs of a
+        repeated step touch; ``extra_words`` leaves room at the end (offset "extra", 8-byte aligned)."""
         S = len(seqs)
         q_lens = [len(s.tokens) for s in seqs]
         N = sum(q_lens)
@@ -251,6 +257,10 @@ class Executor:
         for g, w in enumerate(widths):
             off[f"bt{g}"] = (cur, Sp * w)
             cur += Sp * w
+        if extra_words:
+            cur += cur & 1
+            off["extra"] = (cur, extra_words)
+            cur += extra_words
         arr = np.zeros(cur, dtype=np.int32)
         tok = arr[off["token_ids"][0]:off["token_ids"][0] + Np]
         pos = arr[off["positions"][0]:off["positions"][0] + Np]
@@ -273,7 +283,7 @@ class Executor:
             base += n
         cu[S + 1:] = base
         starts = np.fromiter((s.start for s in seqs), dtype=np.int64, count=S)
-        last_page = (cl[:S].astype(np.int64) - 1) // self.page_size
+        last_page = (cl[:S].astype(np.int64) - 1 + lookahead) // self.page_size
         for g, w in enumerate(widths):
             o, size = off[f"bt{g}"]
             bt = arr[o:o + size].reshape(Sp, w)
@@ -393,6 +403,104 @@ class Executor:
         self._upload(arr, dst=meta)
         graph.replay()
         return logits[:S]
+
+    # ------------------------------------------------------------------------------------
+    # a decode step run several times in a row on the device
+    # ------------------------------------------------------------------------------------
+    def can_repeat(self, num_seqs: int) -> bool:
+        return bool(self.config.use_cuda_graph) and num_seqs <= GRAPH_BUCKETS[-1]
+
+    @torch.inference_mode()
+    def step_repeated(self, seqs: Sequence[SeqStep], repeat: int, temperature: np.ndarray, top_k: np.ndarray,
+                      top_p: np.ndarray, seeds: np.ndarray, counters: np.ndarray) -> np.ndarray:
+        """Runs a step of single decoded tokens ``repeat`` times in a row, as one graph: every run
+        draws a token per sequence (per-sequence sampling arrays of length len(seqs); ``counters``
+        is the index of the first token each sequence draws) and the next run takes it as its
+        input at the next position. The sequences must hold pages for all ``repeat`` positions.
+        Returns the drawn tokens, int32 [repeat, len(seqs)]."""
+        S = len(seqs)
+        if not self.can_repeat(S) or repeat < 1 or any(len(s.tokens) != 1 or list(s.want) != [0] for s in seqs):
+            raise ValueError("a repeated step takes graph-sized batches of single tokens, each wanted")
+        self._validate(seqs, lookahead=repeat - 1)
+        if self.has_state:
+            for s in seqs:
+                if s.start == 0:
+                    for t in self.state_tensors.values():
+                        t[s.state_slot].zero_()
+        bucket = next(b for b in GRAPH_BUCKETS if b >= S)
+        longest = max(s.start + repeat for s in seqs)
+        cap = 1024
+        while cap < longest:
+            cap *= 2
+        cap = min(cap, max(self.config.max_model_len, 1))
+        widths = [self.max_pages_per_seq] * len(self.groups)
+        # sampling arrays behind the step's integers: temperature, top_k, top_p, (seed, counter) pairs
+        arr, off, facts = self._fill(seqs, pad_to=bucket, bt_widths=widths, lookahead=repeat - 1,
+                                     extra_words=7 * bucket)
+        o = off["extra"][0]                              # even: the 64-bit pairs come first
+        rng = np.zeros((bucket, 2), dtype=np.int64)
+        rng[:S, 0] = np.asarray(seeds, dtype=np.int64)
+        rng[:S, 1] = np.asarray(counters, dtype=np.int64)
+        arr[o:o + 4 * bucket] = rng.reshape(-1).view(np.int32)
+        arr[o + 4 * bucket:o + 4 * bucket + S] = np.asarray(temperature, dtype=np.float32).view(np.int32)
+        arr[o + 5 * bucket:o + 5 * bucket + S] = np.asarray(top_k, dtype=np.int32)
+        tp = np.ones(bucket, dtype=np.float32)
+        tp[:S] = np.asarray(top_p, dtype=np.float32)
+        arr[o + 6 * bucket:o + 7 * bucket] = tp.view(np.int32)
+        key = (bucket, cap, repeat)
+        entry = self._repeat_graphs.get(key)
+        if entry is None:
+            entry = self._capture_repeated(key, arr, off, facts, seqs)
+        graph, meta, tokens = entry
+        self._upload(arr, dst=meta)
+        graph.replay()
+        return tokens[:, :S].cpu().numpy()
+
+    def _capture_repeated(self, key, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
+        bucket, cap, repeat = key
+        logger.info("capturing %d decode steps in a row for %d sequences, contexts up to %d", repeat, bucket, cap)
+        if (bucket, cap) not in self._graphs:
+            # the single-step capture sizes the shared scratch area and loads every kernel
+            a1, o1, f1 = self._fill(seqs, pad_to=bucket, bt_widths=[self.max_pages_per_seq] * len(self.groups))
+            self._capture(bucket, cap, a1, o1, f1, seqs)
+        library_gemm = self.ops.use_library_gemm
+        eager_workspace = self.rt.workspace
+        self.ops.use_library_gemm = False
+        try:
+            self.rt.workspace = self._graph_workspace
+            meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
+            self._upload(arr, dst=meta)
+            ctx = self._context(meta, off, facts, seqs)
+            ctx.attention_plan.max_context_len = cap
+            o = off["extra"][0]
+            rng = meta[o:o + 4 * bucket].view(torch.int64).view(bucket, 2)
+            temps = meta[o + 4 * bucket:o + 5 * bucket].view(torch.float32)
+            top_k = meta[o + 5 * bucket:o + 6 * bucket]
+            top_p = meta[o + 6 * bucket:o + 7 * bucket].view(torch.float32)
+            tokens = torch.zeros((repeat, bucket), dtype=torch.int32, device=self.device)
+            logits = self.model.forward(ctx)       # an eager run: it draws into row 0 and changes nothing else
+            self.ops.sample(logits[:bucket], tokens[0], temps, top_k, top_p, rng)
+            torch.cuda.synchronize()
+            self._graph_workspace.frozen = True
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                for j in range(repeat):
+                    logits = self.model.forward(ctx)
+                    self.ops.sample(logits[:bucket], tokens[j], temps, top_k, top_p, rng)
+                    if j + 1 < repeat:             # the next run: the drawn tokens, one position on
+                        ctx.token_ids.copy_(tokens[j])
+                        ctx.positions.add_(1)
+                        ctx.context_lens.add_(1)
+                        rng[:, 1].add_(1)
+            self._graph_pool = graph.pool()
+        finally:
+            self._graph_workspace.frozen = False
+            self.rt.workspace = eager_workspace
+            self.ops.use_library_gemm = library_gemm
+        torch.cuda.synchronize()
+        entry = (graph, meta, tokens)
+        self._repeat_graphs[key] = entry
+        return entry
 
     def _padding_step(self, bucket: int) -> StepContext:
         """A context of ``bucket`` padding rows: every kernel runs, none touches the cache."""

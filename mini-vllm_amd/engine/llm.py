@@ -60,7 +60,8 @@ class LLM:
         if eos is None:
             eos = tuple(getattr(self.executor.model_config, "eos_token_ids", ()))
         self.scheduler = Scheduler(self.manager, config.max_num_batched_tokens, config.max_num_batched_seqs,
-                                   config.max_model_len, eos, config.prefill_chunk)
+                                   config.max_model_len, eos, config.prefill_chunk,
+                                   max_decode_repeat=config.num_scheduler_steps)
         self.sampler = Sampler(self.executor.ops, self.executor.device)
         self.metrics = Metrics()
         self._seeds: Dict[int, int] = {}
@@ -98,13 +99,16 @@ class LLM:
             seqs.append(SeqStep(tokens=r.tokens[s.start:s.start + s.num_tokens], start=s.start,
                                 block_tables=[cache.pages[g] for g in groups], state_slot=cache.state_slot,
                                 want=[s.num_tokens - 1] if s.sample else []))
-        logits = self.executor.step(seqs)
-        drawing = [s.request for s in step.seqs if s.sample]
-        tokens = self.sampler.sample(logits, [r.sampling_params for r in drawing],
-                                     [self._seeds[r.id] for r in drawing],
-                                     [r.num_completion_tokens for r in drawing])
-        it = iter(tokens)
-        sampled = [next(it) if s.sample else None for s in step.seqs]
+        if step.repeat > 1:
+            sampled = self._run_repeated(step, seqs)
+        else:
+            logits = self.executor.step(seqs)
+            drawing = [s.request for s in step.seqs if s.sample]
+            tokens = self.sampler.sample(logits, [r.sampling_params for r in drawing],
+                                         [self._seeds[r.id] for r in drawing],
+                                         [r.num_completion_tokens for r in drawing])
+            it = iter(tokens)
+            sampled = [next(it) if s.sample else None for s in step.seqs]
         preempted_before = self.scheduler.num_preemptions
         done = self.scheduler.update(step, sampled)
         for r in done:
@@ -113,6 +117,28 @@ class LLM:
         self.metrics.preemptions = self.scheduler.num_preemptions
         step.finished = done
         return step
+
+    def _run_repeated(self, step: ScheduledStep, seqs: List[SeqStep]) -> List[List[int]]:
+        """A step of decoded tokens that runs ``step.repeat`` times in a row: as one graph on the
+        device where the executor offers that, else run by run from here. Returns the tokens each
+        sequence drew, in order."""
+        reqs = [s.request for s in step.seqs]
+        params = [r.sampling_params for r in reqs]
+        seeds = [self._seeds[r.id] for r in reqs]
+        counters = [r.num_completion_tokens for r in reqs]
+        if self.executor.can_repeat(len(seqs)):
+            drawn = self.executor.step_repeated(seqs, step.repeat, *Sampler.arrays(params, seeds, counters))
+            return [[int(t) for t in drawn[:, i]] for i in range(len(seqs))]
+        out: List[List[int]] = [[] for _ in seqs]
+        for j in range(step.repeat):
+            if j:
+                seqs = [SeqStep(tokens=[out[i][-1]], start=s.start + 1, block_tables=s.block_tables,
+                                state_slot=s.state_slot, want=[0]) for i, s in enumerate(seqs)]
+            logits = self.executor.step(seqs)
+            tokens = self.sampler.sample(logits, params, seeds, [c + j for c in counters])
+            for i, t in enumerate(tokens):
+                out[i].append(int(t))
+        return out
 
     # ---- batch generation ---------------------------------------------------------------------
     def _encode(self, prompt: Union[str, Sequence[int]]) -> List[int]:

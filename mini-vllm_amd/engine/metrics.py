@@ -49,14 +49,15 @@ class Metrics:
     def update(self, step, finished, elapsed: float) -> None:
         """``step`` is the ScheduledStep that ran, ``finished`` the requests it completed,
         ``elapsed`` its wall time in seconds."""
+        repeat = getattr(step, "repeat", 1)     # a decode-only step may have run several times in a row
         prefill = sum(s.num_tokens for s in step.seqs if not s.is_decode)
-        decode = sum(s.num_tokens for s in step.seqs if s.is_decode)
+        decode = sum(s.num_tokens for s in step.seqs if s.is_decode) * repeat
         total = max(1, prefill + decode)
         self.prefill_time += elapsed * prefill / total
         self.decode_time += elapsed * decode / total
         self.prefill_tokens += prefill
         self.decode_tokens += decode
-        self.decode_steps += 1 if decode else 0
+        self.decode_steps += repeat if decode else 0
         self.steps += 1
         for s in step.seqs:
             r = s.request

@@ -22,6 +22,12 @@ When pages run out:
   * if a step would be empty although requests are running, the newest running one is
     preempted so that the others can go on;
   * a request that could never fit the pool, or exceeds ``max_model_len``, is refused at submit.
+
+A step that holds only decoded tokens may be marked to run several times in a row
+(``ScheduledStep.repeat``, at most ``max_decode_repeat``): the device feeds each run the tokens
+the run before drew, and the host schedules, uploads and reads back once for all of them. It is
+used only while nobody waits, and never past a request's ``max_tokens``; tokens run past an
+end-of-sequence token are dropped. The reference schedules one token per step.
 """
 from __future__ import annotations
 
@@ -50,10 +56,13 @@ class ScheduledSeq:
 class ScheduledStep:
     seqs: List[ScheduledSeq]
     create_time: float = field(default_factory=time.perf_counter)
+    # A step of decoded tokens only may be run ``repeat`` times in a row on the device, each run
+    # taking the tokens the run before drew: the host then works once per ``repeat`` tokens.
+    repeat: int = 1
 
     @property
     def num_tokens(self) -> int:
-        return sum(s.num_tokens for s in self.seqs)
+        return sum(s.num_tokens for s in self.seqs) * self.repeat
 
     @property
     def requests(self) -> List[Request]:
@@ -62,8 +71,10 @@ class ScheduledStep:
 
 class Scheduler:
     def __init__(self, manager: CacheManager, max_num_batched_tokens: int, max_num_batched_seqs: int,
-                 max_model_len: int, eos_token_ids: Sequence[int] = (), prefill_chunk: Optional[int] = None):
+                 max_model_len: int, eos_token_ids: Sequence[int] = (), prefill_chunk: Optional[int] = None,
+                 max_decode_repeat: int = 1):
         self.manager = manager
+        self.max_decode_repeat = max(1, int(max_decode_repeat))
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_num_batched_seqs = max_num_batched_seqs
         self.max_model_len = max_model_len
@@ -179,12 +190,34 @@ class Scheduler:
             n = min(n, self.prefill_chunk)
         return n
 
+    def _decode_repeat(self, seqs: List[ScheduledSeq]) -> int:
+        """How many times in a row the step may run: more than once only when it holds nothing
+        but decoded tokens, nobody waits to be admitted or to go on with a prompt, and every
+        request has that many tokens to go and the pages for them (they are reserved here)."""
+        k = self.max_decode_repeat
+        if k <= 1 or self.waiting or len(seqs) != len(self.running) or not all(s.is_decode for s in seqs):
+            return 1
+        for s in seqs:
+            r = s.request
+            k = min(k, r.sampling_params.max_tokens - r.num_completion_tokens, self.max_model_len - len(r.tokens))
+        while k > 1:
+            # one position each is reserved already; the others must fit together
+            extra = [self.manager.pages_needed(s.request.id, k) for s in seqs]
+            if all(sum(e[g] for e in extra) <= self.manager.pools[g].num_free for g in range(len(self.manager.groups))):
+                break
+            k -= 1
+        if k <= 1:
+            return 1
+        for s in seqs:
+            self.manager.reserve(s.request.id, k)
+        return k
+
     def schedule(self) -> Optional[ScheduledStep]:
         """The next step, or None when nothing is left to do."""
         while True:
             seqs = self._try_schedule()
             if seqs:
-                return ScheduledStep(seqs)
+                return ScheduledStep(seqs, repeat=self._decode_repeat(seqs))
             if self.running:
                 # everyone is stuck waiting for pages: the newest gives way
                 self.preempt(self.running[-1])
@@ -201,29 +234,37 @@ class Scheduler:
         requests that finished."""
         done: List[Request] = []
         now = time.perf_counter()
-        for seq, token in zip(step.seqs, sampled):
+        for seq, drawn in zip(step.seqs, sampled):
             req = seq.request
-            self.manager.commit(req.id, seq.num_tokens, req.tokens)
             if not seq.sample:
+                self.manager.commit(req.id, seq.num_tokens, req.tokens)
                 continue
-            if token is None:
+            if drawn is None:
                 raise ValueError(f"request {req.id} reached its last token but no token was drawn")
-            req.append_output_token(token)
-            if req.first_token_time is None:
-                req.first_token_time = now
-            sp = req.sampling_params
-            reason = None
-            if token in self.eos_token_ids and not sp.ignore_eos:
-                reason = "stop"
-            elif req.num_completion_tokens >= sp.max_tokens:
-                reason = "length"
-            elif len(req.tokens) >= self.max_model_len:
-                reason = "length"
-            if reason is not None:
-                req.state = RequestState.FINISHED
-                req.finish_reason = reason
-                req.finish_time = now
-                self.manager.release(req.id)
-                self.running.remove(req)
-                done.append(req)
+            tokens = [drawn] if isinstance(drawn, int) else list(drawn)
+            if len(tokens) != step.repeat:
+                raise ValueError(f"request {req.id}: the step ran {step.repeat} times but {len(tokens)} tokens came back")
+            for token in tokens:
+                # the run that drew this token wrote the position(s) before it; what the device ran
+                # past a request's end is dropped with its pages
+                self.manager.commit(req.id, seq.num_tokens, req.tokens)
+                req.append_output_token(int(token))
+                if req.first_token_time is None:
+                    req.first_token_time = now
+                sp = req.sampling_params
+                reason = None
+                if token in self.eos_token_ids and not sp.ignore_eos:
+                    reason = "stop"
+                elif req.num_completion_tokens >= sp.max_tokens:
+                    reason = "length"
+                elif len(req.tokens) >= self.max_model_len:
+                    reason = "length"
+                if reason is not None:
+                    req.state = RequestState.FINISHED
+                    req.finish_reason = reason
+                    req.finish_time = now
+                    self.manager.release(req.id)
+                    self.running.remove(req)
+                    done.append(req)
+                    break
         return done

@@ -36,6 +36,14 @@ class Sampler:
         self.device = device
         self._out = torch.empty(1024, dtype=torch.int32, device=device)
 
+    @staticmethod
+    def arrays(params: Sequence[SamplingParams], seeds: Sequence[int], counters: Sequence[int]):
+        """The per-request arrays the kernel reads: temperature, top_k, top_p, seed, counter."""
+        return (np.array([p.temperature for p in params], dtype=np.float32),
+                np.array([p.top_k for p in params], dtype=np.int32),
+                np.array([p.top_p for p in params], dtype=np.float32),
+                np.array(seeds, dtype=np.int64), np.array(counters, dtype=np.int64))
+
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
                counters: Sequence[int]) -> List[int]:
         """``logits`` float32 [M, V] on the device; ``params``, ``seeds`` and ``counters`` (index of

@@ -33,11 +33,11 @@ def expected_output(prompt, max_tokens, ignore_eos=True):
 
 class FakeEngine:
     def __init__(self, num_pages, page_size, groups=None, max_tokens=64, max_seqs=8, chunk=None, prefix=False,
-                 max_model_len=4096):
+                 max_model_len=4096, repeat=1):
         self.groups = groups or [GroupSpec("full", None, (0,))]
         self.manager = CacheManager(self.groups, num_pages, page_size, max_seqs, enable_prefix_caching=prefix)
         self.sched = Scheduler(self.manager, max_tokens, max_seqs, max_model_len, eos_token_ids=(EOS,),
-                               prefill_chunk=chunk)
+                               prefill_chunk=chunk, max_decode_repeat=repeat)
         self.ps = page_size
         self.mem = [dict() for _ in self.groups]          # per group: (page, slot) -> token
         self.steps = []
@@ -50,6 +50,33 @@ class FakeEngine:
         assert len(step.seqs) <= self.sched.max_num_batched_seqs
         assert len({s.request.id for s in step.seqs}) == len(step.seqs)
         sampled = []
+        if step.repeat > 1:
+            # the device's part: every run writes the newest token and draws the next from the cache
+            assert not self.sched.waiting and all(s.is_decode and s.sample for s in step.seqs)
+            for s in step.seqs:
+                r = s.request
+                seq = self.manager.sequence(r.id)
+                assert s.start == seq.num_computed == len(r.tokens) - 1
+                assert r.num_completion_tokens + step.repeat <= r.sampling_params.max_tokens
+                toks, drawn = list(r.tokens), []
+                for j in range(step.repeat):
+                    pos = s.start + j
+                    contexts = []
+                    for g, spec in enumerate(self.groups):
+                        table = seq.pages[g]
+                        assert table[pos // self.ps] >= 0
+                        self.mem[g][(table[pos // self.ps], pos % self.ps)] = toks[pos]
+                        lo = 0 if spec.retention == "full" else max(0, pos - spec.window)
+                        ctx = [self.mem[g][(table[p // self.ps], p % self.ps)] for p in range(lo, pos + 1)]
+                        assert ctx == toks[lo:pos + 1], "the cache does not hold the request's tokens"
+                        contexts.append(ctx)
+                    t = next_token(contexts[0])
+                    toks.append(t); drawn.append(t)
+                sampled.append(drawn)
+            self.steps.append(step)
+            done = self.sched.update(step, sampled)
+            self.manager.check_invariants()
+            return step, done
         for s in step.seqs:
             r = s.request
             seq = self.manager.sequence(r.id)
@@ -223,3 +250,58 @@ def test_max_model_len_ends_a_request():
     r = submit(e, [1, 2, 3, 4, 5], max_tokens=100, ignore_eos=True)
     e.run_all()
     assert len(r.tokens) == 12 and r.finish_reason == "length"
+
+
+def test_decode_steps_run_in_a_row():
+    """Steps of decoded tokens only may run several times before the host looks: same tokens as one
+    by one, never past max_tokens, tokens drawn after an end token are dropped, and a waiting
+    request is admitted at the next step."""
+    rng = random.Random(11)
+    prompts = [[rng.randrange(VOCAB) for _ in range(n)] for n in (5, 17, 9, 2, 30)]
+    limits = [13, 7, 40, 1, 22]
+    for use_eos in (False, True):
+        e = FakeEngine(num_pages=64, page_size=4, max_tokens=32, max_seqs=4, repeat=4)
+        reqs = [submit(e, p, max_tokens=m, ignore_eos=not use_eos) for p, m in zip(prompts[:3], limits[:3])]
+        late = []
+        n = 0
+        while not e.sched.finished:
+            step, _ = e.run_step()
+            n += 1
+            if n == 6:                                   # arrive while the others decode
+                late = [submit(e, p, max_tokens=m, ignore_eos=not use_eos) for p, m in zip(prompts[3:], limits[3:])]
+                assert e.sched.schedule is not None
+            assert n < 1000
+        for r, m in zip(reqs + late, limits):
+            assert r.completion_tokens == expected_output(r.prompt_tokens, m, ignore_eos=not use_eos)
+        repeats = [st.repeat for st in e.steps]
+        assert max(repeats) == 4 and 1 in repeats
+        # the step after the late arrival took them in: nobody waits while steps repeat
+        assert all(st.repeat == 1 or all(s.is_decode for s in st.seqs) for st in e.steps)
+        assert all(p.num_free == p.num_pages for p in e.manager.pools)
+
+
+def test_repeat_shrinks_to_the_free_pages():
+    """With pages for fewer positions than asked, the step repeats fewer times; nothing is preempted
+    for the sake of repeating."""
+    e = FakeEngine(num_pages=5, page_size=4, max_tokens=32, max_seqs=4, repeat=8)
+    rng = random.Random(12)
+    a = submit(e, [rng.randrange(VOCAB) for _ in range(7)], max_tokens=12, ignore_eos=True)
+    b = submit(e, [rng.randrange(VOCAB) for _ in range(6)], max_tokens=3, ignore_eos=True)
+    e.run_all()
+    assert a.completion_tokens == expected_output(a.prompt_tokens, 12)
+    assert b.completion_tokens == expected_output(b.prompt_tokens, 3)
+    assert e.sched.num_preemptions == 0
+    assert any(1 < st.repeat < 8 for st in e.steps)
+    assert all(p.num_free == p.num_pages for p in e.manager.pools)
+
+
+def test_repeat_with_a_window_group():
+    groups = [GroupSpec("full", None, (0,)), GroupSpec("window", 6, (1,))]
+    e = FakeEngine(num_pages=48, page_size=4, groups=groups, max_tokens=32, max_seqs=4, repeat=4)
+    rng = random.Random(13)
+    reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=19, ignore_eos=True) for n in (11, 3)]
+    e.run_all()
+    for r in reqs:
+        assert r.completion_tokens == expected_output(r.prompt_tokens, 19)
+    assert max(st.repeat for st in e.steps) == 4
+    assert all(p.num_free == p.num_pages for p in e.manager.pools)
