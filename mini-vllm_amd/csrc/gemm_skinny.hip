@@ -99,6 +99,20 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
         }
         wrow[r] = reinterpret_cast<const uint4*>(W + (size_t)row * K) + g;
     }
+    // k-steps per register stage of the main loop (see there)
+    // (the fused-norm variants serve small steps, where a deeper first stage pays and registers are free)
+    constexpr int FRAGS = NORM ? SK_STAGE_FRAGS + SK_STAGE_FRAGS / 2 : SK_STAGE_FRAGS;
+    constexpr int U = FRAGS / (R + TM) >= 8 ? 8 : (FRAGS / (R + TM) >= 4 ? 4 : (FRAGS / (R + TM) >= 2 ? 2 : 1));
+    const int nfull = (ks1 - ks0) / U;
+    // NORM: the first stage's weights are asked for before the rows are normalised, so that their
+    // way from memory overlaps the prologue
+    Frag wfirst[NORM ? U : 1][R];
+    if (NORM && nfull > 0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int r = 0; r < R; ++r) wfirst[u][r].u = wrow[r][(size_t)(ks0 + u) * 4];
+    }
     const uint4* arow[TM];
     bool avalid[TM];
     if (NORM) {
@@ -202,7 +216,6 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 
     // Two register stages of U k-steps each: while the MFMAs of one stage run, the loads of the
     // next are in flight, so a wave always has a stage's worth of weight bytes on the way.
-    constexpr int U = SK_STAGE_FRAGS / (R + TM) >= 8 ? 8 : (SK_STAGE_FRAGS / (R + TM) >= 4 ? 4 : (SK_STAGE_FRAGS / (R + TM) >= 2 ? 2 : 1));
     struct Stage {
         Frag w[U][R], a[U][TM];
     };
@@ -225,11 +238,21 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
                 for (int t = 0; t < TM; ++t)
                     acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.w[u][r].v, st.a[u][t].v, acc[r][t], 0, 0, 0);
     };
-    const int nfull = (ks1 - ks0) / U;
     int ks = ks0 + nfull * U;
     if (nfull > 0) {
         Stage s0, s1;
-        fetch(s0, ks0);
+        if (NORM) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) s0.w[u][r] = wfirst[u][r];
+#pragma unroll
+                for (int t = 0; t < TM; ++t)
+                    s0.a[u][t].u = avalid[t] ? arow[t][(size_t)(ks0 + u) * 4] : uint4{0u, 0u, 0u, 0u};
+            }
+        } else {
+            fetch(s0, ks0);
+        }
         int it = 0;
         for (; it + 2 <= nfull; it += 2) {
             fetch(s1, ks0 + (it + 1) * U);
