@@ -149,20 +149,27 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     const int tpu = COLS / G;  // tokens of a unit (the host made sure it is >= 1)
 
     __shared__ int sh_unit[3];
-    if (threadIdx.x == 0) {
-        int seq = -1, t0 = 0, nt = 0;
+    int seq, t0, nt;
+    if (FUSED) {
+        // a decode step: row t of the step is the one token of sequence t (or padding)
         seq = blockIdx.x;
-        t0 = cu_seqlens[seq];
-        nt = cu_seqlens[seq + 1] - t0;
-        if (nt > tpu) nt = tpu;
-        if (FUSED && nt > 1) nt = 1;   // decode steps: one token a sequence
-        if (FUSED && nt == 1 && fz.token_seq[t0] < 0) nt = 0;
-        sh_unit[0] = seq;
-        sh_unit[1] = t0;
-        sh_unit[2] = nt;
+        t0 = seq;
+        nt = fz.token_seq[t0] >= 0 ? 1 : 0;
+    } else {
+        if (threadIdx.x == 0) {
+            const int s0 = blockIdx.x;
+            const int first = cu_seqlens[s0];
+            int count = cu_seqlens[s0 + 1] - first;
+            if (count > tpu) count = tpu;
+            sh_unit[0] = s0;
+            sh_unit[1] = first;
+            sh_unit[2] = count;
+        }
+        __syncthreads();
+        seq = sh_unit[0];
+        t0 = sh_unit[1];
+        nt = sh_unit[2];
     }
-    __syncthreads();
-    const int seq = sh_unit[0], t0 = sh_unit[1], nt = sh_unit[2];
     if (seq < 0 || nt <= 0) return;
     const int ncols = nt * G;
     const int* bt = block_table + (size_t)seq * bt_width;
@@ -178,7 +185,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         col_ok[ct] = col < ncols;
         col_tok[ct] = t0 + (col_ok[ct] ? col / G : 0);
         col_head[ct] = kvh * G + (col_ok[ct] ? col % G : 0);
-        col_pos[ct] = col_ok[ct] ? positions[col_tok[ct]] : -1;
+        col_pos[ct] = col_ok[ct] ? positions[FUSED ? t0 : col_tok[ct]] : -1;   // FUSED: one token, one position
         col_lo[ct] = (window >= 0 && col_pos[ct] - window > 0) ? col_pos[ct] - window : 0;
         if (col_ok[ct]) {
             hi_w = col_pos[ct] > hi_w ? col_pos[ct] : hi_w;
@@ -192,8 +199,13 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         for (int s = 0; s < DS; ++s)
             qop[ct][s].u = col_ok[ct] ? *reinterpret_cast<const uint4*>(qrow + 32 * s) : uint4{0u, 0u, 0u, 0u};
     }
-    hi_w = wave_max_i(hi_w);
-    lo_w = wave_min_i(lo_w);
+    if (FUSED) {   // known without asking the other lanes
+        hi_w = positions[t0];
+        lo_w = (window >= 0 && hi_w - window > 0) ? hi_w - window : 0;
+    } else {
+        hi_w = wave_max_i(hi_w);
+        lo_w = wave_min_i(lo_w);
+    }
 
     float m_run[NT], l_run[NT];
     floatx4_t acc_o[NT][DT];
