@@ -51,7 +51,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     constexpr int KCHUNKS = 2 * DS * 64;       // 16-byte chunks of a K tile
     constexpr int VCHUNKS = DT * 64;           // 16-byte chunks of a V tile (two 8-byte halves each)
     constexpr int KREP = KCHUNKS / AP_THREADS;
-    constexpr int VREP = 2 * VCHUNKS / AP_THREADS / 2;  // 16-byte global loads per thread
+    constexpr int VREP = 2 * VCHUNKS / AP_THREADS;      // 8-byte chunks of a V tile pair per thread
     static_assert(KCHUNKS % AP_THREADS == 0 && (D * 2 * 2) % AP_THREADS == 0, "tile does not divide the workgroup");
 
     __shared__ uint4 sK[2][KCHUNKS];
@@ -152,31 +152,31 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     // Two blocks are in flight: while block b is computed, block b+1 waits in one register set
     // and block b+2 is being loaded into the other. Everything that does not depend on the block
     // (which chunk of the tile a thread copies, where it goes in LDS) is worked out once.
+    // A thread copies the chunks whose place in LDS follows its id, so that the LDS writes of a wave
+    // are consecutive (no bank conflicts); the matching global reads touch, per instruction, 64
+    // contiguous bytes of 16 key rows (K) or the contiguous slots of a page's rows (V).
     struct Staged {
         uint4 k[KREP];
-        uint4 v[VREP];
+        uint2 v[VREP];
     };
     int k_tile[KREP], k_off[KREP], k_lds[KREP];
 #pragma unroll
     for (int rep = 0; rep < KREP; ++rep) {
-        const int r = tid + AP_THREADS * rep;
-        const int key = r / (D / 8);  // 0..31
-        const int dchunk = r % (D / 8);
-        k_tile[rep] = key / 16;
-        k_off[rep] = (key % 16) * D + 8 * dchunk;
-        k_lds[rep] = (k_tile[rep] * DS + dchunk / 4) * 64 + key % 16 + 16 * (dchunk % 4);
+        const int L = tid + AP_THREADS * rep;          // LDS chunk: ((tile * DS + s) * 64 + operand lane)
+        const int ol = L % 64;
+        k_tile[rep] = L / (DS * 64);
+        k_off[rep] = (ol % 16) * D + 32 * ((L / 64) % DS) + 8 * (ol / 16);
+        k_lds[rep] = L;
     }
     int v_tile[VREP], v_off[VREP], v_lds[VREP], v_key[VREP];
 #pragma unroll
     for (int rep = 0; rep < VREP; ++rep) {
-        const int r = tid + AP_THREADS * rep;
-        const int d = (r % (D * 2)) / 2;  // D * 2 sixteen-byte chunks per 16-key tile
-        const int hq = r % 2;
-        v_tile[rep] = r / (D * 2);
-        v_off[rep] = d * page_size + 8 * hq;
-        v_key[rep] = 16 * v_tile[rep] + 8 * hq;
-        // keys 8hq .. 8hq+3 go to lane group 2hq, keys 8hq+4 .. 8hq+7 to lane group 2hq+1 (32 further)
-        v_lds[rep] = ((d / 16) * 64 + d % 16 + 16 * (2 * hq)) * 2 + v_tile[rep];
+        const int L = tid + AP_THREADS * rep;          // LDS chunk: ((d tile * 64 + operand lane) * 2 + key tile)
+        const int ol = (L / 2) % 64;
+        v_tile[rep] = L % 2;
+        v_off[rep] = (16 * (L / 128) + ol % 16) * page_size + 4 * (ol / 16);
+        v_key[rep] = 16 * v_tile[rep] + 4 * (ol / 16);
+        v_lds[rep] = L;
     }
     const int page_mask = page_size - 1;
     auto fetch = [&](int b, Staged& st) {
@@ -202,14 +202,14 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
             st.k[rep] = *reinterpret_cast<const uint4*>((k_tile[rep] ? kbase[1] : kbase[0]) + k_off[rep]);
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep)
-            st.v[rep] = *reinterpret_cast<const uint4*>((v_tile[rep] ? vbase[1] : vbase[0]) + v_off[rep]);
+            st.v[rep] = *reinterpret_cast<const uint2*>((v_tile[rep] ? vbase[1] : vbase[0]) + v_off[rep]);
         if (gone[0] || gone[1]) {
 #pragma unroll
             for (int rep = 0; rep < KREP; ++rep)
                 if (gone[k_tile[rep]]) st.k[rep] = uint4{0u, 0u, 0u, 0u};
 #pragma unroll
             for (int rep = 0; rep < VREP; ++rep)
-                if (gone[v_tile[rep]]) st.v[rep] = uint4{0u, 0u, 0u, 0u};
+                if (gone[v_tile[rep]]) st.v[rep] = uint2{0u, 0u};
         }
     };
     auto stash = [&](int b, const Staged& st) {
@@ -219,14 +219,15 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         const bool tail = 32 * b + 31 > hi_g;  // slots above the newest key were never written
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep) {
-            Frag f;
-            f.u = st.v[rep];
+            uint2 f = st.v[rep];
             if (tail) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) f.s[e] = (32 * b + v_key[rep] + e > hi_g) ? (uint16_t)0 : f.s[e];
+                const int key = 32 * b + v_key[rep];
+                if (key > hi_g) f.x = 0;
+                else if (key + 1 > hi_g) f.x &= 0xffffu;
+                if (key + 2 > hi_g) f.y = 0;
+                else if (key + 3 > hi_g) f.y &= 0xffffu;
             }
-            sV[buf][v_lds[rep]] = f.h[0];
-            sV[buf][v_lds[rep] + 32] = f.h[1];
+            sV[buf][v_lds[rep]] = f;
         }
     };
 
