@@ -44,7 +44,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                          const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                          const int* __restrict__ block_table, int bt_width, int page_size, int page_shift,
                          const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs, int H,
-                         int Hkv, float scale, int window) {
+                         int Hkv, float scale, int window, int fold) {
     constexpr int DS = D / 32;                 // k-steps of the score product
     constexpr int DT = D / 16;                 // d tiles of the output product
     constexpr int COLS = 16 * AP_WAVES * NT;   // columns of a workgroup
@@ -72,7 +72,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
 
     if (tid == 0) {
         int seq = -1, t0 = 0, nt = 0;
-        int u = gridDim.y - 1 - blockIdx.y;  // units with the most keys start first
+        // Units with the most keys start first. When the whole grid is resident at once (two
+        // workgroups a compute unit, dealt out in order), the second half of the grid runs from
+        // the lightest unit upwards instead, so that the two workgroups that share a compute unit
+        // bring about the same number of key blocks together.
+        const int n_all = gridDim.y, half = (n_all + 1) / 2;
+        int u = (!fold || (int)blockIdx.y < half) ? n_all - 1 - (int)blockIdx.y : (int)blockIdx.y - half;
         for (int s = 0; s < n_seqs; ++s) {
             const int ql = cu_seqlens[s + 1] - cu_seqlens[s];
             const int nu = (ql + tpu - 1) / tpu;
@@ -392,10 +397,10 @@ template <int D, int NT>
 static void launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
                            const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                            int page_size, int page_shift, const int* positions, const int* cu_seqlens, int n_seqs,
-                           int H, int Hkv, float scale, int window) {
+                           int H, int Hkv, float scale, int window, int fold) {
     hipLaunchKernelGGL((attention_prefill_kernel<D, NT>), grid, dim3(AP_THREADS), 0, stream, (const bf16*)q, q_stride,
                        (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,
-                       page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window);
+                       page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold);
 }
 
 // nt: column tiles per wave (2 = 128 columns per workgroup, for long prompts; 1 = 64 columns, twice
@@ -420,9 +425,14 @@ extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, lon
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
     dim3 grid(Hkv, n_units, 1);
+    // everything resident at once: two workgroups for each of the device's compute units
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        cus = 256;
+    const int fold = (long)Hkv * n_units <= 2L * cus ? 1 : 0;
 #define AP_LAUNCH(DD, NN)                                                                                          \
     launch_prefill<DD, NN>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,      \
-                           page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window)
+                           page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold)
     if (D == 128 && nt == 2) AP_LAUNCH(128, 2);
     else if (D == 128) AP_LAUNCH(128, 1);
     else if (nt == 2) AP_LAUNCH(64, 2);
