@@ -18,6 +18,11 @@
 // Online softmax (base 2) per column. A wave skips blocks that lie outside the range of all its
 // columns. Value slots above the unit's newest key were never written and are copied as zero.
 //
+// With KW = 2 the workgroup has eight waves: two groups of four that serve the same columns and
+// take the key blocks in turn (group 0 the even ones of the unit's range, group 1 the odd ones),
+// each with LDS tiles of its own, and merge their partial results through LDS at the end. The
+// walk of a unit with many keys takes half as many rounds.
+//
 // Layouts: K[page][kv_head][slot][d], V[page][kv_head][d][slot]; page size a multiple of 16.
 #include "common.h"
 
@@ -38,8 +43,8 @@ union Frag {
 // Two workgroups share a compute unit (LDS and latency hiding are sized for that), so a wave may
 // use half of a SIMD's registers: the accumulators stay in the vector registers and the operand
 // reads from LDS run ahead of the MFMAs.
-template <int D, int NT>
-__global__ void __launch_bounds__(AP_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int D, int NT, int KW>
+__global__ void __launch_bounds__(AP_THREADS * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                          const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                          const int* __restrict__ block_table, int bt_width, int page_size, int page_shift,
@@ -54,10 +59,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     constexpr int VREP = 2 * VCHUNKS / AP_THREADS;      // 8-byte chunks of a V tile pair per thread
     static_assert(KCHUNKS % AP_THREADS == 0 && (D * 2 * 2) % AP_THREADS == 0, "tile does not divide the workgroup");
 
-    __shared__ uint4 sK[2][KCHUNKS];
-    __shared__ uint2 sV[2][VCHUNKS * 2];
+    // [buffer][key group] tiles: K as 16-byte chunks, then V as 8-byte chunks
+    extern __shared__ uint4 lds_tiles[];
+    uint4* const sK_all = lds_tiles;
+    uint2* const sV_all = reinterpret_cast<uint2*>(lds_tiles + 2 * KW * KCHUNKS);
     __shared__ int sh_unit[3];
-    __shared__ int sh_range[2][AP_WAVES];
+    __shared__ int sh_range[2][AP_WAVES * KW];
 
     const int G = H / Hkv;
     // the key/value head is the fastest grid dimension: workgroups are dealt to the eight XCDs in
@@ -66,6 +73,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     const int tid = threadIdx.x;
     const int wave = tid / MV_WAVE;
     const int lane = tid % MV_WAVE;
+    const int cw = wave % AP_WAVES;            // which columns of the unit
+    const int kg = wave / AP_WAVES;            // which of the KW key groups
+    const int gtid = tid % AP_THREADS;         // thread within its key group
     const int i = lane % 16;
     const int g = lane / 16;
     const int tpu = COLS / G;  // tokens of a unit (the host made sure it is >= 1)
@@ -107,7 +117,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     int hi_w = -1, lo_w = 0x7fffffff;
 #pragma unroll
     for (int ct = 0; ct < NT; ++ct) {
-        const int col = (wave * NT + ct) * 16 + i;
+        const int col = (cw * NT + ct) * 16 + i;
         col_ok[ct] = col < ncols;
         col_tok[ct] = t0 + (col_ok[ct] ? col / G : 0);
         col_head[ct] = kvh * G + (col_ok[ct] ? col % G : 0);
@@ -135,7 +145,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     __syncthreads();
     int hi_g = -1, lo_g = 0x7fffffff;
 #pragma unroll
-    for (int w = 0; w < AP_WAVES; ++w) {
+    for (int w = 0; w < AP_WAVES * KW; ++w) {
         hi_g = sh_range[0][w] > hi_g ? sh_range[0][w] : hi_g;
         lo_g = sh_range[1][w] < lo_g ? sh_range[1][w] : lo_g;
     }
@@ -167,7 +177,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     int k_tile[KREP], k_off[KREP], k_lds[KREP];
 #pragma unroll
     for (int rep = 0; rep < KREP; ++rep) {
-        const int L = tid + AP_THREADS * rep;          // LDS chunk: ((tile * DS + s) * 64 + operand lane)
+        const int L = gtid + AP_THREADS * rep;         // LDS chunk: ((tile * DS + s) * 64 + operand lane)
         const int ol = L % 64;
         k_tile[rep] = L / (DS * 64);
         k_off[rep] = (ol % 16) * D + 32 * ((L / 64) % DS) + 8 * (ol / 16);
@@ -176,7 +186,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     int v_tile[VREP], v_off[VREP], v_lds[VREP], v_key[VREP];
 #pragma unroll
     for (int rep = 0; rep < VREP; ++rep) {
-        const int L = tid + AP_THREADS * rep;          // LDS chunk: ((d tile * 64 + operand lane) * 2 + key tile)
+        const int L = gtid + AP_THREADS * rep;         // LDS chunk: ((d tile * 64 + operand lane) * 2 + key tile)
         const int ol = (L / 2) % 64;
         v_tile[rep] = L % 2;
         v_off[rep] = (16 * (L / 128) + ol % 16) * page_size + 4 * (ol / 16);
@@ -185,7 +195,13 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     }
     const int page_mask = page_size - 1;
     auto fetch = [&](int b, Staged& st) {
-        if (b > b1) return;
+        if (b > b1) {   // past the unit's range: nothing to read (the block is not computed either)
+#pragma unroll
+            for (int rep = 0; rep < KREP; ++rep) st.k[rep] = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int rep = 0; rep < VREP; ++rep) st.v[rep] = uint2{0u, 0u};
+            return;
+        }
         const bf16* kbase[2];
         const bf16* vbase[2];
         bool gone[2];
@@ -217,10 +233,14 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 if (gone[v_tile[rep]]) st.v[rep] = uint2{0u, 0u};
         }
     };
-    auto stash = [&](int b, const Staged& st) {
-        const int buf = (b - b0) & 1;
+    // round j of the walk: key group kg has block b0 + j * KW + kg, in the tiles [j & 1][kg]
+    auto block_of = [&](int j) { return b0 + j * KW + kg; };
+    auto stash = [&](int j, const Staged& st) {
+        const int b = block_of(j);
+        uint4* sK = sK_all + ((j & 1) * KW + kg) * KCHUNKS;
+        uint2* sV = sV_all + ((j & 1) * KW + kg) * (VCHUNKS * 2);
 #pragma unroll
-        for (int rep = 0; rep < KREP; ++rep) sK[buf][k_lds[rep]] = st.k[rep];
+        for (int rep = 0; rep < KREP; ++rep) sK[k_lds[rep]] = st.k[rep];
         const bool tail = 32 * b + 31 > hi_g;  // slots above the newest key were never written
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep) {
@@ -232,7 +252,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 if (key + 2 > hi_g) f.y = 0;
                 else if (key + 3 > hi_g) f.y &= 0xffffu;
             }
-            sV[buf][v_lds[rep]] = f;
+            sV[v_lds[rep]] = f;
         }
     };
 
@@ -257,10 +277,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     for (int ct = 0; ct < NT; ++ct) all_cols = all_cols && col_ok[ct];
     const bool wave_full = __all(all_cols);
 
-    auto compute = [&](int b) {
-        const int cur = (b - b0) & 1;
+    auto compute = [&](int j) {
+        const int b = block_of(j);
+        const uint4* sK = sK_all + ((j & 1) * KW + kg) * KCHUNKS;
+        const uint2* sV = sV_all + ((j & 1) * KW + kg) * (VCHUNKS * 2);
         const int base = 32 * b;
-        if (!(base <= hi_w && base + 31 >= lo_w)) return;
+        if (b > b1 || !(base <= hi_w && base + 31 >= lo_w)) return;
         const bool masked = !(wave_full && base + 31 <= full_hi && base >= full_lo);
         // scores^T for the two 16-key tiles
         float p[NT][2][4];
@@ -268,13 +290,13 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int s = 0; s < DS; ++s) kop[t][s].u = sK[cur][(t * DS + s) * 64 + lane];
+            for (int s = 0; s < DS; ++s) kop[t][s].u = sK[(t * DS + s) * 64 + lane];
         // the value operands are asked for now and arrive while the softmax is worked out
         Frag vop[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            vop[dt].h[0] = sV[cur][(dt * 64 + lane) * 2];
-            vop[dt].h[1] = sV[cur][(dt * 64 + lane) * 2 + 1];
+            vop[dt].h[0] = sV[(dt * 64 + lane) * 2];
+            vop[dt].h[1] = sV[(dt * 64 + lane) * 2 + 1];
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -347,21 +369,22 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
     };
 
+    const int rounds = (b1 - b0 + KW) / KW;    // the same for every wave: they meet at the barriers
     Staged sa, sb;
-    fetch(b0, sa);
-    fetch(b0 + 1, sb);
-    stash(b0, sa);
+    fetch(block_of(0), sa);
+    fetch(block_of(1), sb);
+    stash(0, sa);
     __syncthreads();
-    // invariant at the top: LDS holds block b, `sb` holds block b+1 (or zeros past the end)
-    for (int b = b0; b <= b1; b += 2) {
-        fetch(b + 2, sa);
-        compute(b);
-        if (b + 1 <= b1) stash(b + 1, sb);
+    // invariant at the top: LDS holds round j, `sb` holds round j+1 (or zeros past the end)
+    for (int j = 0; j < rounds; j += 2) {
+        fetch(block_of(j + 2), sa);
+        compute(j);
+        if (j + 1 < rounds) stash(j + 1, sb);
         __syncthreads();
-        if (b + 1 > b1) break;
-        fetch(b + 3, sb);
-        compute(b + 1);
-        if (b + 2 <= b1) stash(b + 2, sa);
+        if (j + 1 >= rounds) break;
+        fetch(block_of(j + 3), sb);
+        compute(j + 1);
+        if (j + 2 < rounds) stash(j + 2, sa);
         __syncthreads();
     }
 
@@ -370,6 +393,46 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     for (int ct = 0; ct < NT; ++ct) {
         l_run[ct] += __shfl_xor(l_run[ct], 16, MV_WAVE);
         l_run[ct] += __shfl_xor(l_run[ct], 32, MV_WAVE);
+    }
+
+    if (KW > 1) {
+        // ---- key group 1 hands its partial results to group 0 through LDS (the tiles are no
+        // longer needed: every wave has passed the last barrier of the walk), one column tile at a time
+        float* xo = reinterpret_cast<float*>(lds_tiles);                 // [AP_WAVES][DT][4][64]
+        float* xm = xo + AP_WAVES * DT * 4 * MV_WAVE;                    // [AP_WAVES][16] maxima, then sums
+        float* xl = xm + AP_WAVES * 16;
+#pragma unroll
+        for (int ct = 0; ct < NT; ++ct) {
+            if (ct) __syncthreads();
+            if (kg == 1) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) xo[((cw * DT + dt) * 4 + r) * MV_WAVE + lane] = acc_o[ct][dt][r];
+                if (g == 0) {
+                    xm[cw * 16 + i] = m_run[ct];
+                    xl[cw * 16 + i] = l_run[ct];
+                }
+            }
+            __syncthreads();
+            if (kg == 0) {
+                const float m1 = xm[cw * 16 + i], l1 = xl[cw * 16 + i];
+                const float m_fin = fmaxf(m_run[ct], m1);
+                const float f0 = (m_run[ct] == -INFINITY) ? 0.f : exp2f(m_run[ct] - m_fin);
+                const float f1 = (m1 == -INFINITY) ? 0.f : exp2f(m1 - m_fin);
+                l_run[ct] = f0 * l_run[ct] + f1 * l1;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        acc_o[ct][dt][r] = f0 * acc_o[ct][dt][r] + f1 * xo[((cw * DT + dt) * 4 + r) * MV_WAVE + lane];
+            }
+        }
+        if (kg != 0) return;
+    }
+
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
         if (!col_ok[ct]) continue;
         const float inv = 1.f / l_run[ct];
         bf16* orow = out + (size_t)col_tok[ct] * out_stride + (size_t)col_head[ct] * D;
@@ -385,31 +448,41 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     }
 }
 
-// How many query tokens one workgroup serves with `nt` (1 or 2) column tiles per wave, for `group`
-// query heads per key/value head; 0 if the kernel does not take this combination.
 extern "C" int mv_attention_prefill_unit_tokens(int group, int nt) {
     if (nt != 1 && nt != 2) return 0;
     const int cols = 16 * AP_WAVES * nt;
     return group > 0 && group <= cols ? cols / group : 0;
 }
 
-template <int D, int NT>
-static void launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
-                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
-                           int page_size, int page_shift, const int* positions, const int* cu_seqlens, int n_seqs,
-                           int H, int Hkv, float scale, int window, int fold) {
-    hipLaunchKernelGGL((attention_prefill_kernel<D, NT>), grid, dim3(AP_THREADS), 0, stream, (const bf16*)q, q_stride,
-                       (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,
-                       page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold);
+template <int D, int NT, int KW>
+static int launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
+                          const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
+                          int page_size, int page_shift, const int* positions, const int* cu_seqlens, int n_seqs,
+                          int H, int Hkv, float scale, int window, int fold) {
+    // K and V tiles of 32 keys, double-buffered, one set per key group
+    const size_t lds = (size_t)2 * KW * (2 * (D / 32) * 64 * 16 + (D / 16) * 64 * 16);
+    static bool allowed = false;   // more than 64 KiB of LDS has to be asked for, once per kernel
+    if (!allowed && lds > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, NT, KW>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return mv_fail("attention_prefill: %zu bytes of LDS were refused: %s", lds, hipGetErrorString(e));
+        allowed = true;
+    }
+    hipLaunchKernelGGL((attention_prefill_kernel<D, NT, KW>), grid, dim3(AP_THREADS * KW), lds, stream, (const bf16*)q,
+                       q_stride, (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table,
+                       bt_width, page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold);
+    return 0;
 }
 
 // nt: column tiles per wave (2 = 128 columns per workgroup, for long prompts; 1 = 64 columns, twice
 // the workgroups, for steps too small to fill the chip otherwise).
+// kw: key groups per workgroup (2: eight waves, the walk over a unit's keys takes half as many rounds).
 // n_units = sum over sequences of ceil(q_len / unit tokens(group, nt)). grid = (kv heads, units).
 extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_table, int bt_width, int page_size,
                                     const int* positions, const int* cu_seqlens, int n_seqs, int n_units, int nt,
-                                    int H, int Hkv, int D, float scale, int window, hipStream_t stream) {
+                                    int kw, int H, int Hkv, int D, float scale, int window, hipStream_t stream) {
+    MV_REQUIRE(kw == 1 || kw == 2, "attention_prefill: %d key groups per workgroup (1 or 2)", kw);
     MV_REQUIRE(H > 0 && Hkv > 0 && H % Hkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", H,
                Hkv);
     MV_REQUIRE(D == 64 || D == 128, "attention_prefill: head_dim %d is not served by the MFMA kernel (64 or 128)", D);
@@ -429,14 +502,24 @@ extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, lon
     int cus = 0, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
         cus = 256;
-    const int fold = (long)Hkv * n_units <= 2L * cus ? 1 : 0;
-#define AP_LAUNCH(DD, NN)                                                                                          \
-    launch_prefill<DD, NN>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,      \
-                           page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold)
-    if (D == 128 && nt == 2) AP_LAUNCH(128, 2);
-    else if (D == 128) AP_LAUNCH(128, 1);
-    else if (nt == 2) AP_LAUNCH(64, 2);
-    else AP_LAUNCH(64, 1);
+    const int fold = (kw == 1 && (long)Hkv * n_units <= 2L * cus) ? 1 : 0;
+    int rc = 0;
+#define AP_LAUNCH(DD, NN, KK)                                                                                      \
+    rc = launch_prefill<DD, NN, KK>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,       \
+                                    bt_width, page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale,  \
+                                    window, fold)
+    if (kw == 2) {
+        if (D == 128 && nt == 2) AP_LAUNCH(128, 2, 2);
+        else if (D == 128) AP_LAUNCH(128, 1, 2);
+        else if (nt == 2) AP_LAUNCH(64, 2, 2);
+        else AP_LAUNCH(64, 1, 2);
+    } else {
+        if (D == 128 && nt == 2) AP_LAUNCH(128, 2, 1);
+        else if (D == 128) AP_LAUNCH(128, 1, 1);
+        else if (nt == 2) AP_LAUNCH(64, 2, 1);
+        else AP_LAUNCH(64, 1, 1);
+    }
 #undef AP_LAUNCH
+    if (rc) return rc;
     return mv_check_launch("attention_prefill");
 }

@@ -26,6 +26,8 @@ SAMPLE_CHUNKS = 32
 SAMPLE_WORK_ROWS = 1024
 # compute units of the device the launch heuristics are tuned for
 COMPUTE_UNITS = 256
+# context length from which the prompt attention uses two key groups per workgroup
+PREFILL_TWO_GROUPS_FROM = 1024
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
 # from this many tokens on, value rows are written to their pages by a kernel of their own
@@ -488,10 +490,14 @@ class Ops:
                 break
         if nt == 0:
             return False
+        # two key groups per workgroup (eight waves) halve the walk over long contexts; they pay while
+        # the grid leaves compute units waiting for the longest walk (measured on MI355X: faster up
+        # to two workgroups per compute unit, slower beyond)
+        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_units * Hkv <= 2 * COMPUTE_UNITS else 1
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
-                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, nt, H, Hkv, D, float(scale),
-                      window, self._stream())
+                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, nt, kw, H, Hkv, D,
+                      float(scale), window, self._stream())
         return True
 
     # ------------------------------------------------------------------------------------

@@ -344,6 +344,57 @@ def test_attention_general(dtype, with_plan, H, Hkv, D, ps, window):
     assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= tol
 
 
+@pytest.mark.parametrize("H,Hkv,D,ps,window", [(4, 2, 128, 16, None), (8, 2, 64, 32, 300), (8, 1, 128, 16, None)])
+def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window):
+    """Prompt portions over more than a thousand keys (the MFMA kernel then walks the keys with two
+    wave groups per workgroup and merges them): a whole long prompt, a late portion of another, and
+    a single token, with a far key (or the one at the window's edge) made to stand out."""
+    ops = ops_for(torch.bfloat16)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(61)
+    ctx_lens = [1203, 1170, 1050]
+    q_lens = [1203, 70, 1]
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    pages_per = [-(-c // ps) for c in ctx_lens]
+    num_pages = sum(pages_per) + 5
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, cur = [], 0
+    for n_p in pages_per:
+        tables.append(perm[cur:cur + n_p]); cur += n_p
+    if window is not None:
+        for s, (c, ql) in enumerate(zip(ctx_lens, q_lens)):
+            for i in range(max(0, (c - ql) - window) // ps):
+                tables[s][i] = -1
+    kp, vp = fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype)
+    bt = torch.full((len(tables), max(pages_per)), -1, dtype=torch.int32)
+    for s, t in enumerate(tables):
+        bt[s, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    positions, token_seq = [], []
+    for s, (c, ql) in enumerate(zip(ctx_lens, q_lens)):
+        positions += list(range(c - ql, c)); token_seq += [s] * ql
+    n = len(positions)
+    positions = torch.tensor(positions, dtype=torch.int32)
+    token_seq = torch.tensor(token_seq, dtype=torch.int32)
+    q = torch.randn(n, H, D, generator=g)
+    for row, s in ((1202, 0), (1203 + 69, 1), (n - 1, 2)):      # the last query of every sequence
+        far = 3 if window is None else ctx_lens[s] - 1 - window
+        q[row] = 6.0 * k_all[s][far].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
+    q = q.to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.full((n, H * D), float("nan"), dtype=dtype, device="cuda")
+    plan = make_plan(q_lens, ctx_lens)
+    assert plan.max_context_len >= 1024
+    ops.attention(dev(q.view(n, H * D)), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale,
+                  window, plan=plan)
+    # the reference for a sample of the rows (every row of the short sequences, a spread of the long one)
+    rows = sorted(set(list(range(0, 1203, 37)) + list(range(1180, n))))
+    want = reference_attention(q[rows].double(), k_all, v_all, positions[rows], token_seq[rows], H, Hkv, scale, window)
+    got = out.float().cpu().view(n, H, D)
+    assert not torch.isnan(got).any()
+    assert rel_err(got[rows].numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+
+
 @pytest.mark.parametrize("H,Hkv,D,ps,window", [(16, 8, 128, 16, None), (8, 1, 128, 32, None), (6, 2, 64, 16, 50),
                                                 (16, 1, 64, 16, None)])
 @pytest.mark.parametrize("max_context", [None, 4096, 40000])
