@@ -29,7 +29,7 @@ ARCH = "gfx950"
 COMMON_SOURCES = ["runtime.hip", "elementwise.hip", "gemm_ref.hip", "attention_ref.hip", "sampling.hip"]
 VARIANT_SOURCES: Dict[str, List[str]] = {
     "f32": COMMON_SOURCES,
-    "bf16": COMMON_SOURCES + ["gemm_skinny.hip", "attention_fast.hip", "attention_prefill.hip"],
+    "bf16": COMMON_SOURCES + ["gemm_skinny.hip", "gemm_mid.hip", "attention_fast.hip", "attention_prefill.hip"],
 }
 VARIANT_DEFINES: Dict[str, List[str]] = {
     "f32": ["-DMV_WITH_F32"],

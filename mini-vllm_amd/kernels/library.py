@@ -53,6 +53,10 @@ _OPTIONAL_SIGNATURES = {
     "mv_gemm_skinny_swiglu": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_skinny_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
                                     c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "mv_gemm_mid_workspace": (c_long, [c_int, c_int, c_int]),
+    # A, lda, W, bias, C, ldc, c_dtype, M, N, K, swiglu, work, work_floats, stream
+    "mv_gemm_mid": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
+                            c_void_p, c_long, c_void_p]),
     "mv_attention_decode": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
                                     c_void_p, c_int, c_int, c_void_p, c_void_p]),

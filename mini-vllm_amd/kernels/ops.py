@@ -17,6 +17,10 @@ _NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
 
 # largest number of rows the weight-streaming product takes in one launch
 SKINNY_MAX_M = 64
+# the kernel that shares activation rows through LDS takes over from this many rows on, for weights
+# of at least this many elements
+MID_MIN_M = 17
+MID_MIN_WEIGHT = 12 * 1024 * 1024
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
@@ -69,6 +73,8 @@ class Ops:
         self.use_library_gemm = dtype == torch.bfloat16
         self.stream_handle: Optional[int] = None
         self._transposed = {}
+        self._mid_work: Optional[torch.Tensor] = None
+        self._mid_retired: list = []
         self._sample_work: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------------------------
@@ -267,6 +273,8 @@ class Ops:
         ldc = out.stride(0) if M > 1 else N
         fast = self.use_fast_kernels and not exact and wcode == DTYPE_BF16
         if fast and K % 32 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.lib.has("mv_gemm_skinny"):
+            if self._gemm_mid(a, lda, w, bias, out, ldc, M, N, K, swiglu=False):
+                return
             if M <= SKINNY_MAX_M or out.dtype == torch.float32 or not self.use_library_gemm:
                 for m0 in range(0, M, SKINNY_MAX_M):
                     m = min(SKINNY_MAX_M, M - m0)
@@ -285,6 +293,27 @@ class Ops:
             return
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
+
+    def _gemm_mid(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                  ldc: int, M: int, N: int, K: int, swiglu: bool) -> bool:
+        """The kernel for 17 to 64 rows against a large weight (activation rows shared through LDS,
+        K split over workgroups); False when the shape is left to the weight-streaming kernel."""
+        if not (MID_MIN_M <= M <= SKINNY_MAX_M and N * K >= MID_MIN_WEIGHT and K % 128 == 0
+                and self.lib.has("mv_gemm_mid")):
+            return False
+        need = int(self.lib.dll.mv_gemm_mid_workspace(M, N, K))
+        if need <= 0:
+            return False
+        if self._mid_work is None or self._mid_work.numel() < need:
+            if torch.cuda.is_current_stream_capturing():
+                return False                                   # no allocation inside a capture
+            if self._mid_work is not None:
+                self._mid_retired.append(self._mid_work)       # captured graphs may hold its address
+            self._mid_work = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=a.device)
+        self.lib.call("mv_gemm_mid", a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(), ldc,
+                      _CODES[out.dtype], M, N, K, int(swiglu), self._mid_work.data_ptr(), self._mid_work.numel(),
+                      self._stream())
+        return True
 
     def can_fuse_norm(self, rows: int, width: int) -> bool:
         """Whether a norm over ``rows`` x ``width`` may be deferred into the next product."""
@@ -337,6 +366,9 @@ class Ops:
         self._act(a, "gemm input"); self._act(out, "swiglu output"); _dev(w_gate_up, "gate_up weight")
         if out.shape != (M, two_i // 2) or out.stride(1) != 1:
             raise KernelLibraryError(f"gemm_swiglu: output {tuple(out.shape)} is not [{M}, {two_i // 2}]")
+        if self._gemm_mid(a, a.stride(0) if M > 1 else K, w_gate_up, None, out, out.stride(0) if M > 1 else two_i // 2,
+                          M, two_i, K, swiglu=True):
+            return True
         self.lib.call("mv_gemm_skinny_swiglu", a.data_ptr(), a.stride(0) if M > 1 else K, w_gate_up.data_ptr(),
                       out.data_ptr(), out.stride(0) if M > 1 else two_i // 2, M, two_i // 2, K, self._stream())
         return True

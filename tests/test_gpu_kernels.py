@@ -567,6 +567,47 @@ def test_gemm_weight_streaming(out_dtype, M, N, K):
     assert rel_err(out_w.cpu().numpy(), want.numpy()) <= 3e-6
 
 
+@pytest.mark.parametrize("M,N,K,swiglu,out_dtype", [
+    (17, 3100, 4096, False, torch.bfloat16), (64, 4096, 3072, False, torch.bfloat16),
+    (40, 6144, 2048, False, torch.float32), (64, 6144, 2048, True, torch.bfloat16),
+    (33, 2 * 1571, 4096, True, torch.bfloat16), (20, 151936 // 4, 1024, False, torch.float32)])
+def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dtype):
+    """17 to 64 rows against a weight of tens of megabytes: the kernel that shares the activation
+    rows through LDS and splits K over workgroups (partial sums added in a fixed order)."""
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(19)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    full = a.double() @ w.double().T
+    ops._mid_work = None
+    if swiglu:
+        I = N // 2
+        want = torch.nn.functional.silu(full[:, :I]) * full[:, I:]
+        out = torch.full((M, I), float("nan"), dtype=out_dtype, device="cuda")
+        assert ops.gemm_swiglu(dev(a), dev(w), out)
+        again = torch.full((1, I), float("nan"), dtype=out_dtype, device="cuda")
+    else:
+        b = torch.randn(N, generator=g).to(torch.bfloat16)
+        want = full + b.double()
+        out = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+        ops.gemm(dev(a), dev(w), out, dev(b))
+    assert ops._mid_work is not None, "the shape was left to another kernel"
+    tol = 3e-6 if out_dtype == torch.float32 else OP_TOL[torch.bfloat16]
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= tol
+    # rows in a wider buffer; a row's result does not depend on the rows around it
+    wide = torch.zeros(M, K + 40, dtype=torch.bfloat16)
+    wide[:, :K] = a
+    half = M // 2 + 1
+    if not swiglu:
+        out_w = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+        ops.gemm(dev(wide)[:, :K], dev(w), out_w, dev(b))
+        assert torch.equal(out_w, out)
+        if half >= 17:                   # fewer rows go to the weight-streaming kernel, which sums in another order
+            out_h = torch.full((half, N), float("nan"), dtype=out_dtype, device="cuda")
+            ops.gemm(dev(a[M - half:]), dev(w), out_h, dev(b))
+            assert torch.equal(out_h, out[M - half:])
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 3072, 1024), (40, 100, 96), (64, 560, 256)])
 def test_gemm_swiglu_fused(M, I, K):
     ops = ops_for(torch.bfloat16)
