@@ -100,6 +100,10 @@ def test_engine_config_and_sampling_params():
         EngineConfig(model="x", dtype="float16")
     with pytest.raises(ValueError):
         EngineConfig(model="x", gpu_memory_utilization=0.0)
+    # ours: decode-only steps may run several times in a row on the device
+    assert ec.num_scheduler_steps >= 1 and EngineConfig(model="x", num_scheduler_steps=1).num_scheduler_steps == 1
+    with pytest.raises(ValueError):
+        EngineConfig(model="x", num_scheduler_steps=0)
     sp = SamplingParams()
     # minivllm/config/sampling.py:4-10
     assert (sp.temperature, sp.max_tokens, sp.ignore_eos, sp.top_k, sp.top_p) == (1.0, 512, False, 0, 1.0)
