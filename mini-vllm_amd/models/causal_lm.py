@@ -45,6 +45,15 @@ def plan_tensors(plan: ModelPlan) -> List[Tuple[TensorLocation, TensorDecl]]:
             out.append((TensorLocation(i, "mixer", name), decl))
         for name, decl in FEED_FORWARDS.get(layer.ffn.kind).tensors(layer.ffn).items():
             out.append((TensorLocation(i, "ffn", name), decl))
+    # a position encoding is shared by every mixer that names the same spec: its tensors (a learned
+    # table, say) belong to the model, under the role "position.<kind>"
+    seen = set()
+    for layer in plan.layers:
+        pspec = getattr(layer.mixer, "position", None)
+        if pspec is not None and pspec not in seen:
+            seen.add(pspec)
+            for name, decl in POSITION_ENCODINGS.get(pspec.kind).tensors(pspec).items():
+                out.append((TensorLocation(None, f"position.{pspec.kind}", name), decl))
     return out
 
 
@@ -91,7 +100,7 @@ class CausalLM:
             if pspec is not None:
                 if pspec not in position_parts:
                     pcls = POSITION_ENCODINGS.get(pspec.kind)
-                    position_parts[pspec] = pcls(pspec, {}, rt)
+                    position_parts[pspec] = pcls(pspec, fetch(None, f"position.{pspec.kind}", pcls.tensors(pspec)), rt)
                 kwargs["position"] = position_parts[pspec]
             mixer = mixer_cls(layer.mixer, fetch(i, "mixer", mixer_cls.tensors(layer.mixer)), rt, **kwargs)
             ffn_cls = FEED_FORWARDS.get(layer.ffn.kind)

@@ -214,3 +214,230 @@ def test_toy_model_with_state_steps_through_the_engine(dtype):
         mgr.release(r)
     mgr.check_invariants()
     assert rel_err(run([("again", reqs["b"])]), want["b"]) <= tol
+
+
+def define_routed_toy():
+    """A second toy architecture: a feed-forward that routes every token to one of four experts,
+    and a position encoding with a learned table of its own that is added to queries and keys."""
+    from minivllm_amd.config.model_config import ModelConfig
+    from minivllm_amd.models.registry import Architecture, register_architecture
+    from minivllm_amd.parts import (AttentionSpec, Call, EmbeddingSpec, FeedForward, HeadSpec, LayerPlan, ModelPlan,
+                                    PartSpec, PositionEncoding, PreNormBlockSpec, RMSNormSpec, RotarySpec, SwiGLUSpec,
+                                    TensorDecl, FEED_FORWARDS, POSITION_ENCODINGS, register_feed_forward,
+                                    register_position_encoding)
+
+    @dataclass(frozen=True)
+    class RoutedSpec(PartSpec):
+        kind: ClassVar[str] = "toy_routed"
+        hidden_size: int = 0
+        experts: int = 0
+        inner: int = 0
+
+    class Routed(FeedForward):
+        """y = p_e (relu(x A_e^T) B_e^T) for the expert e with the largest router logit; p = softmax
+        of the router logits in float32."""
+
+        @classmethod
+        def tensors(cls, spec):
+            return {"router": TensorDecl((spec.experts, spec.hidden_size)),
+                    "a": TensorDecl((spec.experts, spec.inner, spec.hidden_size)),
+                    "b": TensorDecl((spec.experts, spec.hidden_size, spec.inner))}
+
+        def __init__(self, spec, tensors, rt):
+            self.spec, self.t = spec, tensors
+
+        def forward(self, x, ctx):
+            xf = x.float()
+            p = torch.softmax(xf @ self.t["router"].float().T, dim=-1)
+            top = p.argmax(dim=-1)
+            y = torch.zeros_like(xf)
+            for e in range(self.spec.experts):
+                rows = (top == e).nonzero().flatten()
+                if rows.numel():
+                    hid = torch.relu(xf[rows] @ self.t["a"][e].float().T)
+                    y[rows] = p[rows, e:e + 1] * (hid @ self.t["b"][e].float().T)
+            return y.to(x.dtype)
+
+    @dataclass(frozen=True)
+    class LearnedSpec(PartSpec):
+        kind: ClassVar[str] = "toy_learned_positions"
+        positions: int = 0
+        head_dim: int = 0
+
+    class Learned(PositionEncoding):
+        """q and k of position p get table[p] added (every head the same)."""
+
+        @classmethod
+        def tensors(cls, spec):
+            return {"table": TensorDecl((spec.positions, spec.head_dim))}
+
+        def __init__(self, spec, tensors, rt):
+            self.table = tensors["table"]
+
+        def apply(self, q, k, ctx):
+            add = self.table[ctx.positions[:q.shape[0]].long()].to(q.dtype)[:, None, :]
+            q += add
+            if k is not None:
+                k += add
+
+    if RoutedSpec.kind not in FEED_FORWARDS.kinds():
+        register_feed_forward(RoutedSpec.kind, Routed)
+    if LearnedSpec.kind not in POSITION_ENCODINGS.kinds():
+        register_position_encoding(LearnedSpec.kind, Learned)
+
+    @dataclass(frozen=True)
+    class RoutedConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyRoutedLM"
+        vocab_size: int = 61
+        hidden_size: int = 40
+        max_position_embeddings: int = 96
+        dtype: str = "float32"
+
+        @classmethod
+        def from_dict(cls, d, where="config.json"):
+            return cls(vocab_size=d["vocab_size"], hidden_size=d["hidden_size"])
+
+    def plan(cfg):
+        h = cfg.hidden_size
+        norm = RMSNormSpec(size=h, eps=1e-6)
+        learned = LearnedSpec(positions=cfg.max_position_embeddings, head_dim=20)
+        a0 = AttentionSpec(hidden_size=h, num_heads=2, num_kv_heads=2, head_dim=20, scale=20 ** -0.5, qk_norm=False,
+                           position=learned)
+        a1 = AttentionSpec(hidden_size=h, num_heads=2, num_kv_heads=1, head_dim=20, scale=20 ** -0.5, qk_norm=True,
+                           position=RotarySpec(rotary_dim=20, theta=50.0))
+        norms = (("mixer", norm), ("ffn", norm))
+        layers = (LayerPlan(PreNormBlockSpec(), a0, RoutedSpec(hidden_size=h, experts=4, inner=24), norms),
+                  LayerPlan(PreNormBlockSpec(), a1, SwiGLUSpec(hidden_size=h, intermediate_size=56), norms))
+        return ModelPlan(hidden_size=h, vocab_size=cfg.vocab_size, max_positions=cfg.max_position_embeddings,
+                         embedding=EmbeddingSpec(cfg.vocab_size, h), layers=layers, calls=(Call(0), Call(1)),
+                         final_norm=norm, head=HeadSpec(cfg.vocab_size, h, tied=False))
+
+    def tensor_name(cfg, loc):
+        if loc.layer is None:
+            return f"{loc.role}.{loc.name}"
+        return f"layers.{loc.layer}.{loc.role}.{loc.name}"
+
+    arch = Architecture("ToyRoutedLM", RoutedConfig, plan, tensor_name)
+    register_architecture(arch, replace=True)
+    return arch, RoutedConfig()
+
+
+def routed_plain(w: Dict[str, torch.Tensor], tokens):
+    """The routed toy model on a whole sequence in float64."""
+    w = {k: v.double() for k, v in w.items()}
+    n = len(tokens)
+    x = w["embedding.weight"][torch.tensor(tokens)]
+    pos = torch.arange(n)
+    mask = torch.tril(torch.ones(n, n, dtype=torch.bool))
+
+    def norm(v, weight, eps=1e-6):
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * weight
+
+    def attend(q, k, v, groups):
+        out = torch.zeros(n, 2, 20, dtype=torch.float64)
+        for h in range(2):
+            sc = (q[:, h] @ k[:, h // groups].T) * 20 ** -0.5
+            out[:, h] = torch.softmax(sc.masked_fill(~mask, float("-inf")), -1) @ v[:, h // groups]
+        return out.reshape(n, 40)
+
+    # layer 0: learned additive positions, two kv heads, routed feed-forward
+    p = "layers.0."
+    hcur = norm(x, w[p + "norm.mixer.weight"])
+    add = w["position.toy_learned_positions.table"][pos][:, None, :]
+    q = (hcur @ w[p + "mixer.q"].T).view(n, 2, 20) + add
+    k = (hcur @ w[p + "mixer.k"].T).view(n, 2, 20) + add
+    v = (hcur @ w[p + "mixer.v"].T).view(n, 2, 20)
+    x = x + attend(q, k, v, 1) @ w[p + "mixer.o"].T
+    hcur = norm(x, w[p + "norm.ffn.weight"])
+    prob = torch.softmax(hcur @ w[p + "ffn.router"].T, dim=-1)
+    top = prob.argmax(-1)
+    y = torch.zeros_like(hcur)
+    for t in range(n):
+        e = int(top[t])
+        y[t] = prob[t, e] * (torch.relu(hcur[t] @ w[p + "ffn.a"][e].T) @ w[p + "ffn.b"][e].T)
+    x = x + y
+    # layer 1: q/k norm, rotation over the whole head, one kv head, SwiGLU
+    p = "layers.1."
+    hcur = norm(x, w[p + "norm.mixer.weight"])
+    inv = 1.0 / (50.0 ** (torch.arange(0, 20, 2, dtype=torch.float) / 20)).double()
+    ang = pos.double()[:, None] * inv[None, :]
+    c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+    def rope(t):
+        a, b = t[..., :10], t[..., 10:]
+        return torch.cat([a * c - b * s, b * c + a * s], dim=-1)
+
+    q = rope(norm((hcur @ w[p + "mixer.q"].T).view(n, 2, 20), w[p + "mixer.q_norm"]))
+    k = rope(norm((hcur @ w[p + "mixer.k"].T).view(n, 1, 20), w[p + "mixer.k_norm"]))
+    v = (hcur @ w[p + "mixer.v"].T).view(n, 1, 20)
+    x = x + attend(q, k, v, 2) @ w[p + "mixer.o"].T
+    hcur = norm(x, w[p + "norm.ffn.weight"])
+    g, u = hcur @ w[p + "ffn.gate"].T, hcur @ w[p + "ffn.up"].T
+    x = x + (g * torch.sigmoid(g) * u) @ w[p + "ffn.down"].T
+    return (norm(x, w["final_norm.weight"]) @ w["head.weight"].T).numpy(), top.numpy()
+
+
+def test_toy_routed_feed_forward_and_learned_positions():
+    """A routed feed-forward and a position encoding with a tensor of its own, defined here and
+    registered without touching the framework's files, through the executor in float32: whole,
+    in portions beside another request, and token by token."""
+    from minivllm_amd.config import EngineConfig
+    from minivllm_amd.engine.executor import Executor
+    from minivllm_amd.engine.step import SeqStep
+    from minivllm_amd.models import expected_tensors
+    from minivllm_amd.weights import DictSource
+
+    arch, cfg = define_routed_toy()
+    decls = expected_tensors(arch, cfg)
+    assert "position.toy_learned_positions.table" in decls and "layers.0.ffn.router" in decls
+    g = torch.Generator().manual_seed(4)
+    weights = {}
+    for name, decl in decls.items():
+        t = torch.randn(decl.shape, generator=g) * 0.2
+        weights[name] = (t + 1.0) if decl.init == "ones_normal" else t
+    weights["layers.0.ffn.router"] *= 8.0                   # clear routing decisions
+    ex = Executor(EngineConfig(model="", dtype="float32", max_model_len=96, kv_cache_block_size=8,
+                               kv_cache_num_blocks=30, max_num_batched_seqs=4, use_cuda_graph=False),
+                  model=(arch, cfg, DictSource(weights)))
+    mgr = ex.new_cache_manager()
+    rng = np.random.default_rng(1)
+    reqs = {r: [int(t) for t in rng.integers(0, 61, size=n)] for r, n in (("a", 41), ("b", 26))}
+    want, routes = {}, {}
+    for r, t in reqs.items():
+        want[r], routes[r] = routed_plain(weights, t)
+    assert len(set(routes["a"].tolist())) >= 3              # several experts are in use
+
+    def run(entries):
+        seqs = []
+        for rid, toks in entries:
+            if rid not in mgr:
+                mgr.admit(rid)
+            mgr.reserve(rid, len(toks))
+            s = mgr.sequence(rid)
+            seqs.append(SeqStep(toks, s.num_computed, [mgr.block_table(rid, g) for g in range(len(ex.groups))],
+                                s.state_slot, list(range(len(toks)))))
+        out = ex.step(seqs).cpu().numpy()
+        for rid, toks in entries:
+            mgr.commit(rid, len(toks))
+        return out
+
+    for rid, toks in reqs.items():
+        assert rel_err(run([(rid, toks)]), want[rid]) <= 3e-5
+        mgr.release(rid)
+    done = {r: 0 for r in reqs}
+    sizes = [6, 2, 11, 1, 1, 4]
+    k = 0
+    while any(done[r] < len(reqs[r]) for r in reqs):
+        entries = []
+        for r in reqs:
+            if done[r] < len(reqs[r]):
+                n = min(sizes[k % len(sizes)], len(reqs[r]) - done[r]); k += 1
+                entries.append((r, reqs[r][done[r]:done[r] + n]))
+        out = run(entries)
+        row = 0
+        for r, toks in entries:
+            assert rel_err(out[row:row + len(toks)], want[r][done[r]:done[r] + len(toks)]) <= 3e-5, (r, done[r])
+            row += len(toks); done[r] += len(toks)
+    for r in reqs:
+        mgr.release(r)
+    mgr.check_invariants()
