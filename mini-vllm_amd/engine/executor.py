@@ -372,7 +372,7 @@ class Executor:
                         t[s.state_slot].zero_()
         S = len(seqs)
         decode_only = all(len(s.tokens) == 1 for s in seqs)
-        if (self.config.use_cuda_graph and decode_only and S <= GRAPH_BUCKETS[-1]
+        if (self.config.use_cuda_graph and self.model.graph_safe and decode_only and S <= GRAPH_BUCKETS[-1]
                 and all(len(s.want) == 1 for s in seqs)):
             return self._step_graph(seqs)
         arr, off, facts = self._fill(seqs)
@@ -408,7 +408,7 @@ class Executor:
     # a decode step run several times in a row on the device
     # ------------------------------------------------------------------------------------
     def can_repeat(self, num_seqs: int) -> bool:
-        return bool(self.config.use_cuda_graph) and num_seqs <= GRAPH_BUCKETS[-1]
+        return bool(self.config.use_cuda_graph) and self.model.graph_safe and num_seqs <= GRAPH_BUCKETS[-1]
 
     @torch.inference_mode()
     def step_repeated(self, seqs: Sequence[SeqStep], repeat: int, temperature: np.ndarray, top_k: np.ndarray,

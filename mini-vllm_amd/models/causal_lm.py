@@ -87,6 +87,7 @@ class CausalLM:
         self.head_weight = fetch(None, "head", {"weight": None})["weight"]
 
         position_parts: Dict[object, object] = {}
+        self.graph_safe = True          # every part allows its forward to be captured in a graph
         self.blocks = []
         self.mixers = []
         for i, layer in enumerate(plan.layers):
@@ -107,6 +108,8 @@ class CausalLM:
             ffn = ffn_cls(layer.ffn, fetch(i, "ffn", ffn_cls.tensors(layer.ffn)), rt)
             self.mixers.append(mixer)
             self.blocks.append(BLOCKS.get(layer.block.kind)(layer.block, norms, mixer, ffn))
+            parts = [mixer, ffn, kwargs.get("position")] + list(norms.values())
+            self.graph_safe = self.graph_safe and all(getattr(p, "graph_safe", True) for p in parts if p is not None)
 
     # ------------------------------------------------------------------------------------
     def cache_needs(self) -> List[Optional[CacheNeed]]:

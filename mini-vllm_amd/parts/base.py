@@ -226,6 +226,11 @@ class PendingNorm:
 # ---------------------------------------------------------------------------------------
 class Part:
     spec_class: ClassVar[Optional[type]] = None
+    # A part whose ``forward`` only launches device work that depends on the step's sizes may be
+    # captured in a graph and replayed with other data. A part that looks at host-side values of
+    # the step (``ctx.q_lens``, ``ctx.starts``, ``ctx.host_state_slots``) must say False: the
+    # executor then runs every step eagerly.
+    graph_safe: ClassVar[bool] = True
 
     @classmethod
     def tensors(cls, spec) -> Dict[str, TensorDecl]:

@@ -29,6 +29,7 @@ def define_toy():
 
     class RunningMean(Mixer):
         """y_t = W mean(x_0 .. x_t); the running sum lives in the request's state slot."""
+        graph_safe = False            # the loop below follows host-side values of the step
 
         @classmethod
         def tensors(cls, spec):
@@ -165,8 +166,9 @@ def test_toy_model_with_state_steps_through_the_engine(dtype):
         t = torch.randn(decl.shape, generator=g) * 0.1
         weights[name] = (t + 1.0) if decl.init == "ones_normal" else t
     ex = Executor(EngineConfig(model="", dtype=dtype, max_model_len=128, kv_cache_block_size=8,
-                               kv_cache_num_blocks=24, max_num_batched_seqs=4, use_cuda_graph=False),
+                               kv_cache_num_blocks=24, max_num_batched_seqs=4),
                   model=(arch, cfg, DictSource(weights)))
+    assert not ex.model.graph_safe and not ex.can_repeat(1)     # the toy mixer forbids graphs: every step is eager
     assert ex.has_state and len(ex.groups) == 1 and ex.groups[0].calls == (0, 2)      # calls 0 and 2 keep caches
     assert sorted(ex.state_tensors) == [1] and sorted(ex.kv_pages) == [0, 2]
     mgr = ex.new_cache_manager(enable_prefix_caching=True)
