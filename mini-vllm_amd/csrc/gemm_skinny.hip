@@ -1,5 +1,5 @@
 // Weight-streaming matrix product for few rows (decode steps, the output head):
-//     C[M, N] = A[M, K] * W[N, K]^T (+ bias),   M <= 64, bf16 inputs, float accumulation,
+//     C[M, N] = A[M, K] * W[N, K]^T (+ bias),   M <= 512, bf16 inputs, float accumulation,
 // on the MFMA units of gfx950 (v_mfma_f32_16x16x32_bf16). Each weight is read from HBM exactly
 // once; the few activation rows come from cache.
 //
@@ -24,6 +24,7 @@ union Frag {
 };
 
 #define SK_MAX_WAVES 8
+#define SK_MAX_ROWS 512      // up to 64 rows per workgroup, more rows are dealt out to groups of workgroups
 #define SK_COMPUTE_UNITS 256
 #ifndef SK_STAGE_FRAGS
 #define SK_STAGE_FRAGS 8    // 16-byte operand loads per lane in one register stage of the main loop
@@ -378,10 +379,10 @@ static int dispatch_tm(const void* A, long lda, const void* W, const void* bias,
     // R + TM operand rows of 16 per workgroup it runs; the choice with the least per unit wins.
     const int tiles_m = (M + 15) / 16;
     const int blocks = skinny_blocks(N, R, SWIGLU);
-    int best_tm = tiles_m;
+    int best_tm = tiles_m < 4 ? tiles_m : 4;
     long best_cost = -1;
-    for (int tm = tiles_m; tm >= 1; --tm) {
-        if (tm == 3 && tiles_m == 4) continue;   // 3 + 1 wastes a workgroup
+    for (int tm = best_tm; tm >= 1; --tm) {
+        if (tm == 3 && tiles_m % 3 == 1) continue;   // a last group of one tile wastes a workgroup
         const int groups = (tiles_m + tm - 1) / tm;
         const long cost = (((long)blocks * groups + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS) * (R + tm);
         if (best_cost < 0 || cost < best_cost) {
@@ -397,7 +398,7 @@ static int dispatch_tm(const void* A, long lda, const void* W, const void* bias,
 }
 
 static int check_skinny(const char* what, const void* A, long lda, const void* W, long ldc, int M, int N, int K) {
-    MV_REQUIRE(M >= 0 && M <= 64, "%s: takes at most 64 rows, got M=%d", what, M);
+    MV_REQUIRE(M >= 0 && M <= SK_MAX_ROWS, "%s: takes at most %d rows, got M=%d", what, SK_MAX_ROWS, M);
     MV_REQUIRE(N > 0 && K > 0 && K % 32 == 0, "%s: K=%d must be a positive multiple of 32 (N=%d)", what, K, N);
     MV_REQUIRE(lda >= K && lda % 8 == 0, "%s: lda=%ld must be a multiple of 8 and at least K=%d", what, lda, K);
     MV_REQUIRE(ldc >= N, "%s: ldc=%ld smaller than N=%d", what, ldc, N);

@@ -17,6 +17,8 @@ _NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
 
 # largest number of rows the weight-streaming product takes in one launch
 SKINNY_MAX_M = 64
+# most rows of one launch of it
+SKINNY_LAUNCH_ROWS = 512
 # the kernel that shares activation rows through LDS takes over from this many rows on, for weights
 # of at least this many elements
 MID_MIN_M = 17
@@ -276,8 +278,9 @@ class Ops:
             if self._gemm_mid(a, lda, w, bias, out, ldc, M, N, K, swiglu=False):
                 return
             if M <= SKINNY_MAX_M or out.dtype == torch.float32 or not self.use_library_gemm:
-                for m0 in range(0, M, SKINNY_MAX_M):
-                    m = min(SKINNY_MAX_M, M - m0)
+                # more rows than one workgroup takes are dealt out to groups of workgroups by the kernel
+                for m0 in range(0, M, SKINNY_LAUNCH_ROWS):
+                    m = min(SKINNY_LAUNCH_ROWS, M - m0)
                     self.lib.call("mv_gemm_skinny", a.data_ptr() + m0 * lda * 2, lda, w.data_ptr(), K, _ptr(bias),
                                   out.data_ptr() + m0 * ldc * out.element_size(), ldc, _CODES[out.dtype], m, N, K,
                                   self._stream())
@@ -359,7 +362,9 @@ class Ops:
             return False
         M, K = a.shape
         two_i = w_gate_up.shape[0]
-        if (M > SKINNY_MAX_M or M == 0 or w_gate_up.dtype != torch.bfloat16 or K % 32 or two_i % 2
+        # with the library's product at hand, more rows than one workgroup takes go there
+        if (M > (SKINNY_MAX_M if self.use_library_gemm else SKINNY_LAUNCH_ROWS) or M == 0
+                or w_gate_up.dtype != torch.bfloat16 or K % 32 or two_i % 2
                 or a.stride(1) != 1 or (M > 1 and a.stride(0) % 8) or a.data_ptr() % 16
                 or not w_gate_up.is_contiguous() or w_gate_up.shape[1] != K):
             return False

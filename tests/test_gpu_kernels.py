@@ -608,6 +608,33 @@ def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dt
             assert torch.equal(out_h, out[M - half:])
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 1024, 2048), (200, 333, 1024), (256, 4096, 1024), (130, 1024, 3072)])
+def test_gemm_weight_streaming_many_rows(M, N, K):
+    """Inside captured graphs the library's product is not used: the weight-streaming kernel deals
+    more than 64 rows out to groups of workgroups, also in the gated form."""
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(23)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    want = a.double() @ w.double().T + b.double()
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    library = ops.use_library_gemm
+    ops.use_library_gemm = False
+    try:
+        ops.gemm(dev(a), dev(w), out, dev(b))
+        assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[torch.bfloat16]
+        if N % 2 == 0:
+            I = N // 2
+            full = a.double() @ w.double().T
+            gated = torch.nn.functional.silu(full[:, :I]) * full[:, I:]
+            act = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+            assert ops.gemm_swiglu(dev(a), dev(w), act)
+            assert rel_err(act.float().cpu().numpy(), gated.numpy()) <= OP_TOL[torch.bfloat16]
+    finally:
+        ops.use_library_gemm = library
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 3072, 1024), (40, 100, 96), (64, 560, 256)])
 def test_gemm_swiglu_fused(M, I, K):
     ops = ops_for(torch.bfloat16)
