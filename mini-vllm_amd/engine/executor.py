@@ -463,9 +463,8 @@ class Executor:
             # the single-step capture sizes the shared scratch area and loads every kernel
             a1, o1, f1 = self._fill(seqs, pad_to=bucket, bt_widths=[self.max_pages_per_seq] * len(self.groups))
             self._capture(bucket, cap, a1, o1, f1, seqs)
-        library_gemm = self.ops.use_library_gemm
         eager_workspace = self.rt.workspace
-        self.ops.use_library_gemm = False
+        self.ops.for_graph = True
         try:
             self.rt.workspace = self._graph_workspace
             meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
@@ -496,7 +495,7 @@ class Executor:
         finally:
             self._graph_workspace.frozen = False
             self.rt.workspace = eager_workspace
-            self.ops.use_library_gemm = library_gemm
+            self.ops.for_graph = False
         torch.cuda.synchronize()
         entry = (graph, meta, tokens)
         self._repeat_graphs[key] = entry
@@ -519,9 +518,8 @@ class Executor:
 
     def _capture(self, bucket: int, cap: int, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
         logger.info("capturing the decode graph for %d sequences, contexts up to %d", bucket, cap)
-        library_gemm = self.ops.use_library_gemm
         eager_workspace = self.rt.workspace
-        self.ops.use_library_gemm = False          # only the engine's own kernels inside a graph
+        self.ops.for_graph = True                  # library products only where a rehearsal allows them
         try:
             if self._graph_workspace is None:
                 # one scratch area for all graphs, sized for the largest bucket; should a later
@@ -550,7 +548,7 @@ class Executor:
         finally:
             self._graph_workspace.frozen = False
             self.rt.workspace = eager_workspace
-            self.ops.use_library_gemm = library_gemm
+            self.ops.for_graph = False
         torch.cuda.synchronize()
         entry = (graph, ctx, meta, logits)
         self._graphs[(bucket, cap)] = entry

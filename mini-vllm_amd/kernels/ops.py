@@ -73,6 +73,10 @@ class Ops:
         self.lib = library.load(library.variant_of(_NAMES[dtype]))
         self.use_fast_kernels = dtype == torch.bfloat16
         self.use_library_gemm = dtype == torch.bfloat16
+        # set by the executor while it rehearses and captures a graph: the library's product then
+        # runs only for shapes that passed a rehearsal of their own (see _library_allowed)
+        self.for_graph = False
+        self._library_in_graph: dict = {}
         self.stream_handle: Optional[int] = None
         self._transposed = {}
         self._mid_work: Optional[torch.Tensor] = None
@@ -277,7 +281,7 @@ class Ops:
         if fast and K % 32 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.lib.has("mv_gemm_skinny"):
             if self._gemm_mid(a, lda, w, bias, out, ldc, M, N, K, swiglu=False):
                 return
-            if M <= SKINNY_MAX_M or out.dtype == torch.float32 or not self.use_library_gemm:
+            if M <= SKINNY_MAX_M or out.dtype == torch.float32 or not self._library_allowed(M, N, K, bias is not None):
                 # more rows than one workgroup takes are dealt out to groups of workgroups by the kernel
                 for m0 in range(0, M, SKINNY_LAUNCH_ROWS):
                     m = min(SKINNY_LAUNCH_ROWS, M - m0)
@@ -285,7 +289,7 @@ class Ops:
                                   out.data_ptr() + m0 * ldc * out.element_size(), ldc, _CODES[out.dtype], m, N, K,
                                   self._stream())
                 return
-        if fast and self.use_library_gemm and out.dtype == self.dtype and M > SKINNY_MAX_M:
+        if fast and out.dtype == self.dtype and M > SKINNY_MAX_M and self._library_allowed(M, N, K, bias is not None):
             wt = self._transposed.get(w.data_ptr())
             if wt is None or wt.shape != (K, N):
                 wt = self._transposed[w.data_ptr()] = w.t()      # the view is made once per weight
@@ -296,6 +300,59 @@ class Ops:
             return
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
+
+    def _library_allowed(self, M: int, N: int, K: int, with_bias: bool) -> bool:
+        """Whether the library's matrix product may serve this shape now. Outside graphs: whenever it
+        is switched on. For a graph: only when a graph holding just this product, replayed several
+        times with other work and synchronisations in between, gave the eager result every time
+        (a library may record nodes that do not replay faithfully). The rehearsal happens in the
+        eager run that precedes every capture; a shape that was never rehearsed stays with the
+        engine's own kernels."""
+        if not self.use_library_gemm:
+            return False
+        if not self.for_graph:
+            return True
+        key = (M, N, K, with_bias)
+        ok = self._library_in_graph.get(key)
+        if ok is None:
+            if torch.cuda.is_current_stream_capturing():
+                return False
+            ok = self._library_in_graph[key] = self._rehearse_library_product(M, N, K, with_bias)
+        return ok
+
+    def _rehearse_library_product(self, M: int, N: int, K: int, with_bias: bool) -> bool:
+        dev = torch.device("cuda", torch.cuda.current_device())
+        a = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+        wt = (torch.randn(N, K, device=dev, dtype=torch.bfloat16) * 0.05).t()
+        bias = torch.randn(N, device=dev, dtype=torch.bfloat16) if with_bias else None
+        out = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+
+        def product(dst):
+            if bias is None:
+                torch.mm(a, wt, out=dst)
+            else:
+                torch.addmm(bias, a, wt, out=dst)
+
+        try:
+            product(out)                                   # loads the kernel, makes the library's handles
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                product(out)
+            ok = True
+            want = torch.empty_like(out)
+            for _ in range(3):
+                a.normal_()                                # eager work between the replays
+                out.fill_(float("nan"))
+                torch.cuda.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                product(want)
+                ok = ok and bool(torch.equal(out, want))
+            del graph
+            return ok
+        except RuntimeError:
+            return False
 
     def _gemm_mid(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   ldc: int, M: int, N: int, K: int, swiglu: bool) -> bool:
@@ -363,7 +420,7 @@ class Ops:
         M, K = a.shape
         two_i = w_gate_up.shape[0]
         # with the library's product at hand, more rows than one workgroup takes go there
-        if (M > (SKINNY_MAX_M if self.use_library_gemm else SKINNY_LAUNCH_ROWS) or M == 0
+        if (M > SKINNY_LAUNCH_ROWS or M == 0 or (M > SKINNY_MAX_M and self._library_allowed(M, two_i, K, False))
                 or w_gate_up.dtype != torch.bfloat16 or K % 32 or two_i % 2
                 or a.stride(1) != 1 or (M > 1 and a.stride(0) % 8) or a.data_ptr() % 16
                 or not w_gate_up.is_contiguous() or w_gate_up.shape[1] != K):

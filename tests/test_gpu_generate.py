@@ -226,3 +226,31 @@ def test_decode_steps_in_a_row_give_the_same_tokens(models, dtype):
     cut, why_cut, _ = run(4, True, eos=(stop,))
     ref, why_ref, _ = run(1, True, eos=(stop,))
     assert cut == ref and why_cut == why_ref and "stop" in why_cut
+
+
+def test_graphs_of_many_sequences_use_rehearsed_library_products(models):
+    """Decode steps of more than 64 sequences: inside a graph the library's matrix product serves
+    the shapes that passed a rehearsal (a graph of just that product, replayed against eager runs);
+    replays must give what eager steps give."""
+    from minivllm_amd.engine.trace import TraceRunner
+    from minivllm_amd.kernels.ops import get_ops
+    cfg, w, path = models["B"]
+    S = 70
+    toks = {f"s{i}": random_tokens(cfg, 12 + i % 5, seed=900 + i) for i in range(S)}
+    runs = {}
+    for use_graph in (False, True):
+        r = TraceRunner(path, "bfloat16", 64 * S, page_size=16, use_graph=use_graph, max_live=128)
+        for rid, t in toks.items():
+            r.run_step({"step": 0, "entries": [{"id": rid, "tokens": t[:8], "want": []}], "end": []})
+        rows = []
+        for p in range(8, 12):
+            out = r.run_step({"step": p, "entries": [{"id": rid, "tokens": [t[p]], "want": [0]}
+                                                      for rid, t in toks.items()], "end": []})
+            rows.append(out.copy())
+            torch.cuda.synchronize()
+        runs[use_graph] = np.stack(rows)
+        del r
+    assert rel_err(runs[True], runs[False]) <= 2e-2
+    verdicts = get_ops(torch.bfloat16)._library_in_graph
+    assert verdicts and all(m > 64 for (m, _, _, _) in verdicts), verdicts
+    assert all(verdicts.values()), f"a library product did not replay faithfully: {verdicts}"
