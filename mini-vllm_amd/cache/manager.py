@@ -24,6 +24,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 from .page_pool import OutOfPages, PagePool, page_hash
 from .state_slots import OutOfSlots, StateSlots
 
@@ -61,6 +63,32 @@ class SequenceCache:
     num_computed: int = 0             # positions whose keys and values are in the cache
     num_cached: int = 0               # of those, how many came from prefix reuse
     hashes: List[int] = field(default_factory=list)   # chained hashes of the full pages so far
+    # the same page ids as int32 arrays (grown in steps), so that a step's block tables are copied
+    # rather than converted element by element
+    arrays: List[np.ndarray] = field(default_factory=list)
+
+    def push(self, group: int, page: int) -> None:
+        pages = self.pages[group]
+        while len(self.arrays) <= group:
+            self.arrays.append(np.full(16, -1, dtype=np.int32))
+        arr = self.arrays[group]
+        if len(pages) >= arr.size:
+            grown = np.full(2 * arr.size, -1, dtype=np.int32)
+            grown[:arr.size] = arr
+            arr = self.arrays[group] = grown
+        arr[len(pages)] = page
+        pages.append(page)
+
+    def drop(self, group: int, index: int) -> None:
+        self.pages[group][index] = -1
+        self.arrays[group][index] = -1
+
+    def table(self, group: int) -> np.ndarray:
+        """The block table of a group as an int32 array (a view: copy it before the next change)."""
+        n = len(self.pages[group])
+        if len(self.arrays) <= group:
+            return np.empty(0, dtype=np.int32)
+        return self.arrays[group][:n]
 
 
 class CacheManager:
@@ -114,6 +142,16 @@ class CacheManager:
                    for g in range(len(self.groups))) if self.groups else 1 << 60
         return max(0, room - seq.num_computed)
 
+    def fits(self, req, num_new_tokens: int) -> bool:
+        """Whether the pages the request already holds take that many more positions."""
+        seq = self.seqs[req]
+        end = seq.num_computed + num_new_tokens
+        ps = self.page_size
+        for pages in seq.pages:
+            if end > len(pages) * ps:
+                return False
+        return True
+
     def can_reserve(self, req, num_new_tokens: int) -> bool:
         return all(n <= self.pools[g].num_free for g, n in enumerate(self.pages_needed(req, num_new_tokens)))
 
@@ -142,7 +180,7 @@ class CacheManager:
                     break
                 for g, p in enumerate(found):
                     self.pools[g].share(p)
-                    seq.pages[g].append(p)
+                    seq.push(g, p)
                 seq.hashes.append(h)
                 prefix = h
                 seq.num_computed += ps
@@ -159,7 +197,7 @@ class CacheManager:
         seq = self.seqs[req]
         for g, n in enumerate(needed):
             for _ in range(n):
-                seq.pages[g].append(self.pools[g].allocate())
+                seq.push(g, self.pools[g].allocate())
 
     def commit(self, req, num_new_tokens: int, tokens: Optional[Sequence[int]] = None) -> None:
         """Records that the step wrote ``num_new_tokens`` more positions. ``tokens`` (the
@@ -191,7 +229,7 @@ class CacheManager:
             for i in range(first):
                 if pages[i] >= 0:
                     self.pools[g].release(pages[i])
-                    pages[i] = -1
+                    seq.drop(g, i)
 
     def release(self, req) -> None:
         """Gives back everything the request holds (it ended or was preempted)."""
@@ -206,6 +244,10 @@ class CacheManager:
     def block_table(self, req, group: int) -> List[int]:
         return self.seqs[req].pages[group]
 
+    def block_table_array(self, req, group: int) -> np.ndarray:
+        """The same as an int32 array (a view that the next reserve or commit may change)."""
+        return self.seqs[req].table(group)
+
     def check_invariants(self) -> None:
         """No page lost, held twice without a count, or freed twice."""
         self.slots.check()
@@ -215,6 +257,7 @@ class CacheManager:
             pool.check()
             holders: Dict[int, int] = {}
             for seq in self.seqs.values():
+                assert seq.table(g).tolist() == list(seq.pages[g]), "the array of a block table lags behind its list"
                 for p in seq.pages[g]:
                     if p >= 0:
                         holders[p] = holders.get(p, 0) + 1

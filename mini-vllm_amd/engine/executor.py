@@ -272,17 +272,26 @@ class Executor:
         lr = arr[off["logit_rows"][0]:off["logit_rows"][0] + Mp]
         lr[:] = -1
         lr[:M] = want_rows
-        base = 0
-        for i, (s, n) in enumerate(zip(seqs, q_lens)):
-            tok[base:base + n] = s.tokens
-            pos[base:base + n] = np.arange(s.start, s.start + n, dtype=np.int32)
-            tsq[base:base + n] = i
-            cu[i + 1] = base + n
-            cl[i] = s.start + n
-            sl[i] = s.state_slot
-            base += n
-        cu[S + 1:] = base
         starts = np.fromiter((s.start for s in seqs), dtype=np.int64, count=S)
+        if N == S:                                  # one token each: no loop over the sequences
+            tok[:S] = np.fromiter((s.tokens[0] for s in seqs), dtype=np.int64, count=S)
+            pos[:S] = starts
+            tsq[:S] = np.arange(S, dtype=np.int32)
+            cu[:S + 1] = np.arange(S + 1, dtype=np.int32)
+            cl[:S] = starts + 1
+            sl[:S] = np.fromiter((s.state_slot for s in seqs), dtype=np.int64, count=S)
+            base = S
+        else:
+            base = 0
+            for i, (s, n) in enumerate(zip(seqs, q_lens)):
+                tok[base:base + n] = s.tokens
+                pos[base:base + n] = np.arange(s.start, s.start + n, dtype=np.int32)
+                tsq[base:base + n] = i
+                cu[i + 1] = base + n
+                cl[i] = s.start + n
+                sl[i] = s.state_slot
+                base += n
+        cu[S + 1:] = base
         last_page = (cl[:S].astype(np.int64) - 1 + lookahead) // self.page_size
         for g, w in enumerate(widths):
             o, size = off[f"bt{g}"]

@@ -97,7 +97,7 @@ class LLM:
             r = s.request
             cache = self.manager.sequence(r.id)
             seqs.append(SeqStep(tokens=r.tokens[s.start:s.start + s.num_tokens], start=s.start,
-                                block_tables=[cache.pages[g] for g in groups], state_slot=cache.state_slot,
+                                block_tables=[cache.table(g) for g in groups], state_slot=cache.state_slot,
                                 want=[s.num_tokens - 1] if s.sample else []))
         if step.repeat > 1:
             sampled = self._run_repeated(step, seqs)

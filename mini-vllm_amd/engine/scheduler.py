@@ -131,7 +131,7 @@ class Scheduler:
             start = self._computed(req)
             if len(req.tokens) - start != 1:
                 continue
-            while not self.manager.can_reserve(req.id, 1):
+            while not (self.manager.fits(req.id, 1) or self.manager.can_reserve(req.id, 1)):
                 victim = self.running[-1]
                 if victim is req or victim.id in scheduled_ids:
                     # nothing newer to take pages from (those already in this step keep theirs)
@@ -142,7 +142,8 @@ class Scheduler:
                     break
             if req.state != RequestState.RUNNING:
                 continue
-            self.manager.reserve(req.id, 1)
+            if not self.manager.fits(req.id, 1):
+                self.manager.reserve(req.id, 1)
             seqs.append(ScheduledSeq(req, start, 1, sample=True))
             scheduled_ids.add(req.id)
             budget -= 1
@@ -241,30 +242,34 @@ class Scheduler:
                 continue
             if drawn is None:
                 raise ValueError(f"request {req.id} reached its last token but no token was drawn")
-            tokens = [drawn] if isinstance(drawn, int) else list(drawn)
+            tokens = [drawn] if isinstance(drawn, int) else [int(t) for t in drawn]
             if len(tokens) != step.repeat:
                 raise ValueError(f"request {req.id}: the step ran {step.repeat} times but {len(tokens)} tokens came back")
-            for token in tokens:
-                # the run that drew this token wrote the position(s) before it; what the device ran
-                # past a request's end is dropped with its pages
-                self.manager.commit(req.id, seq.num_tokens, req.tokens)
-                req.append_output_token(int(token))
-                if req.first_token_time is None:
-                    req.first_token_time = now
-                sp = req.sampling_params
-                reason = None
+            # how many of the drawn tokens the request keeps: up to the one that ends it (what the
+            # device ran past a request's end is dropped with its pages)
+            sp = req.sampling_params
+            keep, reason = len(tokens), None
+            for j, token in enumerate(tokens):
                 if token in self.eos_token_ids and not sp.ignore_eos:
                     reason = "stop"
-                elif req.num_completion_tokens >= sp.max_tokens:
+                elif req.num_completion_tokens + j + 1 >= sp.max_tokens:
                     reason = "length"
-                elif len(req.tokens) >= self.max_model_len:
+                elif len(req.tokens) + j + 1 >= self.max_model_len:
                     reason = "length"
                 if reason is not None:
-                    req.state = RequestState.FINISHED
-                    req.finish_reason = reason
-                    req.finish_time = now
-                    self.manager.release(req.id)
-                    self.running.remove(req)
-                    done.append(req)
+                    keep = j + 1
                     break
+            for token in tokens[:keep]:
+                req.append_output_token(token)
+            if req.first_token_time is None:
+                req.first_token_time = now
+            # the run that drew token j wrote the position(s) before it
+            self.manager.commit(req.id, seq.num_tokens + keep - 1, req.tokens)
+            if reason is not None:
+                req.state = RequestState.FINISHED
+                req.finish_reason = reason
+                req.finish_time = now
+                self.manager.release(req.id)
+                self.running.remove(req)
+                done.append(req)
         return done
