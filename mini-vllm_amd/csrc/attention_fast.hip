@@ -263,10 +263,12 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     // The page ids of this workgroup's key range go to LDS first (one round trip instead of one
     // per block); K and V operands are fetched one block ahead of their use.
     __shared__ int sh_pages[AF_MAX_CACHED_PAGES];
-    const int first_block = hi_w >= 0 ? lo_w / 32 : 0;
+    const int first_block = hi_w >= 0 ? b_begin - wave : 0;          // of this workgroup's share of the keys
     const int p_first = (32 * first_block) / page_size;
     {
-        const int p_last = hi_w >= 0 ? hi_w / page_size : -1;
+        int last_key = 32 * b_end - 1;
+        if (last_key > hi_w) last_key = hi_w;
+        const int p_last = (hi_w >= 0 && b_end > first_block) ? last_key / page_size : -1;
         for (int p = p_first + (int)threadIdx.x; p <= p_last && p - p_first < AF_MAX_CACHED_PAGES; p += blockDim.x)
             sh_pages[p - p_first] = p < bt_width ? bt[p] : -1;
     }

@@ -405,6 +405,8 @@ def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(16)
     ctx_lens = [1, 17, 300, 1200, 33, 64]
+    if max_context == 40000 and Hkv == 1:
+        ctx_lens[2] = 18000                         # more pages than the kernel keeps ids of at once
     q_lens = [1, 1, 1, 0, 1, 1]                     # sequence 3 is padding: no token
     live = [s for s, ql in enumerate(q_lens) if ql]
     k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
@@ -427,7 +429,7 @@ def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
     token_seq = torch.tensor(live, dtype=torch.int32)
     n = len(live)
     q = torch.randn(n, H, D, generator=g)
-    far = 5 if window is None else 300 - 1 - window         # a far key, or the one at the window's edge
+    far = 5 if window is None else ctx_lens[2] - 1 - window  # a far key, or the one at the window's edge
     q[2] = 6.0 * k_all[2][far].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
     q = q.to(dtype)
     scale = 1.0 / math.sqrt(D)
@@ -437,6 +439,35 @@ def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
                   window, plan=plan)
     want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
     assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+
+
+def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
+    """One workgroup walks 18,000 keys (1,125 pages of 16): more page ids than it keeps in LDS, the
+    rest are read from the block table as it goes."""
+    ops = ops_for(torch.bfloat16)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(31)
+    H, Hkv, D, ps, ctx = 4, 1, 64, 16, 18000
+    k_all = [torch.randn(ctx, Hkv, D, generator=g).to(dtype).double()]
+    v_all = [torch.randn(ctx, Hkv, D, generator=g).to(dtype).double()]
+    pages = -(-ctx // ps)
+    table = torch.randperm(pages + 2, generator=g).tolist()[:pages]
+    kp, vp = fill_pages(k_all, v_all, [table], ps, Hkv, D, pages + 2, dtype)
+    bt = dev(torch.tensor([table], dtype=torch.int32))
+    q = torch.randn(1, H, D, generator=g)
+    q[0] = 6.0 * k_all[0][17000].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)   # a key far into the walk
+    q = q.to(dtype)
+    qd = dev(q.view(1, H * D))
+    out = torch.full((1, H * D), float("nan"), dtype=dtype, device="cuda")
+    pos = dev(torch.tensor([ctx - 1], dtype=torch.int32))
+    cu = dev(torch.tensor([0, 1], dtype=torch.int32))
+    seq0 = dev(torch.zeros(1, dtype=torch.int32))
+    ops.lib.call("mv_attention_decode", qd.data_ptr(), H * D, out.data_ptr(), H * D, kp.data_ptr(), vp.data_ptr(),
+                 bt.data_ptr(), pages, ps, pos.data_ptr(), cu.data_ptr(), 1, H, Hkv, D, D ** -0.5, -1, 0, 1, 4,
+                 seq0.data_ptr(), ops._stream())
+    torch.cuda.synchronize()
+    want = reference_attention(q.double(), k_all, v_all, torch.tensor([ctx - 1]), torch.tensor([0]), H, Hkv, D ** -0.5, None)
+    assert rel_err(out.float().cpu().view(1, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
 
 
 @pytest.mark.parametrize("H,Hkv,D,ps,window", [(16, 8, 128, 16, None), (8, 1, 128, 32, None), (6, 2, 64, 16, 50),
