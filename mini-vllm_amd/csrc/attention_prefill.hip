@@ -4,19 +4,24 @@
 // A workgroup of four waves serves one key/value head of one unit: up to 64*NT columns, a column
 // being a (query token, query head of the group) pair of a run of consecutive tokens of one
 // sequence. Each wave owns 16*NT columns. The workgroup walks the keys the unit may see in blocks
-// of 32; every block's K tile [32 keys x D] and transposed V tile [D x 32 keys] are copied from
-// the cache pages into LDS once, in the order the MFMA operands are read (so the reads are
-// conflict-free 16-byte loads), double-buffered: the copy of block b+1 is in flight while block
-// b is computed, with one barrier per block.
+// of 32. Every block's K tile [32 keys x D] and V tile [D x 32 keys] go from the cache pages
+// straight into LDS (global_load_lds: no registers in between, no LDS store instructions), in the
+// order the MFMA operands are read (so the reads are conflict-free 16-byte loads), into a ring of
+// three stages: while block b is computed, block b+1 has landed or is landing and block b+2 is
+// being asked for, with one barrier per block.
 //
 //   scores^T = K Q^T     A operand: 16 keys x 32 d from LDS, B operand: the wave's queries (registers);
-//                        result: lane l holds column l%16, keys 4*(l/16)+0..3 of the 16-key tile.
+//                        result: lane l holds column l%16 and rows 4*(l/16)+0..3 of the tile.
 //   out^T    = V^T P^T   A operand: 16 d x 32 keys from LDS, B operand: the probabilities the lane
-//                        already holds: its eight k-slots are bound to keys {4g..4g+3} of the two
-//                        16-key tiles of the block (g = l/16), and V is stored in LDS for exactly
-//                        those keys, so nothing is shuffled between the two products.
+//                        already holds. Its eight k-slots must be eight keys that lie side by side
+//                        in a page's V rows (one 16-byte load per operand), so row 4g+r of score tile
+//                        t is bound to key 8g + 4t + r of the block (g = l/16): the two score tiles
+//                        interleave in groups of four keys, and nothing is shuffled between the two
+//                        products.
 // Online softmax (base 2) per column. A wave skips blocks that lie outside the range of all its
-// columns. Value slots above the unit's newest key were never written and are copied as zero.
+// columns. Value slots above the unit's newest key were never written and may hold anything; the
+// lane that brought them in clears them in LDS before the block is used (keys above a column's
+// position get probability zero, and zero times a stray NaN would not be zero).
 //
 // With KW = 2 the workgroup has eight waves: two groups of four that serve the same columns and
 // take the key blocks in turn (group 0 the even ones of the unit's range, group 1 the odd ones),
@@ -31,10 +36,17 @@ typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
 union Frag {
     uint4 u;
-    uint2 h[2];
     uint16_t s[8];
     bf16x8_t v;
 };
+
+typedef __attribute__((address_space(1))) const void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// s_waitcnt that only bounds the vector memory counter (N outstanding loads may remain)
+#define AP_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 15) | (((N) >> 4) << 14))
+// s_waitcnt that only waits for the LDS (and scalar memory) counter
+#define AP_WAIT_LDS() __builtin_amdgcn_s_waitcnt(0xc07f)
 
 #define AP_WAVES 4
 #define AP_THREADS (64 * AP_WAVES)
@@ -54,15 +66,19 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     constexpr int DT = D / 16;                 // d tiles of the output product
     constexpr int COLS = 16 * AP_WAVES * NT;   // columns of a workgroup
     constexpr int KCHUNKS = 2 * DS * 64;       // 16-byte chunks of a K tile
-    constexpr int VCHUNKS = DT * 64;           // 16-byte chunks of a V tile (two 8-byte halves each)
-    constexpr int KREP = KCHUNKS / AP_THREADS;
-    constexpr int VREP = 2 * VCHUNKS / AP_THREADS;      // 8-byte chunks of a V tile pair per thread
-    static_assert(KCHUNKS % AP_THREADS == 0 && (D * 2 * 2) % AP_THREADS == 0, "tile does not divide the workgroup");
+    constexpr int VCHUNKS = DT * 64;           // 16-byte chunks of a V tile
+    constexpr int TILE = KCHUNKS + VCHUNKS;    // chunks of a block: its K tile, then its V tile
+    constexpr int KREP = 2 * DS / AP_WAVES;    // load instructions a wave issues for a K tile (64 chunks each)
+    constexpr int VREP = DT / AP_WAVES;        // ... and for a V tile
+    constexpr int LOADS = KREP + VREP;
+    static_assert((2 * DS) % AP_WAVES == 0 && DT % AP_WAVES == 0, "tile does not divide the workgroup");
 
-    // [buffer][key group] tiles: K as 16-byte chunks, then V as 8-byte chunks
-    extern __shared__ uint4 lds_tiles[];
-    uint4* const sK_all = lds_tiles;
-    uint2* const sV_all = reinterpret_cast<uint2*>(lds_tiles + 2 * KW * KCHUNKS);
+    // The ring: three stages of [key group] blocks. They are three arrays, not one, so that the
+    // compiler can tell a load into one stage from the operand reads of another and does not make
+    // the reads wait for the loads in flight.
+    __shared__ uint4 stage0[KW * TILE];
+    __shared__ uint4 stage1[KW * TILE];
+    __shared__ uint4 stage2[KW * TILE];
     __shared__ int sh_unit[3];
     __shared__ int sh_range[2][AP_WAVES * KW];
 
@@ -73,8 +89,10 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     const int tid = threadIdx.x;
     const int wave = tid / MV_WAVE;
     const int lane = tid % MV_WAVE;
-    const int cw = wave % AP_WAVES;            // which columns of the unit
-    const int kg = wave / AP_WAVES;            // which of the KW key groups
+    const int cw = __builtin_amdgcn_readfirstlane(wave % AP_WAVES);   // which columns of the unit
+    // which of the KW key groups; the same for a whole wave, and said so: everything that follows
+    // from it (block numbers, page ids, tile addresses) then lives in scalar registers
+    const int kg = __builtin_amdgcn_readfirstlane(wave / AP_WAVES);
     const int gtid = tid % AP_THREADS;         // thread within its key group
     const int i = lane % 16;
     const int g = lane / 16;
@@ -105,7 +123,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         sh_unit[2] = nt;
     }
     __syncthreads();
-    const int seq = sh_unit[0], t0 = sh_unit[1], nt = sh_unit[2];
+    const int seq = __builtin_amdgcn_readfirstlane(sh_unit[0]);
+    const int t0 = __builtin_amdgcn_readfirstlane(sh_unit[1]);
+    const int nt = __builtin_amdgcn_readfirstlane(sh_unit[2]);
     if (seq < 0 || nt <= 0) return;
     const int ncols = nt * G;
     const int* bt = block_table + (size_t)seq * bt_width;
@@ -138,6 +158,8 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         hi_w = a > hi_w ? a : hi_w;
         lo_w = b < lo_w ? b : lo_w;
     }
+    hi_w = __builtin_amdgcn_readfirstlane(hi_w);
+    lo_w = __builtin_amdgcn_readfirstlane(lo_w);
     if (lane == 0) {
         sh_range[0][wave] = hi_w;
         sh_range[1][wave] = lo_w;
@@ -149,6 +171,8 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         hi_g = sh_range[0][w] > hi_g ? sh_range[0][w] : hi_g;
         lo_g = sh_range[1][w] < lo_g ? sh_range[1][w] : lo_g;
     }
+    hi_g = __builtin_amdgcn_readfirstlane(hi_g);
+    lo_g = __builtin_amdgcn_readfirstlane(lo_g);
     if (hi_g < 0) return;
     const int b0 = lo_g / 32, b1 = hi_g / 32;
 
@@ -163,99 +187,114 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     }
     const float sc_mul = scale * LOG2E;
 
-    // ---- copy of a block from the pages: global -> registers -> LDS.
-    // Two blocks are in flight: while block b is computed, block b+1 waits in one register set
-    // and block b+2 is being loaded into the other. Everything that does not depend on the block
-    // (which chunk of the tile a thread copies, where it goes in LDS) is worked out once.
-    // A thread copies the chunks whose place in LDS follows its id, so that the LDS writes of a wave
-    // are consecutive (no bank conflicts); the matching global reads touch, per instruction, 64
-    // contiguous bytes of 16 key rows (K) or the contiguous slots of a page's rows (V).
-    struct Staged {
-        uint4 k[KREP];
-        uint2 v[VREP];
+    // ---- a block's way from the pages into LDS.
+    // A load instruction of a wave fills 64 consecutive 16-byte chunks of LDS, one per lane, from
+    // addresses the lanes choose: the chunks of one (score tile, k-step) pair of K, or of one d tile
+    // of V. A lane's chunk is the operand that lane will read back: 8 d of one key (K), or 8 keys of
+    // one d row (V). Everything that does not depend on the block is worked out once. The block
+    // number is the same for a wave, so its page ids are scalar loads, asked for a round before they
+    // are used.
+    struct PageIds {
+        int pg[2];    // the pages of the block's two halves of 16 keys
     };
-    int k_tile[KREP], k_off[KREP], k_lds[KREP];
+    const int rho = lane % 16;
+    // K: row rho of score tile t is key 8*(rho/4) + 4t + rho%4; the half of the block it lies in
+    // does not depend on t
+    const int k_half = rho / 8;
+    unsigned k_off[KREP];
 #pragma unroll
     for (int rep = 0; rep < KREP; ++rep) {
-        const int L = gtid + AP_THREADS * rep;         // LDS chunk: ((tile * DS + s) * 64 + operand lane)
-        const int ol = L % 64;
-        k_tile[rep] = L / (DS * 64);
-        k_off[rep] = (ol % 16) * D + 32 * ((L / 64) % DS) + 8 * (ol / 16);
-        k_lds[rep] = L;
+        const int pair = cw + AP_WAVES * rep;   // (score tile, k-step): LDS chunks pair * 64 ...
+        const int t = pair / DS, ks = pair % DS;
+        const int slot = 8 * ((rho / 4) % 2) + 4 * t + rho % 4;    // within its half
+        k_off[rep] = (unsigned)((slot * D + 32 * ks + 8 * g) * sizeof(bf16));
     }
-    int v_tile[VREP], v_off[VREP], v_lds[VREP], v_key[VREP];
+    // V: lane group g holds keys 8g .. 8g+7 of d row 16*dt + rho
+    const int v_half = g / 2;
+    unsigned v_off[VREP];
 #pragma unroll
     for (int rep = 0; rep < VREP; ++rep) {
-        const int L = gtid + AP_THREADS * rep;         // LDS chunk: ((d tile * 64 + operand lane) * 2 + key tile)
-        const int ol = (L / 2) % 64;
-        v_tile[rep] = L % 2;
-        v_off[rep] = (16 * (L / 128) + ol % 16) * page_size + 4 * (ol / 16);
-        v_key[rep] = 16 * v_tile[rep] + 4 * (ol / 16);
-        v_lds[rep] = L;
+        const int dt = cw + AP_WAVES * rep;
+        v_off[rep] = (unsigned)(((16 * dt + rho) * page_size + 8 * (g % 2)) * sizeof(bf16));
     }
     const int page_mask = page_size - 1;
-    auto fetch = [&](int b, Staged& st) {
-        if (b > b1) {   // past the unit's range: nothing to read (the block is not computed either)
-#pragma unroll
-            for (int rep = 0; rep < KREP; ++rep) st.k[rep] = uint4{0u, 0u, 0u, 0u};
-#pragma unroll
-            for (int rep = 0; rep < VREP; ++rep) st.v[rep] = uint2{0u, 0u};
-            return;
-        }
-        const bf16* kbase[2];
-        const bf16* vbase[2];
-        bool gone[2];
+    // round j of the walk: key group kg has block b0 + j * KW + kg
+    auto block_of = [&](int j) { return b0 + j * KW + kg; };
+    auto page_ids = [&](int j) {
+        int b = block_of(j);
+        b = b < b1 ? b : b1;    // past the unit's range: some valid entry (the block is not fetched)
+        PageIds ids;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int key0 = 32 * b + 16 * t;
-            int pidx = key0 >> page_shift;
+            int pidx = (32 * b + 16 * t) >> page_shift;
             pidx = pidx < bt_width ? pidx : bt_width - 1;
-            int pg = bt[pidx];
-            gone[t] = pg < 0;      // a page that was given back (it lies below every column's range):
-            pg = gone[t] ? 0 : pg; // read some page, then put zeros in its place
-            const int slot0 = key0 & page_mask;
-            const size_t head = (size_t)pg * Hkv + kvh;
-            kbase[t] = k_pages + (head * page_size + slot0) * D;
-            vbase[t] = v_pages + head * D * page_size + slot0;
+            ids.pg[t] = bt[pidx];
         }
+        return ids;
+    };
+    // a page's bytes per tensor, and where this key/value head starts in it (K [slot][d] and V [d][slot]
+    // have the same size)
+    const unsigned page_bytes = (unsigned)Hkv * page_size * D * sizeof(bf16);
+    const char* const k_head = reinterpret_cast<const char*>(k_pages) + (size_t)kvh * page_size * D * sizeof(bf16);
+    const char* const v_head = reinterpret_cast<const char*>(v_pages) + (size_t)kvh * page_size * D * sizeof(bf16);
+    // Asks for the block of round j (at most the unit's last one: the same block again does no harm).
+    // Returns a bit per half whose page was given back (its keys lie below every column's range):
+    // some page is read in its place and the values are cleared when they have landed.
+    auto fetch = [&](int j, const PageIds& ids, uint4* stage) {
+        int b = block_of(j);
+        b = b < b1 ? b : b1;
+        const char* kbase[2];
+        const char* vbase[2];
+        int gone = 0;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            int pg = ids.pg[t];
+            if (pg < 0) {
+                gone |= 1 << t;
+                pg = 0;
+            }
+            const unsigned slot0 = (unsigned)((32 * b + 16 * t) & page_mask);
+            const size_t page_off = (size_t)(unsigned)pg * page_bytes;
+            kbase[t] = k_head + page_off + slot0 * (unsigned)(D * sizeof(bf16));
+            vbase[t] = v_head + page_off + slot0 * (unsigned)sizeof(bf16);
+        }
+        const char* kb = k_half ? kbase[1] : kbase[0];
+        const char* vb = v_half ? vbase[1] : vbase[0];
+        uint4* tile = stage + kg * TILE;
 #pragma unroll
         for (int rep = 0; rep < KREP; ++rep)
-            st.k[rep] = *reinterpret_cast<const uint4*>((k_tile[rep] ? kbase[1] : kbase[0]) + k_off[rep]);
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(kb + k_off[rep]),
+                                             (lds_ptr_t)(tile + (cw + AP_WAVES * rep) * 64), 16, 0, 0);
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep)
-            st.v[rep] = *reinterpret_cast<const uint2*>((v_tile[rep] ? vbase[1] : vbase[0]) + v_off[rep]);
-        if (gone[0] || gone[1]) {
-#pragma unroll
-            for (int rep = 0; rep < KREP; ++rep)
-                if (gone[k_tile[rep]]) st.k[rep] = uint4{0u, 0u, 0u, 0u};
-#pragma unroll
-            for (int rep = 0; rep < VREP; ++rep)
-                if (gone[v_tile[rep]]) st.v[rep] = uint2{0u, 0u};
-        }
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(vb + v_off[rep]),
+                                             (lds_ptr_t)(tile + KCHUNKS + (cw + AP_WAVES * rep) * 64), 16, 0, 0);
+        return gone;
     };
-    // round j of the walk: key group kg has block b0 + j * KW + kg, in the tiles [j & 1][kg]
-    auto block_of = [&](int j) { return b0 + j * KW + kg; };
-    auto stash = [&](int j, const Staged& st) {
+    // After the wave's own loads of round j have landed: clears the values of keys that were never
+    // written (above the unit's newest key) or whose page was given back. Each lane mends the chunks
+    // it brought in, so no other wave is involved before the barrier.
+    auto mend = [&](int j, int gone, uint4* stage) {
         const int b = block_of(j);
-        uint4* sK = sK_all + ((j & 1) * KW + kg) * KCHUNKS;
-        uint2* sV = sV_all + ((j & 1) * KW + kg) * (VCHUNKS * 2);
-#pragma unroll
-        for (int rep = 0; rep < KREP; ++rep) sK[k_lds[rep]] = st.k[rep];
-        const bool tail = 32 * b + 31 > hi_g;  // slots above the newest key were never written
+        const bool tail = 32 * b + 31 > hi_g;
+        if (!tail && gone == 0) return;
+        uint4* sV = stage + kg * TILE + KCHUNKS;
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep) {
-            uint2 f = st.v[rep];
-            if (tail) {
-                const int key = 32 * b + v_key[rep];
-                if (key > hi_g) f.x = 0;
-                else if (key + 1 > hi_g) f.x &= 0xffffu;
-                if (key + 2 > hi_g) f.y = 0;
-                else if (key + 3 > hi_g) f.y &= 0xffffu;
+            const int idx = (cw + AP_WAVES * rep) * 64 + lane;
+            Frag f;
+            f.u = sV[idx];
+            if ((gone >> v_half) & 1) {
+                f.u = uint4{0u, 0u, 0u, 0u};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (32 * b + 8 * g + e > hi_g) f.s[e] = 0;
             }
-            sV[v_lds[rep]] = f;
+            sV[idx] = f.u;
         }
+        AP_WAIT_LDS();
     };
-
     // keys at or below `full_hi` and at or above `full_lo` are visible to every column of the wave:
     // blocks inside need no mask
     int full_hi = 0x7fffffff, full_lo = 0;
@@ -272,32 +311,39 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         full_hi = a < full_hi ? a : full_hi;
         full_lo = c > full_lo ? c : full_lo;
     }
+    full_hi = __builtin_amdgcn_readfirstlane(full_hi);
+    full_lo = __builtin_amdgcn_readfirstlane(full_lo);
     bool all_cols = true;
 #pragma unroll
     for (int ct = 0; ct < NT; ++ct) all_cols = all_cols && col_ok[ct];
     const bool wave_full = __all(all_cols);
 
-    auto compute = [&](int j) {
-        const int b = block_of(j);
-        const uint4* sK = sK_all + ((j & 1) * KW + kg) * KCHUNKS;
-        const uint2* sV = sV_all + ((j & 1) * KW + kg) * (VCHUNKS * 2);
-        const int base = 32 * b;
-        if (b > b1 || !(base <= hi_w && base + 31 >= lo_w)) return;
-        const bool masked = !(wave_full && base + 31 <= full_hi && base >= full_lo);
-        // scores^T for the two 16-key tiles
-        float p[NT][2][4];
+    // A round's computation comes in two parts, so that the loads of a later round can be asked for
+    // in between: first the operands of the block are read from LDS into registers ...
+    struct Operands {
         Frag kop[2][DS];
+        Frag vop[DT];   // asked for with the keys; they arrive while the softmax is worked out
+    };
+    auto wanted = [&](int j) {   // whether the wave has anything to do with the block of round j
+        const int b = block_of(j);
+        return b <= b1 && 32 * b <= hi_w && 32 * b + 31 >= lo_w;
+    };
+    auto read_operands = [&](const uint4* stage, Operands& op) {
+        const uint4* sK = stage + kg * TILE;
+        const uint4* sV = sK + KCHUNKS;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int s = 0; s < DS; ++s) kop[t][s].u = sK[(t * DS + s) * 64 + lane];
-        // the value operands are asked for now and arrive while the softmax is worked out
-        Frag vop[DT];
+            for (int s = 0; s < DS; ++s) op.kop[t][s].u = sK[(t * DS + s) * 64 + lane];
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            vop[dt].h[0] = sV[(dt * 64 + lane) * 2];
-            vop[dt].h[1] = sV[(dt * 64 + lane) * 2 + 1];
-        }
+        for (int dt = 0; dt < DT; ++dt) op.vop[dt].u = sV[dt * 64 + lane];
+    };
+    // ... then the two products with the softmax between them
+    auto compute = [&](int j, const Operands& op) {
+        const int base = 32 * block_of(j);
+        const bool masked = !(wave_full && base + 31 <= full_hi && base >= full_lo);
+        // scores^T for the two 16-key tiles
+        float p[NT][2][4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -305,7 +351,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s = 0; s < DS; ++s)
-                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[t][s].v, qop[ct][s].v, sacc, 0, 0, 0);
+                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.kop[t][s].v, qop[ct][s].v, sacc, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) p[ct][t][r] = sacc[r];
             }
@@ -317,7 +363,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const int key = base + 16 * t + 4 * g + r;
+                        const int key = base + 8 * g + 4 * t + r;
                         const bool ok = col_ok[ct] && key <= col_pos[ct] && key >= col_lo[ct];
                         p[ct][t][r] = ok ? p[ct][t][r] : -INFINITY;
                     }
@@ -366,27 +412,56 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct)
-                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
+                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
     };
 
     const int rounds = (b1 - b0 + KW) / KW;    // the same for every wave: they meet at the barriers
-    Staged sa, sb;
-    fetch(block_of(0), sa);
-    fetch(block_of(1), sb);
-    stash(0, sa);
-    __syncthreads();
-    // invariant at the top: LDS holds round j, `sb` holds round j+1 (or zeros past the end)
-    for (int j = 0; j < rounds; j += 2) {
-        fetch(block_of(j + 2), sa);
-        compute(j);
-        if (j + 1 < rounds) stash(j + 1, sb);
-        __syncthreads();
-        if (j + 1 >= rounds) break;
-        fetch(block_of(j + 3), sb);
-        compute(j + 1);
-        if (j + 2 < rounds) stash(j + 2, sa);
-        __syncthreads();
+    // One round: read the operands of round j, ask for round j+2, compute round j, make sure round
+    // j+1 has landed, meet.
+    // `cur`, `nxt` and `far` are the stages of rounds j, j+1 and j+2. The barrier orders the operand
+    // reads of a stage before the loads that refill it two rounds later, and makes every wave's loads
+    // of the next round visible to the others (each wave has waited for its own).
+    PageIds ids_far;
+    int gone_nxt = 0;
+    auto round = [&](int j, uint4* cur, uint4* nxt, uint4* far) {
+        const bool more = j + 2 < rounds;
+        const bool busy = wanted(j);
+        int gone_far = 0;
+        Operands op;
+        if (busy) read_operands(cur, op);
+        if (more) {
+            gone_far = fetch(j + 2, ids_far, far);
+            ids_far = page_ids(j + 3);
+        }
+        if (busy) compute(j, op);
+        // (the wait is not left out where no round follows: the compiler could then no longer see
+        // that nothing is in flight into a stage when the loop comes back to read it)
+        if (more) AP_WAIT_VMCNT(LOADS);
+        else AP_WAIT_VMCNT(0);
+        if (j + 1 < rounds) mend(j + 1, gone_nxt, nxt);
+        __builtin_amdgcn_s_barrier();
+        gone_nxt = gone_far;
+    };
+    {
+        const PageIds i0 = page_ids(0), i1 = page_ids(1);
+        const int gone0 = fetch(0, i0, stage0);
+        if (rounds > 1) {
+            gone_nxt = fetch(1, i1, stage1);
+            AP_WAIT_VMCNT(LOADS);
+        } else {
+            AP_WAIT_VMCNT(0);
+        }
+        ids_far = page_ids(2);
+        mend(0, gone0, stage0);
+        __builtin_amdgcn_s_barrier();
     }
+    // (rounds past the last one do nothing but meet at the barrier)
+    for (int j = 0; j < rounds; j += 3) {
+        round(j, stage0, stage1, stage2);
+        round(j + 1, stage1, stage2, stage0);
+        round(j + 2, stage2, stage0, stage1);
+    }
+    // nothing is in flight any more: the last rounds fetch nothing and wait for everything
 
     // the sum of a column is spread over the four lane groups
 #pragma unroll
@@ -395,37 +470,44 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         l_run[ct] += __shfl_xor(l_run[ct], 32, MV_WAVE);
     }
 
-    if (KW > 1) {
-        // ---- key group 1 hands its partial results to group 0 through LDS (the tiles are no
-        // longer needed: every wave has passed the last barrier of the walk), one column tile at a time
-        float* xo = reinterpret_cast<float*>(lds_tiles);                 // [AP_WAVES][DT][4][64]
-        float* xm = xo + AP_WAVES * DT * 4 * MV_WAVE;                    // [AP_WAVES][16] maxima, then sums
+    if constexpr (KW > 1) {
+        // ---- the other key groups hand their partial results to group 0 through LDS, one after the
+        // other and one column tile at a time (the tiles are no longer needed: every wave has passed
+        // the last barrier of the walk, and nothing is in flight)
+        static_assert(sizeof(stage0) >= AP_WAVES * DT * 4 * MV_WAVE * sizeof(float) && sizeof(stage1) >= 2 * AP_WAVES * 16 * sizeof(float),
+                      "the stages are too small for the exchange");
+        float* xo = reinterpret_cast<float*>(stage0);                    // [AP_WAVES][DT][4][64]
+        float* xm = reinterpret_cast<float*>(stage1);                    // [AP_WAVES][16] maxima, then sums
         float* xl = xm + AP_WAVES * 16;
 #pragma unroll
-        for (int ct = 0; ct < NT; ++ct) {
-            if (ct) __syncthreads();
-            if (kg == 1) {
+        for (int src = 1; src < KW; ++src) {
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
+            for (int ct = 0; ct < NT; ++ct) {
+                if (src > 1 || ct > 0) __syncthreads();
+                if (kg == src) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) xo[((cw * DT + dt) * 4 + r) * MV_WAVE + lane] = acc_o[ct][dt][r];
-                if (g == 0) {
-                    xm[cw * 16 + i] = m_run[ct];
-                    xl[cw * 16 + i] = l_run[ct];
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) xo[((cw * DT + dt) * 4 + r) * MV_WAVE + lane] = acc_o[ct][dt][r];
+                    if (g == 0) {
+                        xm[cw * 16 + i] = m_run[ct];
+                        xl[cw * 16 + i] = l_run[ct];
+                    }
                 }
-            }
-            __syncthreads();
-            if (kg == 0) {
-                const float m1 = xm[cw * 16 + i], l1 = xl[cw * 16 + i];
-                const float m_fin = fmaxf(m_run[ct], m1);
-                const float f0 = (m_run[ct] == -INFINITY) ? 0.f : exp2f(m_run[ct] - m_fin);
-                const float f1 = (m1 == -INFINITY) ? 0.f : exp2f(m1 - m_fin);
-                l_run[ct] = f0 * l_run[ct] + f1 * l1;
+                __syncthreads();
+                if (kg == 0) {
+                    const float m1 = xm[cw * 16 + i], l1 = xl[cw * 16 + i];
+                    const float m_fin = fmaxf(m_run[ct], m1);
+                    const float f0 = (m_run[ct] == -INFINITY) ? 0.f : exp2f(m_run[ct] - m_fin);
+                    const float f1 = (m1 == -INFINITY) ? 0.f : exp2f(m1 - m_fin);
+                    m_run[ct] = m_fin;
+                    l_run[ct] = f0 * l_run[ct] + f1 * l1;
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
+                    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        acc_o[ct][dt][r] = f0 * acc_o[ct][dt][r] + f1 * xo[((cw * DT + dt) * 4 + r) * MV_WAVE + lane];
+                        for (int r = 0; r < 4; ++r)
+                            acc_o[ct][dt][r] = f0 * acc_o[ct][dt][r] + f1 * xo[((cw * DT + dt) * 4 + r) * MV_WAVE + lane];
+                }
             }
         }
         if (kg != 0) return;
@@ -459,16 +541,8 @@ static int launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_s
                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                           int page_size, int page_shift, const int* positions, const int* cu_seqlens, int n_seqs,
                           int H, int Hkv, float scale, int window, int fold) {
-    // K and V tiles of 32 keys, double-buffered, one set per key group
-    const size_t lds = (size_t)2 * KW * (2 * (D / 32) * 64 * 16 + (D / 16) * 64 * 16);
-    static bool allowed = false;   // more than 64 KiB of LDS has to be asked for, once per kernel
-    if (!allowed && lds > 48 * 1024) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, NT, KW>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return mv_fail("attention_prefill: %zu bytes of LDS were refused: %s", lds, hipGetErrorString(e));
-        allowed = true;
-    }
-    hipLaunchKernelGGL((attention_prefill_kernel<D, NT, KW>), grid, dim3(AP_THREADS * KW), lds, stream, (const bf16*)q,
+    // the ring of K and V tiles is static LDS (three stages of 16 KiB per key group with D = 128)
+    hipLaunchKernelGGL((attention_prefill_kernel<D, NT, KW>), grid, dim3(AP_THREADS * KW), 0, stream, (const bf16*)q,
                        q_stride, (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table,
                        bt_width, page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold);
     return 0;
