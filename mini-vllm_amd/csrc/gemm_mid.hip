@@ -1,17 +1,19 @@
-// Matrix product for a few dozen rows against a large weight (decode steps of 17 to 64 sequences
-// on models whose weights take tens of megabytes per matrix):
+// Matrix product for up to 64 rows against a large weight (decode steps on models whose weights
+// take tens or hundreds of megabytes per matrix, the output head):
 //     C[M, N] = A[M, K] * W[N, K]^T (+ bias)      or      C[M, I] = silu(A Wg^T) * (A Wu^T),
 // M <= 64, bf16 inputs, float accumulation, on the MFMA units of gfx950.
 //
-// Each weight is still read from HBM exactly once, but here the activation rows, which every
-// weight tile needs, weigh as much as the weights themselves. So a workgroup (4 waves) takes
-// 64 * R weight rows and a slice of K, stages the activation rows of that slice through LDS once
-// for all its waves (chunks of 128 columns, double-buffered, written in the order the MFMA operands
-// are read), and every wave multiplies its R tiles of 16 weight rows, loaded straight from global
-// memory one chunk ahead, with all token tiles. K is split over `F` workgroups so that the
-// chip is filled although there are few weight tiles; with F > 1 the partial sums go to a float
-// work area [F][M][N] and a second kernel adds them in a fixed order (no atomics: a row's result
-// does not depend on what else runs), applies bias or the gated activation, and rounds.
+// Each weight is still read from HBM exactly once, but with dozens of rows the activation rows,
+// which every weight tile needs, weigh as much as the weights themselves. So a workgroup (8 waves)
+// takes 128 or 256 weight rows and a slice of K and stages the activation rows of that slice in
+// LDS once for all its waves: in chunks of 128 columns, one chunk ahead, straight from global
+// memory (global_load_lds) in the order the MFMA operands are read. Every wave multiplies its one
+// or two tiles of 16 weight rows, loaded into registers one chunk ahead, with all token tiles. K
+// is split over `F` workgroups so that the chip is filled although there are few weight tiles
+// (that also makes it the faster kernel for a single row against the largest weights); the partial
+// sums go to a float work area [F][M][N] and a second kernel adds them in a fixed order (no
+// atomics: a row's result does not depend on what else runs), applies bias or the gated
+// activation, and rounds.
 #include "dispatch.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -23,28 +25,49 @@ union Frag {
     bf16x8_t v;
 };
 
-#define GM_WAVES 4
-#define GM_THREADS (64 * GM_WAVES)
+#define GM_WAVES 8
 #ifndef GM_KC
 #define GM_KC 128          // columns of a chunk
 #endif
 #define GM_KS (GM_KC / 32)  // MFMA steps of a chunk
 #define GM_COMPUTE_UNITS 256
 
-// R: tiles of 16 weight rows per wave; TM: tiles of 16 tokens (M <= 16 * TM).
-template <int R, int TM>
-__global__ void __launch_bounds__(GM_THREADS)
+#define GM_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 15) | (((N) >> 4) << 14))
+
+// One load instruction that takes 16 bytes per lane from global memory straight into LDS: lane l's
+// bytes land at lds_base + 16 * l (lds_base the same for the whole wave). It is written as assembly,
+// not as the compiler's builtin, on purpose: the compiler then neither counts it nor guards it, and
+// the waits for it are the explicit ones at the places marked below. (With the builtin the compiler
+// puts a wait for all loads in flight in front of the first LDS read after a loop's head, which
+// undoes the prefetch.) Counting it itself, the compiler could only wait longer, never too short:
+// the vector memory counter retires in order.
+__device__ __forceinline__ void load_to_lds_16(const void* src, __attribute__((address_space(3))) void* lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(src), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+// WAVES waves to a workgroup, R tiles of 16 weight rows each; TM: tiles of 16 tokens (M <= 16 * TM).
+// The activation chunks land in one of two LDS arrays in turn.
+template <int WAVES, int R, int TM>
+__global__ void __launch_bounds__(64 * WAVES)
 gemm_mid_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W, float* __restrict__ part, int M,
-                int N, int K, int F, int chunks_per_split) {
-    __shared__ uint4 sA[2][TM * GM_KS * 64];  // [buffer][(token tile * GM_KS + k-step) * 64 + operand lane]
+                     int N, int K, int F, int chunks_per_split) {
+    constexpr int PAIRS = TM * GM_KS;                       // (token tile, k-step) pairs of a chunk: 64 LDS chunks each
+    constexpr int AREP = (PAIRS + WAVES - 1) / WAVES;       // load instructions a wave issues per chunk
+    // a wave with fewer pairs than AREP loads its last one again into a spare slot: every wave has
+    // the same number of loads in flight, which the waits below count
+    __shared__ uint4 ring0[(PAIRS + 1) * 64];
+    __shared__ uint4 ring1[(PAIRS + 1) * 64];
     const int tid = threadIdx.x;
-    const int wave = tid / MV_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / MV_WAVE);
     const int lane = tid % MV_WAVE;
     const int i = lane % 16;
     const int g = lane / 16;
     const int f = blockIdx.x % F;            // neighbouring workgroups take the splits of one row block
     const int nblock = blockIdx.x / F;
-    const int n_base = (nblock * GM_WAVES + wave) * R * 16;
+    const int n_base = (nblock * WAVES + wave) * 16 * R;
     const int chunks_total = K / GM_KC;
     const int c0 = f * chunks_per_split;
     int c1 = c0 + chunks_per_split;
@@ -57,17 +80,18 @@ gemm_mid_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W
         if (row > N - 1) row = N - 1;        // rows past the end are loaded again and never stored
         wrow[r] = reinterpret_cast<const uint4*>(W + (size_t)row * K) + g;
     }
-    // which chunks of the activation tile this thread copies (its place in LDS follows its id)
-    constexpr int AREP = TM * GM_KS * 64 / GM_THREADS;
-    const uint4* asrc[AREP];
-    bool avalid[AREP];
+
+    const char* asrc[AREP];
+    int aslot[AREP];
 #pragma unroll
     for (int rep = 0; rep < AREP; ++rep) {
-        const int L = tid + GM_THREADS * rep;          // (token tile * GM_KS + k-step) * 64 + operand lane
-        const int ol = L % 64, ks = (L / 64) % GM_KS, t = L / (64 * GM_KS);
-        const int tok = 16 * t + ol % 16;
-        avalid[rep] = tok < M;
-        asrc[rep] = reinterpret_cast<const uint4*>(A + (size_t)(avalid[rep] ? tok : 0) * lda + 32 * ks) + ol / 16;
+        int pair = wave + WAVES * rep;
+        aslot[rep] = pair < PAIRS ? pair : PAIRS;
+        pair = pair < PAIRS ? pair : PAIRS - 1;
+        const int t = pair / GM_KS, ks = pair % GM_KS;
+        int tok = 16 * t + i;
+        tok = tok < M ? tok : M - 1;         // rows past the end: some row; their products are never stored
+        asrc[rep] = reinterpret_cast<const char*>(A + (size_t)tok * lda + 32 * ks + 8 * g);
     }
 
     floatx4_t acc[R][TM];
@@ -76,32 +100,28 @@ gemm_mid_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W
 #pragma unroll
         for (int t = 0; t < TM; ++t) acc[r][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    struct Stage {
+    struct Weights {
         Frag w[GM_KS][R];
-        uint4 a[AREP];
     };
-    auto fetch = [&](int c, Stage& st) {
-        if (c >= c1) return;
+    auto fetch_w = [&](int c, Weights& st) {
         const size_t k16 = (size_t)c * (GM_KC / 8);    // offset of the chunk in 16-byte units
 #pragma unroll
         for (int ks = 0; ks < GM_KS; ++ks)
 #pragma unroll
             for (int r = 0; r < R; ++r) st.w[ks][r].u = wrow[r][k16 + 4 * ks];
-#pragma unroll
-        for (int rep = 0; rep < AREP; ++rep) st.a[rep] = avalid[rep] ? asrc[rep][k16] : uint4{0u, 0u, 0u, 0u};
     };
-    auto stash = [&](int c, const Stage& st) {
-        if (c >= c1) return;
+    auto fetch_a = [&](int c, uint4* ring) {
 #pragma unroll
-        for (int rep = 0; rep < AREP; ++rep) sA[(c - c0) & 1][tid + GM_THREADS * rep] = st.a[rep];
+        for (int rep = 0; rep < AREP; ++rep)
+            load_to_lds_16(asrc[rep] + (size_t)c * (GM_KC * sizeof(bf16)),
+                           (__attribute__((address_space(3))) void*)(ring + aslot[rep] * 64));
     };
-    auto multiply = [&](int c, const Stage& st) {
-        const uint4* a = sA[(c - c0) & 1];
+    auto multiply = [&](const Weights& st, const uint4* ring) {
 #pragma unroll
         for (int ks = 0; ks < GM_KS; ++ks) {
             Frag af[TM];
 #pragma unroll
-            for (int t = 0; t < TM; ++t) af[t].u = a[(t * GM_KS + ks) * 64 + lane];
+            for (int t = 0; t < TM; ++t) af[t].u = ring[(t * GM_KS + ks) * 64 + lane];
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -109,23 +129,34 @@ gemm_mid_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W
                     acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.w[ks][r].v, af[t].v, acc[r][t], 0, 0, 0);
         }
     };
-
-    // chunk c is multiplied from LDS and `s0` while the weights and activations of chunk c + 1 are
-    // on their way into `s1`
-    Stage s0, s1;
-    fetch(c0, s0);
-    stash(c0, s0);
-    __syncthreads();
-    for (int c = c0; c < c1; c += 2) {
-        fetch(c + 1, s1);
-        multiply(c, s0);
-        stash(c + 1, s1);
-        __syncthreads();
-        if (c + 1 >= c1) break;
-        fetch(c + 2, s0);
-        multiply(c + 1, s1);
-        stash(c + 2, s0);
-        __syncthreads();
+    // One chunk that has a successor: ask for the activations and the weights of the next one,
+    // multiply this one, make sure the next activations have landed (the weights that were asked
+    // for after them may still be on their way), meet. The barrier also orders this chunk's operand
+    // reads before the load that refills their array a chunk later. The body is straight-line code:
+    // where two paths with different loads in flight meet, the compiler's one wait has to assume
+    // the worse of them.
+    auto step = [&](int c, const Weights& cur, Weights& nxt, const uint4* ring_cur, uint4* ring_nxt) {
+        fetch_a(c + 1, ring_nxt);
+        fetch_w(c + 1, nxt);
+        multiply(cur, ring_cur);
+        GM_WAIT_VMCNT(GM_KS * R);         // explicit wait: the activations of chunk c + 1 are in LDS
+        __builtin_amdgcn_s_barrier();
+    };
+    Weights s0, s1;
+    fetch_a(c0, ring0);
+    fetch_w(c0, s0);
+    GM_WAIT_VMCNT(GM_KS * R);             // explicit wait: the activations of the first chunk are in LDS
+    __builtin_amdgcn_s_barrier();
+    int c = c0;
+    for (; c + 2 < c1; c += 2) {
+        step(c, s0, s1, ring0, ring1);
+        step(c + 1, s1, s0, ring1, ring0);
+    }
+    if (c + 1 < c1) {                     // two chunks left
+        step(c, s0, s1, ring0, ring1);
+        multiply(s1, ring1);
+    } else if (c < c1) {
+        multiply(s0, ring0);
     }
 
     // lane l holds C[token 16 t + l%16][n_base + 16 r + 4 (l/16) + 0..3]
@@ -177,21 +208,33 @@ struct MidPlan {
     int R, F, chunks_per_split, blocks;
 };
 
-// Rows per workgroup and splits of K: enough workgroups for every compute unit to hold two, as few
-// splits as that allows (their partial sums cost traffic), and at least two chunks per split.
+// Splits of K. The weights are dealt out to blocks * F workgroups, which the chip takes in rounds
+// of one per compute unit (the product is bound by memory, so one workgroup keeps a unit's share
+// of the bandwidth busy): the time goes with rounds / F, and with the traffic, which every split
+// raises by its float partial sums, written and read once, 4 F M / K of the weights. At least two
+// chunks per split. The choice does not look at the number of rows (the traffic is priced at 32
+// of them): a row's sum is then split the same way whatever else is in the step.
 static MidPlan mid_plan(int N, int K) {
     const int chunks = K / GM_KC;
-    // 64 weight rows per workgroup (measured on MI355X against 128: faster at every shape tried),
-    // and as many splits of K as bring about two workgroups to every compute unit
-    const int R = 1;
-    const int nblocks = (N + 64 * R - 1) / (64 * R);
-    int F = (2 * GM_COMPUTE_UNITS + nblocks - 1) / nblocks;
-    if (F > chunks / 2) F = chunks / 2;
-    if (F < 1) F = 1;
-    if (F > 32) F = 32;
-    const int cps = (chunks + F - 1) / F;
-    F = (chunks + cps - 1) / cps;
-    MidPlan best{R, F, cps, nblocks};
+    // two tiles of weight rows per wave where that still leaves many workgroups: the activation
+    // rows a workgroup stages then serve 256 weight rows (measured on MI355X: faster from about
+    // ten thousand weight rows on, slower below)
+    const int R = N >= 10240 ? 2 : 1;
+    const int blocks = (N + 16 * GM_WAVES * R - 1) / (16 * GM_WAVES * R);
+    MidPlan best{R, 1, chunks, blocks};
+    double best_cost = -1.0;
+    for (int cps = chunks; cps >= 2 || cps == chunks; --cps) {
+        const int F = (chunks + cps - 1) / cps;
+        if (F > 32) break;
+        const long wgs = (long)blocks * F;
+        const long rounds = (wgs + GM_COMPUTE_UNITS - 1) / GM_COMPUTE_UNITS;
+        const double cost = (double)rounds / F * (1.0 + 4.0 * F * 32 / K);
+        if (best_cost < 0.0 || cost < best_cost) {
+            best_cost = cost;
+            best = MidPlan{R, F, cps, blocks};
+        }
+        if (cps == 1) break;
+    }
     return best;
 }
 
@@ -219,8 +262,8 @@ extern "C" int mv_gemm_mid(const void* A, long lda, const void* W, const void* b
     const dim3 grid((unsigned)(p.blocks * p.F));
     const int TM = (M + 15) / 16;
 #define GM_LAUNCH(RR, TT)                                                                                          \
-    hipLaunchKernelGGL((gemm_mid_kernel<RR, TT>), grid, dim3(GM_THREADS), 0, stream, (const bf16*)A, lda,           \
-                       (const bf16*)W, work, M, N, K, p.F, p.chunks_per_split)
+    hipLaunchKernelGGL((gemm_mid_kernel<GM_WAVES, RR, TT>), grid, dim3(64 * GM_WAVES), 0, stream, (const bf16*)A,  \
+                       lda, (const bf16*)W, work, M, N, K, p.F, p.chunks_per_split)
     if (p.R == 2) {
         if (TM == 1) GM_LAUNCH(2, 1);
         else if (TM == 2) GM_LAUNCH(2, 2);

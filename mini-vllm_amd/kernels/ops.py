@@ -19,10 +19,13 @@ _NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
 SKINNY_MAX_M = 64
 # most rows of one launch of it
 SKINNY_LAUNCH_ROWS = 512
-# the kernel that shares activation rows through LDS takes over from this many rows on, for weights
-# of at least this many elements
-MID_MIN_M = 17
+# the kernel that shares activation rows through LDS and splits K over workgroups takes over from
+# this many rows on for weights of at least MID_MIN_WEIGHT elements, and at any number of rows for
+# weights of at least MID_ALWAYS_WEIGHT elements (measured on MI355X: below these the second kernel
+# that adds its partial sums costs more than its better use of the memory system brings)
+MID_MIN_M = 9
 MID_MIN_WEIGHT = 12 * 1024 * 1024
+MID_ALWAYS_WEIGHT = 120 * 1000 * 1000
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
@@ -358,8 +361,7 @@ class Ops:
                   ldc: int, M: int, N: int, K: int, swiglu: bool) -> bool:
         """The kernel for 17 to 64 rows against a large weight (activation rows shared through LDS,
         K split over workgroups); False when the shape is left to the weight-streaming kernel."""
-        if not (MID_MIN_M <= M <= SKINNY_MAX_M and N * K >= MID_MIN_WEIGHT and K % 128 == 0
-                and self.lib.has("mv_gemm_mid")):
+        if not (self.wants_mid(M, N, K) and self.lib.has("mv_gemm_mid")):
             return False
         need = int(self.lib.dll.mv_gemm_mid_workspace(M, N, K))
         if need <= 0:
@@ -374,6 +376,13 @@ class Ops:
                       _CODES[out.dtype], M, N, K, int(swiglu), self._mid_work.data_ptr(), self._mid_work.numel(),
                       self._stream())
         return True
+
+    @staticmethod
+    def wants_mid(M: int, N: int, K: int) -> bool:
+        """Whether a product of M rows with an [N, K] weight goes to the kernel that splits K."""
+        if M > SKINNY_MAX_M or K % 128:
+            return False
+        return N * K >= MID_ALWAYS_WEIGHT or (N * K >= MID_MIN_WEIGHT and M >= MID_MIN_M)
 
     def can_fuse_norm(self, rows: int, width: int) -> bool:
         """Whether a norm over ``rows`` x ``width`` may be deferred into the next product."""
@@ -397,6 +406,8 @@ class Ops:
         N = w.shape[0] // 2 if swiglu else w.shape[0]
         if out.shape != (M, N) or out.dtype not in (torch.bfloat16, torch.float32):
             return False
+        if self.wants_mid(M, w.shape[0], K) and self.lib.has("mv_gemm_mid"):
+            return False    # the norm as a kernel of its own and the K-splitting product are faster here
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N):
             return False
         resid_in, delta, resid_out = pending.fused()

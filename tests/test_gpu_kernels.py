@@ -601,10 +601,13 @@ def test_gemm_weight_streaming(out_dtype, M, N, K):
 @pytest.mark.parametrize("M,N,K,swiglu,out_dtype", [
     (17, 3100, 4096, False, torch.bfloat16), (64, 4096, 3072, False, torch.bfloat16),
     (40, 6144, 2048, False, torch.float32), (64, 6144, 2048, True, torch.bfloat16),
-    (33, 2 * 1571, 4096, True, torch.bfloat16), (20, 151936 // 4, 1024, False, torch.float32)])
+    (33, 2 * 1571, 4096, True, torch.bfloat16), (20, 151936 // 4, 1024, False, torch.float32),
+    (9, 3100, 4096, False, torch.bfloat16), (1, 151936, 1024, False, torch.float32),
+    (3, 2 * 12032, 5120, True, torch.bfloat16)])
 def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dtype):
-    """17 to 64 rows against a weight of tens of megabytes: the kernel that shares the activation
-    rows through LDS and splits K over workgroups (partial sums added in a fixed order)."""
+    """9 to 64 rows against a weight of tens of megabytes, any number of rows up to 64 against one
+    of hundreds: the kernel that shares the activation rows through LDS and splits K over
+    workgroups (partial sums added in a fixed order)."""
     ops = ops_for(torch.bfloat16)
     g = torch.Generator().manual_seed(19)
     a = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -633,7 +636,7 @@ def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dt
         out_w = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
         ops.gemm(dev(wide)[:, :K], dev(w), out_w, dev(b))
         assert torch.equal(out_w, out)
-        if half >= 17:                   # fewer rows go to the weight-streaming kernel, which sums in another order
+        if ops.wants_mid(half, N, K):    # fewer rows may go to the weight-streaming kernel, which sums in another order
             out_h = torch.full((half, N), float("nan"), dtype=out_dtype, device="cuda")
             ops.gemm(dev(a[M - half:]), dev(w), out_h, dev(b))
             assert torch.equal(out_h, out[M - half:])
