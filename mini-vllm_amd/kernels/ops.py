@@ -359,7 +359,7 @@ class Ops:
 
     def _gemm_mid(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   ldc: int, M: int, N: int, K: int, swiglu: bool) -> bool:
-        """The kernel for 17 to 64 rows against a large weight (activation rows shared through LDS,
+        """The kernel for up to 64 rows against a large weight (activation rows shared through LDS,
         K split over workgroups); False when the shape is left to the weight-streaming kernel."""
         if not (self.wants_mid(M, N, K) and self.lib.has("mv_gemm_mid")):
             return False
