@@ -21,11 +21,13 @@ SKINNY_MAX_M = 64
 SKINNY_LAUNCH_ROWS = 512
 # the kernel that shares activation rows through LDS and splits K over workgroups takes over from
 # this many rows on for weights of at least MID_MIN_WEIGHT elements, and at any number of rows for
-# weights of at least MID_ALWAYS_WEIGHT elements (measured on MI355X: below these the second kernel
-# that adds its partial sums costs more than its better use of the memory system brings)
+# weights of at least MID_ALWAYS_WEIGHT elements with rows of at least MID_ALWAYS_K (measured on
+# MI355X: below these the second kernel that adds its partial sums costs more than its better use of
+# the memory system brings; with short rows, as in the output head of a narrow model, nothing is gained)
 MID_MIN_M = 9
 MID_MIN_WEIGHT = 12 * 1024 * 1024
 MID_ALWAYS_WEIGHT = 120 * 1000 * 1000
+MID_ALWAYS_K = 2048
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
@@ -382,7 +384,7 @@ class Ops:
         """Whether a product of M rows with an [N, K] weight goes to the kernel that splits K."""
         if M > SKINNY_MAX_M or K % 128:
             return False
-        return N * K >= MID_ALWAYS_WEIGHT or (N * K >= MID_MIN_WEIGHT and M >= MID_MIN_M)
+        return (N * K >= MID_ALWAYS_WEIGHT and K >= MID_ALWAYS_K) or (N * K >= MID_MIN_WEIGHT and M >= MID_MIN_M)
 
     def can_fuse_norm(self, rows: int, width: int) -> bool:
         """Whether a norm over ``rows`` x ``width`` may be deferred into the next product."""
