@@ -352,7 +352,101 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, long row_stride, 
 // 128, 256 or 512): a head is spread over L = D / 8 neighbouring lanes, eight elements each, read
 // and written 16 bytes (bf16) at a time; sums and rotation partners travel by lane shuffles, so
 // nothing goes through LDS and a wave serves 64 / L heads.
-template <typename T, int L>
+template <typename T, int L, int HP>
+__device__ __forceinline__ void
+qk_norm_rope_store_vec(long block, T* __restrict__ qkv, long row_stride, int q_off, int k_off, int v_off,
+                       const int* __restrict__ positions, const int* __restrict__ token_seq,
+                       const int* __restrict__ block_table, int bt_width, int page_size,
+                       T* __restrict__ k_pages, T* __restrict__ v_pages, int n, int H, int Hkv,
+                       WeightPtr qw, WeightPtr kw, int has_norm, float eps, int unit_offset,
+                       const float* __restrict__ table, int store_kv) {
+    // A group of L lanes takes HP heads of one token in turn: the token's angles (twice a head's
+    // bytes when the table is float) and the norm weights are read once for all of them.
+    constexpr int D = 8 * L;
+    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
+    const int groups = (heads + HP - 1) / HP;    // lane groups of a token
+    const long gid = block * blockDim.x + threadIdx.x;
+    const long hidx = gid / L;
+    const int j = (int)(gid % L);            // this lane's eight elements start at d0 = 8 j
+    const int tok = (int)(hidx / groups), head0 = (int)(hidx % groups) * HP;
+    const int seq = tok < n ? token_seq[tok] : -1;
+    const bool active = tok < n && seq >= 0;
+    const int pos = active ? positions[tok] : 0;
+    float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sn[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (table != nullptr) {
+        const float* cs = table + (size_t)pos * D + 8 * (j % (L / 2));
+        const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
+        const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2);
+        const float4 s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
+        c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+        sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+    }
+    float wq[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, wk[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (has_norm) {
+        qw.at8(8 * j, wq);
+        if (head0 + HP > H) kw.at8(8 * j, wk);   // (a query-only launch may come without key weights)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            wq[e] = unit_offset ? wq[e] + 1.f : wq[e];
+            wk[e] = unit_offset ? wk[e] + 1.f : wk[e];
+        }
+    }
+    const bool low = j < L / 2;              // holds d < D/2; its partner d + D/2 sits L/2 lanes on
+    int page = -2;                           // the token's page, looked up when the first key or value comes
+#pragma unroll
+    for (int hp = 0; hp < HP; ++hp) {
+        const int head = head0 + hp;
+        if (head >= heads) break;            // the same for the whole lane group
+        int kind = 0, hh = head;             // 0 q, 1 k, 2 v
+        if (head >= H + Hkv) {
+            kind = 2;
+            hh = head - H - Hkv;
+        } else if (head >= H) {
+            kind = 1;
+            hh = head - H;
+        }
+        T* src = qkv + (size_t)(active ? tok : 0) * row_stride + (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) +
+                 (size_t)hh * D + 8 * j;
+        float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (active) Vec8<T>::load(src, x);
+        if (kind != 2) {
+            if (has_norm) {
+                float ss = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+                for (int o = L / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, MV_WAVE);
+                const float rinv = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = x[e] * rinv * (kind == 0 ? wq[e] : wk[e]);
+            }
+            if (table != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float other = __shfl_xor(x[e], L / 2, MV_WAVE);
+                    x[e] = low ? x[e] * c[e] - other * sn[e] : x[e] * c[e] + other * sn[e];
+                }
+            }
+        }
+        if (!active) continue;
+        if (kind == 0) {
+            Vec8<T>::store(src, x);
+            continue;
+        }
+        if (page == -2) page = block_table[(size_t)seq * bt_width + pos / page_size];
+        if (page < 0) continue;
+        const int slot = pos % page_size;
+        if (kind == 1) {
+            Vec8<T>::store(k_pages + (((size_t)page * Hkv + hh) * page_size + slot) * D + 8 * j, x);
+        } else {
+            T* dst = v_pages + (((size_t)page * Hkv + hh) * D + 8 * j) * page_size + slot;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dst[(size_t)e * page_size] = from_f<T>(x[e]);
+        }
+    }
+}
+
+template <typename T, int L, int HP>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, int k_off, int v_off,
                               const int* __restrict__ positions, const int* __restrict__ token_seq,
@@ -360,154 +454,22 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, i
                               T* __restrict__ k_pages, T* __restrict__ v_pages, int n, int H, int Hkv,
                               WeightPtr qw, WeightPtr kw, int has_norm, float eps, int unit_offset,
                               const float* __restrict__ table, int store_kv) {
-    constexpr int D = 8 * L;
-    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
-    const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    const long hidx = gid / L;
-    const int j = (int)(gid % L);            // this lane's eight elements start at d0 = 8 j
-    const int tok = (int)(hidx / heads), head = (int)(hidx % heads);
-    const int seq = tok < n ? token_seq[tok] : -1;
-    const bool active = tok < n && seq >= 0;
-    int kind = 0, hh = head;                 // 0 q, 1 k, 2 v
-    if (head >= H + Hkv) {
-        kind = 2;
-        hh = head - H - Hkv;
-    } else if (head >= H) {
-        kind = 1;
-        hh = head - H;
-    }
-    const int pos = active ? positions[tok] : 0;
-    T* src = qkv + (size_t)(active ? tok : 0) * row_stride + (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) +
-             (size_t)hh * D + 8 * j;
-    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (active) Vec8<T>::load(src, x);
-    if (kind != 2) {
-        if (has_norm) {
-            float ss = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
-#pragma unroll
-            for (int o = L / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, MV_WAVE);
-            const float rinv = rsqrtf(ss / (float)D + eps);
-            float wt[8];
-            (kind == 0 ? qw : kw).at8(8 * j, wt);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = x[e] * rinv * (unit_offset ? wt[e] + 1.f : wt[e]);
-        }
-        if (table != nullptr) {
-            const float* cs = table + (size_t)pos * D + 8 * (j % (L / 2));
-            const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
-            const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2);
-            const float4 s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
-            const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-            const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-            const bool low = j < L / 2;      // holds d < D/2; its partner d + D/2 sits L/2 lanes on
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float other = __shfl_xor(x[e], L / 2, MV_WAVE);
-                x[e] = low ? x[e] * c[e] - other * sn[e] : x[e] * c[e] + other * sn[e];
-            }
-        }
-    }
-    if (!active) return;
-    if (kind == 0) {
-        Vec8<T>::store(src, x);
-        return;
-    }
-    const int page = block_table[(size_t)seq * bt_width + pos / page_size];
-    if (page < 0) return;
-    const int slot = pos % page_size;
-    if (kind == 1) {
-        Vec8<T>::store(k_pages + (((size_t)page * Hkv + hh) * page_size + slot) * D + 8 * j, x);
-    } else {
-        T* dst = v_pages + (((size_t)page * Hkv + hh) * D + 8 * j) * page_size + slot;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dst[(size_t)e * page_size] = from_f<T>(x[e]);
-    }
+    qk_norm_rope_store_vec<T, L, HP>(blockIdx.x, qkv, row_stride, q_off, k_off, v_off, positions, token_seq, block_table,
+                                     bt_width, page_size, k_pages, v_pages, n, H, Hkv, qw, kw, has_norm, eps, unit_offset,
+                                 table, store_kv);
 }
 
-template <typename T>
-static bool launch_qk_vec(T* qkv, long row_stride, int q_off, int k_off, int v_off, const int* positions,
-                          const int* token_seq, const int* block_table, int bt_width, int page_size, T* k_pages,
-                          T* v_pages, int n, int H, int Hkv, int D, WeightPtr qw, WeightPtr kw, int has_norm, float eps,
-                          int unit_offset, const float* table, int store_kv, hipStream_t stream) {
-    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
-    const long lanes = (long)n * heads * (D / 8);
-    const dim3 grid((unsigned)((lanes + 255) / 256));
-#define QK_VEC(LL)                                                                                                 \
-    hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<T, LL>), grid, dim3(256), 0, stream, qkv, row_stride, q_off,   \
-                       k_off, v_off, positions, token_seq, block_table, bt_width, page_size, k_pages, v_pages, n, H, \
-                       Hkv, qw, kw, has_norm, eps, unit_offset, table, store_kv)
-    if (D == 64) QK_VEC(8);
-    else if (D == 128) QK_VEC(16);
-    else if (D == 256) QK_VEC(32);
-    else if (D == 512) QK_VEC(64);
-    else return false;
-#undef QK_VEC
-    return true;
-}
-
-extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int k_off, int v_off,
-                                     const int* positions, const int* token_seq, const int* block_table,
-                                     int bt_width, int page_size, void* k_pages, void* v_pages, int n, int H,
-                                     int Hkv, int D, const void* q_weight, const void* k_weight, int weight_dtype,
-                                     float eps, int unit_offset, const float* table, int rot_dim, int interleaved,
-                                     int store_kv, int dtype, hipStream_t stream) {
-    MV_REQUIRE(n >= 0 && H > 0 && Hkv >= 0 && D > 0, "qk_norm_rope_store: bad sizes n=%d H=%d Hkv=%d D=%d", n, H,
-               Hkv, D);
-    MV_REQUIRE(D <= MV_MAX_HEAD_DIM, "qk_norm_rope_store: head_dim %d exceeds the supported maximum %d", D,
-               MV_MAX_HEAD_DIM);
-    MV_REQUIRE(table == nullptr || (rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= D),
-               "qk_norm_rope_store: rotary dim %d must be even and at most head_dim %d", rot_dim, D);
-    MV_REQUIRE(!store_kv || (block_table && k_pages && v_pages && page_size > 0 && bt_width > 0),
-               "qk_norm_rope_store: cache write asked without pages or block table");
-    const int has_norm = q_weight != nullptr;
-    MV_REQUIRE(!has_norm || (k_weight != nullptr || !store_kv), "qk_norm_rope_store: q norm without k norm");
-    MV_REQUIRE(!has_norm || eps > 0.f, "qk_norm_rope_store: eps must be positive");
-    MV_REQUIRE(mv_valid_dtype(weight_dtype), "qk_norm_rope_store: bad weight dtype %d", weight_dtype);
-    if (n == 0) return 0;
-    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
-    WeightPtr qw{q_weight, weight_dtype}, kw{k_weight, weight_dtype};
-    // the vector kernel: rotation over the whole head in half-split pairs, everything 16-byte aligned
-    const size_t esz = dtype == MV_F32 ? 4 : 2;
-    const bool aligned = ((uintptr_t)qkv % 16) == 0 && (row_stride * esz) % 16 == 0 && (q_off * esz) % 16 == 0 &&
-                         (k_off * esz) % 16 == 0 && (v_off * esz) % 16 == 0 && ((uintptr_t)k_pages % 16) == 0 &&
-                         ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0 &&
-                         ((uintptr_t)table % 16) == 0;
-    if (aligned && (D == 64 || D == 128 || D == 256 || D == 512) && (table == nullptr || (rot_dim == D && !interleaved)) &&
-        (long)n * heads * (D / 8) < (1L << 31)) {
-        bool took = false;
-        MV_DISPATCH_T(dtype, "qk_norm_rope_store",
-                      took = launch_qk_vec<T>((T*)qkv, row_stride, q_off, k_off, v_off, positions, token_seq,
-                                              block_table, bt_width, page_size, (T*)k_pages, (T*)v_pages, n, H, Hkv, D,
-                                              qw, kw, has_norm, eps, unit_offset, table, store_kv, stream));
-        if (took) return mv_check_launch("qk_norm_rope_store");
-    }
-    dim3 grid(n, (heads + 3) / 4);
-    MV_DISPATCH_T(dtype, "qk_norm_rope_store",
-                  hipLaunchKernelGGL(qk_norm_rope_store_kernel<T>, grid, dim3(256), 0, stream, (T*)qkv, row_stride,
-                                     q_off, k_off, v_off, positions, token_seq, block_table, bt_width, page_size,
-                                     (T*)k_pages, (T*)v_pages, H, Hkv, D, qw, kw, has_norm, eps, unit_offset, table,
-                                     rot_dim, interleaved, store_kv));
-    return mv_check_launch("qk_norm_rope_store");
-}
-
-// ---------------------------------------------------------------------------------------
-// Value rows of many tokens into the transposed value pages V[page][kv_head][d][slot].
-// A workgroup takes 16 consecutive tokens of the step and one kv head, stages their value rows in
-// LDS, and writes with the token index running fastest over the lanes: tokens that follow each
-// other in a sequence fill neighbouring slots, so the two-byte stores of a wave merge into
-// 32-byte segments (the per-token kernel above scatters them 2 bytes at a time).
-// ---------------------------------------------------------------------------------------
-template <typename T>
-__global__ void __launch_bounds__(256)
-store_v_pages_kernel(const T* __restrict__ qkv, long row_stride, int v_off, const int* __restrict__ positions,
-                     const int* __restrict__ token_seq, const int* __restrict__ block_table, int bt_width,
-                     int page_size, T* __restrict__ v_pages, int n, int Hkv, int D) {
-    __shared__ float tile[16][MV_MAX_HEAD_DIM + 1];
-    __shared__ long dst_base[16];
-    const int tok0 = blockIdx.x * 16;
-    const int kvh = blockIdx.y;
+// Value rows of 16 consecutive tokens of the step and one kv head into the transposed value pages
+// V[page][kv_head][d][slot]: the rows are staged in LDS and written with the token index running
+// fastest over the lanes, so that tokens that follow each other in a sequence fill neighbouring
+// slots and the two-byte stores of a wave merge into 32-byte segments (a store per token and
+// head scatters them 2 bytes at a time). `tile` has a row pitch of W >= D + 1 floats.
+template <typename T, int W>
+__device__ __forceinline__ void
+store_v_tile(int tok0, int kvh, const T* __restrict__ qkv, long row_stride, int v_off,
+             const int* __restrict__ positions, const int* __restrict__ token_seq,
+             const int* __restrict__ block_table, int bt_width, int page_size, T* __restrict__ v_pages, int n,
+             int Hkv, int D, float (*tile)[W], long* dst_base) {
     const int tid = threadIdx.x;
     if (tid < 16) {
         const int tok = tok0 + tid;
@@ -532,6 +494,136 @@ store_v_pages_kernel(const T* __restrict__ qkv, long row_stride, int v_off, cons
     const long base = dst_base[j];
     if (base < 0) return;
     for (int d = tid / 16; d < D; d += 16) v_pages[base + (long)d * page_size] = from_f<T>(tile[j][d]);
+}
+
+// Prompt portions: queries and keys as above (store_kv == 2) in the first `qk_blocks` workgroups,
+// the value rows tile by tile in the others, in one launch.
+template <typename T, int L, int HP>
+__global__ void __launch_bounds__(256)
+qkv_prompt_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, int k_off, int v_off,
+                      const int* __restrict__ positions, const int* __restrict__ token_seq,
+                      const int* __restrict__ block_table, int bt_width, int page_size, T* __restrict__ k_pages,
+                      T* __restrict__ v_pages, int n, int H, int Hkv, WeightPtr qw, WeightPtr kw, int has_norm,
+                      float eps, int unit_offset, const float* __restrict__ table, int qk_blocks) {
+    if ((int)blockIdx.x < qk_blocks) {
+        qk_norm_rope_store_vec<T, L, HP>(blockIdx.x, qkv, row_stride, q_off, k_off, v_off, positions, token_seq,
+                                     block_table, bt_width, page_size, k_pages, v_pages, n, H, Hkv, qw, kw, has_norm,
+                                     eps, unit_offset, table, 2);
+        return;
+    }
+    __shared__ float tile[16][8 * L + 1];
+    __shared__ long dst_base[16];
+    const int vb = (int)blockIdx.x - qk_blocks;
+    store_v_tile<T, 8 * L + 1>((vb / Hkv) * 16, vb % Hkv, qkv, row_stride, v_off, positions, token_seq, block_table,
+                               bt_width, page_size, v_pages, n, Hkv, 8 * L, tile, dst_base);
+}
+
+template <typename T>
+static bool launch_qk_vec(T* qkv, long row_stride, int q_off, int k_off, int v_off, const int* positions,
+                          const int* token_seq, const int* block_table, int bt_width, int page_size, T* k_pages,
+                          T* v_pages, int n, int H, int Hkv, int D, WeightPtr qw, WeightPtr kw, int has_norm, float eps,
+                          int unit_offset, const float* table, int store_kv, hipStream_t stream) {
+    const bool v_tiles = store_kv == 3;     // keys per head here, values tile by tile in the same launch
+    if (v_tiles) store_kv = 2;
+    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
+    // four heads to a lane group in steps of many tokens (the angles are read once for them); one
+    // head each otherwise: smaller steps need the lanes more than the bytes (measured on MI355X:
+    // even at 2048 tokens of 24 heads, faster at 8192)
+    const int hp = (long)n * heads >= 65536 ? 4 : 1;
+    const long lanes = (long)n * ((heads + hp - 1) / hp) * (D / 8);
+    const unsigned qk_blocks = (unsigned)((lanes + 255) / 256);
+    const dim3 grid(qk_blocks + (v_tiles ? (unsigned)((n + 15) / 16) * Hkv : 0u));
+#define QK_VEC_HP(LL, PP)                                                                                          \
+    if (v_tiles)                                                                                                   \
+        hipLaunchKernelGGL((qkv_prompt_vec_kernel<T, LL, PP>), grid, dim3(256), 0, stream, qkv, row_stride, q_off, \
+                           k_off, v_off, positions, token_seq, block_table, bt_width, page_size, k_pages, v_pages, \
+                           n, H, Hkv, qw, kw, has_norm, eps, unit_offset, table, (int)qk_blocks);                  \
+    else                                                                                                           \
+        hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<T, LL, PP>), grid, dim3(256), 0, stream, qkv,            \
+                           row_stride, q_off, k_off, v_off, positions, token_seq, block_table, bt_width,           \
+                           page_size, k_pages, v_pages, n, H, Hkv, qw, kw, has_norm, eps, unit_offset, table,      \
+                           store_kv)
+#define QK_VEC(LL)                                                                                                 \
+    do {                                                                                                           \
+        if (hp == 4) { QK_VEC_HP(LL, 4); } else { QK_VEC_HP(LL, 1); }                                              \
+    } while (0)
+    if (D == 64) QK_VEC(8);
+    else if (D == 128) QK_VEC(16);
+    else if (D == 256) QK_VEC(32);
+    else if (D == 512) QK_VEC(64);
+    else return false;
+#undef QK_VEC
+#undef QK_VEC_HP
+    return true;
+}
+
+extern "C" int mv_store_v_pages(const void* qkv, long row_stride, int v_off, const int* positions,
+                                const int* token_seq, const int* block_table, int bt_width, int page_size,
+                                void* v_pages, int n, int Hkv, int D, int dtype, hipStream_t stream);
+
+// store_kv: 0 nothing goes to the cache; 1 keys and values, a store per token and head; 2 keys only;
+// 3 keys per token and head, values tile by tile (16 tokens of a kv head at a time, for steps of
+// many tokens), in the same launch where the vector kernel serves the shape.
+extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int k_off, int v_off,
+                                     const int* positions, const int* token_seq, const int* block_table,
+                                     int bt_width, int page_size, void* k_pages, void* v_pages, int n, int H,
+                                     int Hkv, int D, const void* q_weight, const void* k_weight, int weight_dtype,
+                                     float eps, int unit_offset, const float* table, int rot_dim, int interleaved,
+                                     int store_kv, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && Hkv >= 0 && D > 0, "qk_norm_rope_store: bad sizes n=%d H=%d Hkv=%d D=%d", n, H,
+               Hkv, D);
+    MV_REQUIRE(D <= MV_MAX_HEAD_DIM, "qk_norm_rope_store: head_dim %d exceeds the supported maximum %d", D,
+               MV_MAX_HEAD_DIM);
+    MV_REQUIRE(table == nullptr || (rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= D),
+               "qk_norm_rope_store: rotary dim %d must be even and at most head_dim %d", rot_dim, D);
+    MV_REQUIRE(!store_kv || (block_table && k_pages && v_pages && page_size > 0 && bt_width > 0),
+               "qk_norm_rope_store: cache write asked without pages or block table");
+    const int has_norm = q_weight != nullptr;
+    MV_REQUIRE(!has_norm || (k_weight != nullptr || !store_kv), "qk_norm_rope_store: q norm without k norm");
+    MV_REQUIRE(!has_norm || eps > 0.f, "qk_norm_rope_store: eps must be positive");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype), "qk_norm_rope_store: bad weight dtype %d", weight_dtype);
+    MV_REQUIRE(store_kv >= 0 && store_kv <= 3, "qk_norm_rope_store: bad cache mode %d", store_kv);
+    if (n == 0) return 0;
+    const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv >= 2 ? Hkv : 0));
+    WeightPtr qw{q_weight, weight_dtype}, kw{k_weight, weight_dtype};
+    // the vector kernel: rotation over the whole head in half-split pairs, everything 16-byte aligned
+    const size_t esz = dtype == MV_F32 ? 4 : 2;
+    const bool aligned = ((uintptr_t)qkv % 16) == 0 && (row_stride * esz) % 16 == 0 && (q_off * esz) % 16 == 0 &&
+                         (k_off * esz) % 16 == 0 && (v_off * esz) % 16 == 0 && ((uintptr_t)k_pages % 16) == 0 &&
+                         ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0 &&
+                         ((uintptr_t)table % 16) == 0;
+    if (aligned && (D == 64 || D == 128 || D == 256 || D == 512) && (table == nullptr || (rot_dim == D && !interleaved)) &&
+        (long)n * heads * (D / 8) < (1L << 31)) {
+        bool took = false;
+        MV_DISPATCH_T(dtype, "qk_norm_rope_store",
+                      took = launch_qk_vec<T>((T*)qkv, row_stride, q_off, k_off, v_off, positions, token_seq,
+                                              block_table, bt_width, page_size, (T*)k_pages, (T*)v_pages, n, H, Hkv, D,
+                                              qw, kw, has_norm, eps, unit_offset, table, store_kv, stream));
+        if (took) return mv_check_launch("qk_norm_rope_store");
+    }
+    dim3 grid(n, (heads + 3) / 4);
+    MV_DISPATCH_T(dtype, "qk_norm_rope_store",
+                  hipLaunchKernelGGL(qk_norm_rope_store_kernel<T>, grid, dim3(256), 0, stream, (T*)qkv, row_stride,
+                                     q_off, k_off, v_off, positions, token_seq, block_table, bt_width, page_size,
+                                     (T*)k_pages, (T*)v_pages, H, Hkv, D, qw, kw, has_norm, eps, unit_offset, table,
+                                     rot_dim, interleaved, store_kv == 3 ? 2 : store_kv));
+    if (int rc = mv_check_launch("qk_norm_rope_store")) return rc;
+    if (store_kv == 3)
+        return mv_store_v_pages(qkv, row_stride, v_off, positions, token_seq, block_table, bt_width, page_size, v_pages,
+                                n, Hkv, D, dtype, stream);
+    return 0;
+}
+
+// The value rows of a step as a launch of their own (one workgroup per 16 tokens and kv head).
+template <typename T>
+__global__ void __launch_bounds__(256)
+store_v_pages_kernel(const T* __restrict__ qkv, long row_stride, int v_off, const int* __restrict__ positions,
+                     const int* __restrict__ token_seq, const int* __restrict__ block_table, int bt_width,
+                     int page_size, T* __restrict__ v_pages, int n, int Hkv, int D) {
+    __shared__ float tile[16][MV_MAX_HEAD_DIM + 1];
+    __shared__ long dst_base[16];
+    store_v_tile<T, MV_MAX_HEAD_DIM + 1>(blockIdx.x * 16, blockIdx.y, qkv, row_stride, v_off, positions, token_seq,
+                                         block_table, bt_width, page_size, v_pages, n, Hkv, D, tile, dst_base);
 }
 
 extern "C" int mv_store_v_pages(const void* qkv, long row_stride, int v_off, const int* positions,

@@ -41,7 +41,7 @@ COMPUTE_UNITS = 256
 PREFILL_TWO_GROUPS_FROM = 1024
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
-# from this many tokens on, value rows are written to their pages by a kernel of their own
+# from this many tokens on, value rows are written to their pages 16 tokens of a kv head at a time
 STORE_V_SPLIT_TOKENS = 64
 
 
@@ -224,19 +224,14 @@ class Ops:
         q_dim = num_heads * head_dim
         kv_dim = num_kv_heads * head_dim
         stride = qkv.stride(0) if n > 1 else width
-        # with many tokens the values go to their transposed pages in a pass of their own, in
-        # which neighbouring tokens write neighbouring slots; with few, one launch does everything
-        split_v = store and n >= STORE_V_SPLIT_TOKENS
-        mode = 0 if not store else (2 if split_v else 1)
+        # with many tokens the values go to their transposed pages tile by tile, so that
+        # neighbouring tokens write neighbouring slots (mode 3); with few, a store per token and head
+        mode = 0 if not store else (3 if n >= STORE_V_SPLIT_TOKENS else 1)
         self.lib.call("mv_qk_norm_rope_store", qkv.data_ptr(), stride, 0, q_dim,
                       q_dim + kv_dim, positions.data_ptr(), token_seq.data_ptr(), _ptr(block_table), bt_width,
                       page_size, _ptr(k_pages), _ptr(v_pages), n, num_heads, num_kv_heads, head_dim,
                       _ptr(q_weight), _ptr(k_weight), wcode, float(eps), int(unit_offset), _ptr(rope_table), rot,
                       int(interleaved), mode, self.code, self._stream())
-        if split_v:
-            self.lib.call("mv_store_v_pages", qkv.data_ptr(), stride, q_dim + kv_dim, positions.data_ptr(),
-                          token_seq.data_ptr(), block_table.data_ptr(), bt_width, page_size, v_pages.data_ptr(), n,
-                          num_kv_heads, head_dim, self.code, self._stream())
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
         """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
