@@ -16,6 +16,11 @@ JSON line is printed:
                divided by its time, against 8 TB/s of HBM
   points       decode tokens/s at batch 1 and batch 64
 
+``--only serve`` runs a continuous-batching workload instead (``--requests`` requests, 256 by
+default, with prompt lengths uniform in 128..2048 and ``--gen-len`` generated tokens each, all
+submitted at once under a budget of ``--token-budget`` tokens a step) and prints its own line:
+generated tokens per second over the whole run, with the time of the run and the number of steps.
+
 Weights are seeded random tensors of the named shape and prompts are seeded uniform token ids
 (there is no network for checkpoints or datasets). The reference publishes no number for this
 metric, so ``vs_baseline`` is null.
@@ -56,7 +61,7 @@ def model_numbers(c, layers):
                 matrix_params=matrix_params, kv_bytes_per_token=layers * 2 * kv)
 
 
-def build_llm(args, shape, layers):
+def build_llm(args, shape, layers, max_seqs=None, token_budget=None, num_pages=None):
     import torch
     from minivllm_amd import LLM
     from minivllm_amd.config import EngineConfig
@@ -71,9 +76,10 @@ def build_llm(args, shape, layers):
     source = DeviceRandomSource(expected_tensors(arch, cfg), args.seed, stored, dev)
     pages_per_seq = -(-args.context // args.block_size)
     ec = EngineConfig(model="", dtype=args.dtype, max_model_len=args.context,
-                      max_num_batched_tokens=max(args.prefill_tokens, 2048), max_num_batched_seqs=max(64, args.batch),
+                      max_num_batched_tokens=token_budget or max(args.prefill_tokens, 2048),
+                      max_num_batched_seqs=max_seqs or max(64, args.batch),
                       kv_cache_block_size=args.block_size,
-                      kv_cache_num_blocks=max(64, args.batch) * pages_per_seq + 16,
+                      kv_cache_num_blocks=num_pages or max(64, args.batch) * pages_per_seq + 16,
                       use_cuda_graph=not args.no_graph, num_scheduler_steps=args.scheduler_steps, seed=args.seed)
     return LLM(config=ec, model_source=(arch, cfg, source)), cfg
 
@@ -134,6 +140,30 @@ def measure_prefill(llm, vocab, tokens, repeats, seed):
     return min(times[1:]) if repeats else times[0]
 
 
+def measure_serve(llm, vocab, requests, gen_len, seed):
+    """All requests submitted at once; returns (seconds, generated tokens, prompt tokens, steps, preemptions)."""
+    import numpy as np
+    import torch
+    from minivllm_amd import SamplingParams
+    rng = np.random.default_rng(seed)
+    prompts = [[int(t) for t in rng.integers(0, vocab, size=int(n))] for n in rng.integers(128, 2049, size=requests)]
+    # a few requests through every kind of step first (graphs are captured on first use)
+    llm.generate(prompts[:4], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
+    torch.cuda.synchronize()
+    sp = SamplingParams(temperature=0.0, max_tokens=gen_len, ignore_eos=True)
+    before = llm.scheduler.num_preemptions
+    reqs = [llm.submit(p, sp) for p in prompts]
+    steps = 0
+    t0 = time.perf_counter()
+    while llm.has_unfinished():
+        llm.step()
+        steps += 1
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return (dt, sum(r.num_completion_tokens for r in reqs), sum(len(p) for p in prompts), steps,
+            llm.scheduler.num_preemptions - before)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -152,8 +182,12 @@ def main() -> int:
                     help="decode steps run in a row on the device before the host looks at the tokens")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
-                    help="measure one phase alone (for profiling); the line then lacks the other's fields")
+    ap.add_argument("--only", "--mode", dest="only", choices=["all", "decode", "prefill", "serve"], default="all",
+                    help="measure one phase alone (for profiling); the line then lacks the other's fields. "
+                         "'serve': the continuous-batching workload")
+    ap.add_argument("--requests", type=int, default=256, help="requests of the serve workload")
+    ap.add_argument("--gen-len", type=int, default=256, help="generated tokens per request of the serve workload")
+    ap.add_argument("--token-budget", type=int, default=8192, help="tokens per step of the serve workload")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -166,6 +200,27 @@ def main() -> int:
     shape = SHAPES[args.shape]
     layers_full = shape["num_hidden_layers"]
     layers = args.layers or layers_full
+    if args.only == "serve":
+        if 2048 + args.gen_len > args.context:
+            print(f"bench.py: prompts of up to 2048 tokens + {args.gen_len} generated exceed the context {args.context}")
+            return 2
+        pages = args.requests * (-(-(2048 + args.gen_len) // args.block_size) + 1) + 64
+        llm, cfg = build_llm(args, shape, layers, max_seqs=min(256, args.requests), token_budget=args.token_budget,
+                             num_pages=pages)
+        dt, gen, prompt, steps, preempted = measure_serve(llm, cfg.vocab_size, args.requests, args.gen_len, args.seed)
+        print(json.dumps({
+            "metric": "generated tok/s, continuous batching (%d requests, prompts 128..2048, %d generated each)"
+                      % (args.requests, args.gen_len),
+            "value": round(gen / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+            "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": {"model": f"qwen3-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
+                       "requests": args.requests, "gen_len": args.gen_len, "token_budget": args.token_budget,
+                       "seq_len": args.context, "block_size": args.block_size, "graph": not args.no_graph,
+                       "scheduler_steps": args.scheduler_steps, "parallelism": "single-gpu"},
+            "seconds": round(dt, 3), "prompt_tokens": prompt, "generated_tokens": gen,
+            "total_tok_s": round((gen + prompt) / dt, 1), "preemptions": preempted}))
+        return 0
     llm, cfg = build_llm(args, shape, layers)
     nums = model_numbers(shape, layers)
     item = 2 if args.dtype == "bfloat16" else 4
