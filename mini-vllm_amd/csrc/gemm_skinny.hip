@@ -55,7 +55,8 @@ struct NormInput {
 template <int R, int TM, bool SWIGLU, bool NORM, typename TC>
 __global__ void __launch_bounds__(64 * SK_MAX_WAVES)
 gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W, const bf16* __restrict__ bias,
-                   TC* __restrict__ C, long ldc, int M, int N, int K, int groups, int blocks, NormInput norm) {
+                   TC* __restrict__ C, long ldc, int M, int N, int K, int groups, int blocks, int rows,
+                   NormInput norm) {
     extern __shared__ float red[];  // [S - 1][R * TM][64][4], then (NORM) bf16 [M][K + 8]
     // The tokens may be dealt out to `groups` workgroups per weight tile (16 * TM tokens each): with
     // few weight tiles that fills more compute units, and each unit pulls fewer activation rows.
@@ -78,8 +79,11 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     const int lane = threadIdx.x % MV_WAVE;
     const int i = lane % 16;
     const int g = lane / 16;
-    // output columns of this workgroup: SWIGLU -> 16 columns of I = N; else 16 * R columns of N
-    const int n_base = SWIGLU ? block * 16 : block * 16 * R;
+    // output columns of this workgroup (SWIGLU: of I = N, at most 16): `rows` of them (at most 16 * R; fewer where that makes the
+    // workgroups a whole number of rounds of the chip: the rows of a tile beyond them are loaded
+    // again from the last one and never stored)
+    const int n_base = block * rows;
+    const int n_end = n_base + rows < N ? n_base + rows : N;
 
     const int ksteps = K / 32;
     const int per = ksteps / S, rem = ksteps % S;
@@ -92,11 +96,11 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
         int row;
         if (SWIGLU) {
             int col = n_base + i;
-            if (col > N - 1) col = N - 1;
+            if (col > n_end - 1) col = n_end - 1;
             row = r == 0 ? col : N + col;  // gate rows [0, N), up rows [N, 2N)
         } else {
             row = n_base + 16 * r + i;
-            if (row > N - 1) row = N - 1;  // rows past the end are loaded again and never stored
+            if (row > n_end - 1) row = n_end - 1;  // rows past the end are loaded again and never stored
         }
         wrow[r] = reinterpret_cast<const uint4*>(W + (size_t)row * K) + g;
     }
@@ -306,7 +310,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int col = n_base + 4 * g + e;
-                if (col >= N) continue;
+                if (col >= n_end) continue;
                 const float gate = acc[0][t][e], up = acc[R - 1][t][e];
                 store_c<TC>(C + (size_t)tok * ldc + col, gate / (1.f + expf(-gate)) * up);
             }
@@ -321,7 +325,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int col = n_base + 16 * r + 4 * g + e;
-                    if (col >= N) continue;
+                    if (col >= n_end) continue;
                     float v = acc[r][t][e];
                     if (bias) v += to_f(bias[col]);
                     store_c<TC>(C + (size_t)tok * ldc + col, v);
@@ -336,32 +340,50 @@ static size_t skinny_lds_bytes(int S, int R, int TM, bool with_norm, int M, int 
     return lds;
 }
 
-static int skinny_blocks(int N, int R, bool swiglu) {
-    const int tiles = (N + 15) / 16;
-    return swiglu ? tiles : (tiles + R - 1) / R;
+static int skinny_blocks(int N, int rows) { return (N + rows - 1) / rows; }
+
+// Output columns per workgroup when there are few tiles and few tokens. The chip takes the
+// workgroups in rounds of one per compute unit, and a last round that is not full costs as much as
+// a full one (320 tiles on 256 units: two rounds for the work of 1.25). So a workgroup takes 8 to
+// `most` columns, not a whole number of tiles, such that the rounds are as few and as full as
+// possible: rounds * columns is what a unit streams. (The rows of a tile beyond the workgroup's
+// own are loaded again from its last row.) Of equal choices the largest: fewer workgroups read
+// the tokens.
+static int pick_rows(int N, int most) {
+    int rows = most;
+    long best = -1;
+    for (int p = most; p >= 8; p -= 4) {
+        const long wgs = (N + p - 1) / p;
+        const long cost = ((wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS) * p;
+        if (best < 0 || cost < best) {
+            best = cost;
+            rows = p;
+        }
+    }
+    return rows;
 }
 
 template <int R, int TM, bool SWIGLU, typename TC>
 static void launch_skinny(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N,
-                          int K, int S, hipStream_t stream) {
-    const int blocks = skinny_blocks(N, R, SWIGLU);
+                          int K, int S, int rows, hipStream_t stream) {
+    const int blocks = skinny_blocks(N, rows);
     const int groups = (M + 16 * TM - 1) / (16 * TM);
     const int grid = groups > 1 ? (blocks + 7) / 8 * 8 * groups : blocks;
     const size_t lds = skinny_lds_bytes(S, R, TM, false, M, K);
     hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC>), dim3(grid), dim3(64 * S), lds, stream,
                        (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, groups, blocks,
-                       NormInput{});
+                       rows, NormInput{});
 }
 
 template <int R, bool SWIGLU, typename TC>
 static void launch_skinny_norm(const NormInput& norm, const void* W, const void* bias, void* C, long ldc, int M, int N,
                                int K, int S, hipStream_t stream) {
-    const int tiles = (N + 15) / 16;
-    const int blocks = SWIGLU ? tiles : (tiles + R - 1) / R;
+    const int rows = pick_rows(N, 16);     // (R == 1, or the gated pair of one tile each)
+    const int blocks = skinny_blocks(N, rows);
     const size_t lds = skinny_lds_bytes(S, R, 1, true, M, K);
     hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC>), dim3(blocks), dim3(64 * S), lds, stream,
                        (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, 1, blocks,
-                       norm);
+                       rows, norm);
 }
 
 static int pick_waves(int K) {
@@ -373,12 +395,12 @@ static int pick_waves(int K) {
 
 template <int R, bool SWIGLU, typename TC>
 static int dispatch_tm(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N, int K,
-                       int S, hipStream_t stream) {
+                       int S, int rows, hipStream_t stream) {
     // Token tiles per workgroup: all of them (the weights pass each compute unit once), or fewer
     // with the tokens dealt out to several workgroups per weight tile. A compute unit pulls
     // R + TM operand rows of 16 per workgroup it runs; the choice with the least per unit wins.
     const int tiles_m = (M + 15) / 16;
-    const int blocks = skinny_blocks(N, R, SWIGLU);
+    const int blocks = skinny_blocks(N, rows);
     int best_tm = tiles_m < 4 ? tiles_m : 4;
     long best_cost = -1;
     for (int tm = best_tm; tm >= 1; --tm) {
@@ -390,10 +412,10 @@ static int dispatch_tm(const void* A, long lda, const void* W, const void* bias,
             best_tm = tm;
         }
     }
-    if (best_tm == 1) launch_skinny<R, 1, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-    else if (best_tm == 2) launch_skinny<R, 2, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-    else if (best_tm == 3) launch_skinny<R, 3, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-    else launch_skinny<R, 4, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
+    if (best_tm == 1) launch_skinny<R, 1, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+    else if (best_tm == 2) launch_skinny<R, 2, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+    else if (best_tm == 3) launch_skinny<R, 3, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+    else launch_skinny<R, 4, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
     return 0;
 }
 
@@ -420,15 +442,20 @@ extern "C" int mv_gemm_skinny(const void* A, long lda, const void* W, long ldw, 
     // and the partial tiles of the waves within 56 KiB of LDS
     int R = tiles >= 2048 ? 4 : (tiles >= 1024 ? 2 : 1);
     while (R > 1 && (size_t)(S - 1) * R * TM * 1024 > 56 * 1024) R /= 2;
+    int rows = 16 * R;
+    if (R == 1 && M <= 16) {
+        rows = pick_rows(N, 32);
+        R = rows > 16 ? 2 : 1;
+    }
     int rc = 0;
     if (c_dtype == MV_F32) {
-        if (R == 4) rc = dispatch_tm<4, false, float>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-        else if (R == 2) rc = dispatch_tm<2, false, float>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-        else rc = dispatch_tm<1, false, float>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
+        if (R == 4) rc = dispatch_tm<4, false, float>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+        else if (R == 2) rc = dispatch_tm<2, false, float>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+        else rc = dispatch_tm<1, false, float>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
     } else {
-        if (R == 4) rc = dispatch_tm<4, false, bf16>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-        else if (R == 2) rc = dispatch_tm<2, false, bf16>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
-        else rc = dispatch_tm<1, false, bf16>(A, lda, W, bias, C, ldc, M, N, K, S, stream);
+        if (R == 4) rc = dispatch_tm<4, false, bf16>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+        else if (R == 2) rc = dispatch_tm<2, false, bf16>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+        else rc = dispatch_tm<1, false, bf16>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
     }
     if (rc) return rc;
     return mv_check_launch("gemm_skinny");
@@ -440,7 +467,7 @@ extern "C" int mv_gemm_skinny_swiglu(const void* A, long lda, const void* Wgu, v
     if (int rc = check_skinny("gemm_skinny_swiglu", A, lda, Wgu, ldo, M, I, K)) return rc;
     if (M == 0) return 0;
     const int S = pick_waves(K);
-    int rc = dispatch_tm<2, true, bf16>(A, lda, Wgu, nullptr, out, ldo, M, I, K, S, stream);
+    int rc = dispatch_tm<2, true, bf16>(A, lda, Wgu, nullptr, out, ldo, M, I, K, S, M <= 16 ? pick_rows(I, 16) : 16, stream);
     if (rc) return rc;
     return mv_check_launch("gemm_skinny_swiglu");
 }
