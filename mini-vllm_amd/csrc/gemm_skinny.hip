@@ -82,8 +82,11 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     // output columns of this workgroup (SWIGLU: of I = N, at most 16): `rows` of them (at most 16 * R; fewer where that makes the
     // workgroups a whole number of rounds of the chip: the rows of a tile beyond them are loaded
     // again from the last one and never stored)
-    const int n_base = block * rows;
-    const int n_end = n_base + rows < N ? n_base + rows : N;
+    // (The variant with the norm in front keeps whole tiles: more workgroups would each pay its
+    // prologue, and the extra registers would cost it a wave per SIMD.)
+    const int own = NORM ? (SWIGLU ? 16 : 16 * R) : rows;
+    const int n_base = block * own;
+    const int n_end = n_base + own < N ? n_base + own : N;
 
     const int ksteps = K / 32;
     const int per = ksteps / S, rem = ksteps % S;
@@ -378,7 +381,7 @@ static void launch_skinny(const void* A, long lda, const void* W, const void* bi
 template <int R, bool SWIGLU, typename TC>
 static void launch_skinny_norm(const NormInput& norm, const void* W, const void* bias, void* C, long ldc, int M, int N,
                                int K, int S, hipStream_t stream) {
-    const int rows = pick_rows(N, 16);     // (R == 1, or the gated pair of one tile each)
+    const int rows = SWIGLU ? 16 : 16 * R;
     const int blocks = skinny_blocks(N, rows);
     const size_t lds = skinny_lds_bytes(S, R, 1, true, M, K);
     hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC>), dim3(blocks), dim3(64 * S), lds, stream,
