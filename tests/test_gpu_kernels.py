@@ -573,8 +573,11 @@ def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_ro
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 70, 96), (8, 1024, 1024), (17, 4100, 64), (64, 333, 3072), (33, 2048, 512),
-                                    (5, 151936 // 8, 1024)])
+                                    (5, 151936 // 8, 1024), (5, 5120, 256), (16, 6144, 128), (3, 330, 64)])
 def test_gemm_weight_streaming(out_dtype, M, N, K):
+    """The weight-streaming product, also at sizes where a workgroup takes a number of output
+    columns that is no multiple of a tile (5120 and 6144 columns: 20 and 24 each; 330: 8, the last
+    workgroup two)."""
     ops = ops_for(torch.bfloat16)
     g = torch.Generator().manual_seed(17)
     a = torch.randn(M, K, generator=g).to(torch.bfloat16)
