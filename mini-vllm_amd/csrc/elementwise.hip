@@ -106,10 +106,23 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
 // of 256 serves 256 / TPR rows), each keeps its chunks of eight columns in registers between the
 // sum of squares and the scaling, so a row is read once.
 #define ARN_MAX_CHUNKS 4
-template <typename T>
+// A delta that is still the partial sums of a product whose K was split over workgroups:
+// delta[m][n] = round_T(sum over f < F of part[f * plane + m * h + n] (+ bias[n])), the sum taken
+// in that order and rounded to the activation type as the kernel that adds them up would.
+struct SplitDelta {
+    const float* part;
+    int F;
+    long plane;
+    const bf16* bias;
+};
+
+// SPLIT: the delta is given as `split` (then `delta` is null); a variant of its own, so that the
+// plain one keeps its few registers.
+template <typename T, bool SPLIT>
 __global__ void __launch_bounds__(256)
-add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta, WeightPtr w, float eps, int unit_offset,
-                       T* __restrict__ out, const int* __restrict__ rows, int n_out, int h, int tpr) {
+add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta, SplitDelta split, WeightPtr w,
+                       float eps, int unit_offset, T* __restrict__ out, const int* __restrict__ rows, int n_out, int h,
+                       int tpr) {
     __shared__ float part[256 / MV_WAVE];
     const int rpb = 256 / tpr;                        // rows of this block
     const int sub = threadIdx.x / tpr, t = threadIdx.x % tpr;
@@ -118,6 +131,38 @@ add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta, W
     const int r = live ? (rows ? rows[i] : i) : -1;
     float x[ARN_MAX_CHUNKS][8];
     float ss = 0.f;
+    // the partial sums of a split product first: four planes of all the thread's chunks are asked
+    // for at a time (the loads of one plane after the other would each wait for the last), and
+    // added in the order of the planes
+    float sum[SPLIT ? ARN_MAX_CHUNKS : 1][8];
+    if (SPLIT && r >= 0) {
+#pragma unroll
+        for (int c = 0; c < ARN_MAX_CHUNKS; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sum[c][e] = 0.f;
+        const float* pr = split.part + (size_t)r * h;
+        for (int f0 = 0; f0 < split.F; f0 += 4) {
+            float dv[4][ARN_MAX_CHUNKS][8];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int c = 0; c < ARN_MAX_CHUNKS; ++c) {
+                    const int d = (c * tpr + t) * 8;
+                    if (d < h && f0 + u < split.F) {
+                        Vec8<float>::load(pr + (size_t)(f0 + u) * split.plane + d, dv[u][c]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) dv[u][c][e] = 0.f;   // (adding +0 changes nothing)
+                    }
+                }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int c = 0; c < ARN_MAX_CHUNKS; ++c)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sum[c][e] += dv[u][c][e];
+        }
+    }
     if (r >= 0) {
         float* xr = resid + (size_t)r * h;
         const T* dl = delta ? delta + (size_t)r * h : nullptr;
@@ -131,6 +176,13 @@ add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta, W
                     Vec8<T>::load(dl + d, dv);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) x[c][e] += dv[e];
+                } else if (SPLIT) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float v = sum[SPLIT ? c : 0][e];
+                        if (split.bias) v += to_f(split.bias[d + e]);
+                        x[c][e] += to_f(from_f<T>(v));
+                    }
                 }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) ss += x[c][e] * x[c][e];
@@ -154,7 +206,7 @@ add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta, W
         return;
     }
     const float rinv = rsqrtf(ss / (float)h + eps);
-    const bool write_back = rows == nullptr && delta != nullptr;
+    const bool write_back = rows == nullptr && (delta != nullptr || SPLIT);
 #pragma unroll
     for (int c = 0; c < ARN_MAX_CHUNKS; ++c) {
         const int d = (c * tpr + t) * 8;
@@ -187,14 +239,44 @@ extern "C" int mv_add_rmsnorm(float* resid, const void* delta, const void* weigh
         while (tpr < 256 && tpr * 8 * 2 <= h) tpr *= 2;
         const int rpb = 256 / tpr;
         MV_DISPATCH_T(dtype, "add_rmsnorm",
-                      hipLaunchKernelGGL(add_rmsnorm_vec_kernel<T>, dim3((n_out + rpb - 1) / rpb), dim3(256), 0, stream,
-                                         resid, (const T*)delta, w, eps, unit_offset, (T*)out, rows, n_out, h, tpr));
+                      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, false>), dim3((n_out + rpb - 1) / rpb), dim3(256), 0, stream,
+                                         resid, (const T*)delta, SplitDelta{nullptr, 0, 0, nullptr}, w, eps, unit_offset,
+                                         (T*)out, rows, n_out, h, tpr));
         return mv_check_launch("add_rmsnorm");
     }
     MV_DISPATCH_T(dtype, "add_rmsnorm",
                   hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(256), 0, stream, resid,
                                      (const T*)delta, w, eps, unit_offset, (T*)out, rows, h));
     return mv_check_launch("add_rmsnorm");
+}
+
+// The same with a delta that is still the F partial sums of a product (see SplitDelta): the kernel
+// that would add them up and round is saved. Returns 2 (and sets the error text) when the sizes
+// are not served by the vector kernel; the caller then adds the sums up first.
+extern "C" int mv_add_rmsnorm_split(float* resid, const float* part, int F, long plane, const void* bias,
+                                    const void* weight, int weight_dtype, float eps, int unit_offset, void* out,
+                                    const int* rows, int n_out, int h, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n_out >= 0 && h > 0 && F > 0 && part != nullptr && plane >= (long)h,
+               "add_rmsnorm_split: bad sizes n=%d h=%d F=%d", n_out, h, F);
+    MV_REQUIRE(out != nullptr && weight != nullptr, "add_rmsnorm_split: the norm's output and weight are needed");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype), "add_rmsnorm_split: bad weight dtype %d", weight_dtype);
+    MV_REQUIRE(eps > 0.f, "add_rmsnorm_split: eps must be positive");
+    if (n_out == 0) return 0;
+    if (!(h % 8 == 0 && h <= 8 * 256 * ARN_MAX_CHUNKS && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)part % 16) == 0 &&
+          (plane * sizeof(float)) % 16 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)weight % 16) == 0)) {
+        mv_fail("add_rmsnorm_split: rows of %d are not served", h);
+        return 2;
+    }
+    WeightPtr w{weight, weight_dtype};
+    int tpr = 64;
+    while (tpr < 256 && tpr * 8 * 2 <= h) tpr *= 2;
+    const int rpb = 256 / tpr;
+    const SplitDelta split{part, F, plane, (const bf16*)bias};
+    MV_DISPATCH_T(dtype, "add_rmsnorm_split",
+                  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, true>), dim3((n_out + rpb - 1) / rpb), dim3(256), 0, stream,
+                                     resid, (const T*)nullptr, split, w, eps, unit_offset, (T*)out, rows, n_out, h,
+                                     tpr));
+    return mv_check_launch("add_rmsnorm_split");
 }
 
 // Plain RMSNorm over the last dimension of a strided [n, h] view.

@@ -245,17 +245,20 @@ extern "C" long mv_gemm_mid_workspace(int M, int N, int K) {
     return (long)p.F * M * N;
 }
 
-// c_dtype: MV_BF16 or MV_F32. With `swiglu`, W is the packed gate/up weight [N = 2 I, K] and C is
-// [M, I]. `work` holds at least mv_gemm_mid_workspace(M, N, K) floats.
-extern "C" int mv_gemm_mid(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int c_dtype,
-                           int M, int N, int K, int swiglu, float* work, long work_floats, hipStream_t stream) {
+// The number of partial sums a product with an [N, K] weight is split into.
+extern "C" int mv_gemm_mid_splits(int N, int K) {
+    if (N <= 0 || K <= 0 || K % GM_KC) return 0;
+    return mid_plan(N, K).F;
+}
+
+// The first half alone: the partial sums work[f][m][n], f < mv_gemm_mid_splits(N, K), of
+// A[M, K] * W[N, K]^T. `work` holds at least mv_gemm_mid_workspace(M, N, K) floats.
+extern "C" int mv_gemm_mid_sums(const void* A, long lda, const void* W, int M, int N, int K, float* work,
+                                long work_floats, hipStream_t stream) {
     MV_REQUIRE(M > 0 && M <= 64, "gemm_mid: takes 1 to 64 rows, got M=%d", M);
     MV_REQUIRE(N > 0 && K > 0 && K % GM_KC == 0, "gemm_mid: K=%d must be a positive multiple of %d (N=%d)", K, GM_KC, N);
     MV_REQUIRE(lda >= K && lda % 8 == 0, "gemm_mid: lda=%ld must be a multiple of 8 and at least K=%d", lda, K);
     MV_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_mid: operands must be 16-byte aligned");
-    MV_REQUIRE(!swiglu || (N % 2 == 0 && bias == nullptr), "gemm_mid: the gated form takes an even N and no bias");
-    MV_REQUIRE(ldc >= (swiglu ? N / 2 : N), "gemm_mid: ldc=%ld too small for N=%d", ldc, N);
-    MV_REQUIRE(c_dtype == MV_F32 || c_dtype == MV_BF16, "gemm_mid: bad output dtype %d", c_dtype);
     const MidPlan p = mid_plan(N, K);
     MV_REQUIRE(work != nullptr && ((uintptr_t)work % 16) == 0 && work_floats >= (long)p.F * M * N,
                "gemm_mid: the work area holds %ld floats, %ld are needed", work_floats, (long)p.F * M * N);
@@ -276,14 +279,31 @@ extern "C" int mv_gemm_mid(const void* A, long lda, const void* W, const void* b
         else GM_LAUNCH(1, 4);
     }
 #undef GM_LAUNCH
-    if (int rc = mv_check_launch("gemm_mid")) return rc;
+    return mv_check_launch("gemm_mid");
+}
+
+// The second half alone: C = sum over f < F of work[f] (+ bias), or the gated activation of the two
+// halves of the sum. c_dtype: MV_BF16 or MV_F32.
+extern "C" int mv_gemm_mid_reduce(const float* work, const void* bias, void* C, long ldc, int c_dtype, int M, int N,
+                                  int F, int swiglu, hipStream_t stream) {
+    MV_REQUIRE(M > 0 && N > 0 && F > 0 && work != nullptr && C != nullptr, "gemm_mid: bad sizes M=%d N=%d F=%d", M, N, F);
+    MV_REQUIRE(!swiglu || (N % 2 == 0 && bias == nullptr), "gemm_mid: the gated form takes an even N and no bias");
+    MV_REQUIRE(ldc >= (swiglu ? N / 2 : N), "gemm_mid: ldc=%ld too small for N=%d", ldc, N);
+    MV_REQUIRE(c_dtype == MV_F32 || c_dtype == MV_BF16, "gemm_mid: bad output dtype %d", c_dtype);
     const long total = (long)M * (swiglu ? N / 2 : N);
     const unsigned blocks = (unsigned)((total + 255) / 256);
     if (c_dtype == MV_F32)
         hipLaunchKernelGGL(gemm_mid_reduce_kernel<float>, dim3(blocks), dim3(256), 0, stream, work, (const bf16*)bias,
-                           (float*)C, ldc, M, N, p.F, swiglu);
+                           (float*)C, ldc, M, N, F, swiglu);
     else
         hipLaunchKernelGGL(gemm_mid_reduce_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, work, (const bf16*)bias,
-                           (bf16*)C, ldc, M, N, p.F, swiglu);
+                           (bf16*)C, ldc, M, N, F, swiglu);
     return mv_check_launch("gemm_mid (reduce)");
+}
+
+// Both halves. With `swiglu`, W is the packed gate/up weight [N = 2 I, K] and C is [M, I].
+extern "C" int mv_gemm_mid(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int c_dtype,
+                           int M, int N, int K, int swiglu, float* work, long work_floats, hipStream_t stream) {
+    if (int rc = mv_gemm_mid_sums(A, lda, W, M, N, K, work, work_floats, stream)) return rc;
+    return mv_gemm_mid_reduce(work, bias, C, ldc, c_dtype, M, N, mid_plan(N, K).F, swiglu, stream);
 }

@@ -54,6 +54,14 @@ _OPTIONAL_SIGNATURES = {
     "mv_gemm_skinny_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
                                     c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_mid_workspace": (c_long, [c_int, c_int, c_int]),
+    "mv_gemm_mid_splits": (c_int, [c_int, c_int]),
+    # A, lda, W, M, N, K, work, work_floats, stream
+    "mv_gemm_mid_sums": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_void_p]),
+    # work, bias, C, ldc, c_dtype, M, N, F, swiglu, stream
+    "mv_gemm_mid_reduce": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    # resid, part, F, plane, bias, weight, weight_dtype, eps, unit_offset, out, rows, n_out, h, dtype, stream
+    "mv_add_rmsnorm_split": (c_int, [c_void_p, c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_float, c_int,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     # A, lda, W, bias, C, ldc, c_dtype, M, N, K, swiglu, work, work_floats, stream
     "mv_gemm_mid": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                             c_void_p, c_long, c_void_p]),

@@ -69,6 +69,34 @@ def _weight_code(w: torch.Tensor, what: str) -> int:
     return code
 
 
+class SplitSum:
+    """The output of a matrix product that exists only as the float partial sums of its splits of K
+    so far: ``out[m, n] = round(sum_f work[f, m, n] + bias[n])``. The next residual add + norm can
+    take it as its delta and add the sums up itself (``Ops.add_rmsnorm``), which saves the kernel
+    that would; anything else calls ``materialize``. The sums live in the work area all such
+    products share, so the next of them adds this one up first if nobody has asked for it yet."""
+
+    def __init__(self, ops: "Ops", out: torch.Tensor, work: torch.Tensor, splits: int, bias: Optional[torch.Tensor]):
+        self.ops, self.out, self.work, self.splits, self.bias = ops, out, work, splits, bias
+        self.shape = out.shape
+        self.done = False          # the sums were added up into ``out``, or are no longer needed
+
+    def materialize(self) -> torch.Tensor:
+        if not self.done:
+            M, N = self.out.shape
+            self.ops.lib.call("mv_gemm_mid_reduce", self.work.data_ptr(), _ptr(self.bias), self.out.data_ptr(),
+                              self.out.stride(0) if M > 1 else N, _CODES[self.out.dtype], M, N, self.splits, 0,
+                              self.ops._stream())
+            self.discard()
+        return self.out
+
+    def discard(self) -> None:
+        """The sums will not be asked for again (they were consumed, or the step is over)."""
+        self.done = True
+        if self.ops._split_pending is self:
+            self.ops._split_pending = None
+
+
 class Ops:
     def __init__(self, dtype: torch.dtype):
         if dtype not in _CODES:
@@ -85,6 +113,7 @@ class Ops:
         self.stream_handle: Optional[int] = None
         self._transposed = {}
         self._mid_work: Optional[torch.Tensor] = None
+        self._split_pending: Optional[SplitSum] = None     # partial sums in the work area nobody has used yet
         self._mid_retired: list = []
         self._sample_work: Optional[torch.Tensor] = None
 
@@ -129,6 +158,10 @@ class Ops:
         if resid.dtype != torch.float32 or resid.dim() != 2 or not resid.is_contiguous():
             raise KernelLibraryError("add_rmsnorm: the residual must be a contiguous float32 [n, h]")
         n, h = resid.shape
+        if isinstance(delta, SplitSum):
+            if self._add_rmsnorm_split(resid, delta, weight, eps, out, rows, unit_offset):
+                return
+            delta = delta.materialize()
         if delta is not None:
             self._act(delta, "delta")
             if delta.shape != resid.shape or not delta.is_contiguous():
@@ -152,6 +185,25 @@ class Ops:
                 raise KernelLibraryError(f"add_rmsnorm: output {tuple(out.shape)} does not fit [{n_out}, {h}]")
         self.lib.call("mv_add_rmsnorm", resid.data_ptr(), _ptr(delta), _ptr(weight), wcode, float(eps),
                       int(unit_offset), _ptr(out), _ptr(rows), n_out, h, self.code, self._stream())
+
+    def _add_rmsnorm_split(self, resid: torch.Tensor, delta: "SplitSum", weight: Optional[torch.Tensor], eps: float,
+                           out: Optional[torch.Tensor], rows: Optional[torch.Tensor], unit_offset: bool) -> bool:
+        """add + norm straight from a product's partial sums; False (nothing done) when the sizes
+        are not served. With ``rows`` the delta stays pending in the stream, so the sums are kept."""
+        n, h = resid.shape
+        if (delta.done or out is None or weight is None or tuple(delta.shape) != (n, h) or h % 8 or h > 8192
+                or out.dtype != self.dtype or out.dim() != 2 or out.shape[1] != h or not out.is_contiguous()
+                or not weight.is_contiguous() or weight.numel() != h or weight.data_ptr() % 16
+                or (rows is not None and (rows.dtype != torch.int32 or out.shape[0] < rows.numel()))
+                or (rows is None and out.shape[0] < n)):
+            return False
+        n_out = n if rows is None else rows.numel()
+        self.lib.call("mv_add_rmsnorm_split", resid.data_ptr(), delta.work.data_ptr(), delta.splits, n * h,
+                      _ptr(delta.bias), weight.data_ptr(), _weight_code(weight, "norm weight"), float(eps),
+                      int(unit_offset), out.data_ptr(), _ptr(rows), n_out, h, self.code, self._stream())
+        if rows is None:
+            delta.discard()
+        return True
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
                 unit_offset: bool = False) -> None:
@@ -243,8 +295,13 @@ class Ops:
 
     # ------------------------------------------------------------------------------------
     def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
-             exact: bool = False) -> None:
+             exact: bool = False, defer_sum: bool = False) -> Optional["SplitSum"]:
         """out[M, N] = a[M, K] @ w[N, K]^T (+ bias). ``out`` is the activation type or float32.
+
+        With ``defer_sum`` the caller can take a ``SplitSum`` instead of the finished ``out``: when
+        the product runs on the kernel that splits K, its partial sums are left to whoever uses the
+        result (a residual add + norm adds them up on the way; ``materialize()`` gives ``out``).
+        The return value is that object, or None when ``out`` is complete.
 
         float32 compute always takes the exact kernel. bfloat16 compute takes the
         weight-streaming MFMA kernel for up to SKINNY_MAX_M rows, the library's matrix product
@@ -255,7 +312,7 @@ class Ops:
         the product run as one kernel when the step has at most 16 rows, else the norm runs first."""
         if not isinstance(a, torch.Tensor):
             if not exact and self._gemm_fused_norm(a, w, out, bias, swiglu=False):
-                return
+                return None
             a = a.materialize()
         self._act(a, "gemm input"); _dev(w, "gemm weight"); _dev(out, "gemm output")
         if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
@@ -274,13 +331,15 @@ class Ops:
             if bias.dtype != w.dtype or bias.numel() != N:
                 raise KernelLibraryError("gemm: the bias must have the weight's dtype and N elements")
         if M == 0:
-            return
+            return None
         lda = a.stride(0) if M > 1 else K
         ldc = out.stride(0) if M > 1 else N
         fast = self.use_fast_kernels and not exact and wcode == DTYPE_BF16
         if fast and K % 32 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.lib.has("mv_gemm_skinny"):
-            if self._gemm_mid(a, lda, w, bias, out, ldc, M, N, K, swiglu=False):
-                return
+            done = self._gemm_mid(a, lda, w, bias, out, ldc, M, N, K, swiglu=False,
+                                  defer_sum=defer_sum and out.dtype == self.dtype and out.is_contiguous())
+            if done:
+                return done if isinstance(done, SplitSum) else None
             if M <= SKINNY_MAX_M or out.dtype == torch.float32 or not self._library_allowed(M, N, K, bias is not None):
                 # more rows than one workgroup takes are dealt out to groups of workgroups by the kernel
                 for m0 in range(0, M, SKINNY_LAUNCH_ROWS):
@@ -355,9 +414,10 @@ class Ops:
             return False
 
     def _gemm_mid(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                  ldc: int, M: int, N: int, K: int, swiglu: bool) -> bool:
+                  ldc: int, M: int, N: int, K: int, swiglu: bool, defer_sum: bool = False):
         """The kernel for up to 64 rows against a large weight (activation rows shared through LDS,
-        K split over workgroups); False when the shape is left to the weight-streaming kernel."""
+        K split over workgroups); False when the shape is left to the weight-streaming kernel.
+        With ``defer_sum`` the partial sums are not added up: a ``SplitSum`` is returned."""
         if not (self.wants_mid(M, N, K) and self.lib.has("mv_gemm_mid")):
             return False
         need = int(self.lib.dll.mv_gemm_mid_workspace(M, N, K))
@@ -366,9 +426,19 @@ class Ops:
         if self._mid_work is None or self._mid_work.numel() < need:
             if torch.cuda.is_current_stream_capturing():
                 return False                                   # no allocation inside a capture
+            if self._split_pending is not None:
+                self._split_pending.materialize()
             if self._mid_work is not None:
                 self._mid_retired.append(self._mid_work)       # captured graphs may hold its address
             self._mid_work = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=a.device)
+        if self._split_pending is not None:
+            self._split_pending.materialize()                  # its sums are about to be overwritten
+        if defer_sum and not swiglu and self.lib.has("mv_add_rmsnorm_split"):
+            self.lib.call("mv_gemm_mid_sums", a.data_ptr(), lda, w.data_ptr(), M, N, K, self._mid_work.data_ptr(),
+                          self._mid_work.numel(), self._stream())
+            pending = SplitSum(self, out, self._mid_work, int(self.lib.dll.mv_gemm_mid_splits(N, K)), bias)
+            self._split_pending = pending
+            return pending
         self.lib.call("mv_gemm_mid", a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(), ldc,
                       _CODES[out.dtype], M, N, K, int(swiglu), self._mid_work.data_ptr(), self._mid_work.numel(),
                       self._stream())
@@ -408,6 +478,8 @@ class Ops:
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N):
             return False
         resid_in, delta, resid_out = pending.fused()
+        if isinstance(delta, SplitSum):
+            delta = delta.materialize()
         self.lib.call("mv_gemm_skinny_norm", resid_in.data_ptr(), _ptr(delta), _ptr(resid_out), weight.data_ptr(),
                       _weight_code(weight, "norm weight"), float(spec.eps), int(spec.unit_offset), w.data_ptr(),
                       _ptr(bias), out.data_ptr(), out.stride(0) if M > 1 else N, _CODES[out.dtype], M, N, K,

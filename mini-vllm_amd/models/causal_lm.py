@@ -155,7 +155,14 @@ class CausalLM:
         m = ctx.n_logit_rows
         logits = rt.workspace.get("logits", (m, plan.vocab_size), torch.float32)
         if m == 0:
+            discard = getattr(stream.delta, "discard", None)
+            if discard is not None:
+                discard()
             return logits
         h = self.final_norm.forward(stream, ctx, rows=ctx.logit_rows, tag="final_normed")
+        # the stream ends here: a last delta that was left as partial sums is not needed again
+        discard = getattr(stream.delta, "discard", None)
+        if discard is not None:
+            discard()
         rt.ops.gemm(h, self.head_weight, logits)
         return logits

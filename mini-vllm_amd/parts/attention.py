@@ -124,8 +124,7 @@ class Attention(Mixer):
                                           spec.head_dim, spec.scale, spec.window, plan, self.q_norm, self.k_norm,
                                           spec.qk_norm_eps, table, interleaved, not spec.shares_kv):
                 y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
-                ops.gemm(attn, self.w_o, y, self.b_o)
-                return y
+                return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True) or y
         ops.qk_norm_rope_store(
             qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, ctx.positions, ctx.token_seq,
             self.q_norm, self.k_norm, spec.qk_norm_eps, table, interleaved,
@@ -135,5 +134,5 @@ class Attention(Mixer):
                       kv.block_table, kv.page_size, ctx.positions, ctx.token_seq, spec.num_heads,
                       spec.num_kv_heads, spec.head_dim, spec.scale, spec.window, plan=ctx.attention_plan)
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
-        ops.gemm(attn, self.w_o, y, self.b_o)
-        return y
+        # (the sums of a product whose K was split may be left to the next norm)
+        return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True) or y

@@ -170,7 +170,9 @@ class Runtime:
 class HiddenStream:
     """The residual stream of a step: a float32 sum ``resid`` and the last part's output
     ``delta`` that has not been added yet. A norm consumes the pending delta (one fused
-    kernel adds it and normalises the sum)."""
+    kernel adds it and normalises the sum). ``delta`` is a tensor, or whatever ``ops.gemm(...,
+    defer_sum=True)`` returned in its place (an output whose partial sums the norm's kernel adds
+    up itself; it has ``shape``, ``materialize()`` and ``discard()``)."""
 
     __slots__ = ("resid", "delta", "spare")
 

@@ -51,5 +51,5 @@ class SwiGLU(FeedForward):
             ops.gemm(x, self.w_gate_up, gu)
             ops.swiglu(gu, act)
         y = rt.workspace.get("ffn.out", (n, spec.hidden_size), rt.dtype)
-        ops.gemm(act, self.w_down, y)
-        return y
+        # (the sums of a product whose K was split may be left to the next norm)
+        return ops.gemm(act, self.w_down, y, defer_sum=True) or y

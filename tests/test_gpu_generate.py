@@ -285,3 +285,47 @@ def test_generation_with_head_size_128(tmp_path):
     # eager steps split the keys differently and round differently: the same tokens but for near ties
     same = sum(a == b for a, b in zip(results["eager"], results["graphs of one"]))
     assert same >= len(prompts) - 1
+
+
+def test_generation_with_wide_layers_leaves_partial_sums_to_the_norms(tmp_path, monkeypatch):
+    """Two layers as wide as a large model's (output and down projections of 16 Mi elements): with
+    ten sequences decoding, these products split K over workgroups and leave their partial sums to
+    the norm that follows. The tokens are the plain model's, and the same as when every product
+    adds its sums up itself."""
+    from minivllm_amd import LLM, SamplingParams
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 2048,
+           "num_attention_heads": 64, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 8192,
+           "vocab_size": 1000, "max_position_embeddings": 4096, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+           "tie_word_embeddings": False, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
+    w = make_weights(cfg, seed=91, stored=torch.bfloat16, qk_gain=1.5)
+    path = write_model_dir(str(tmp_path / "wide"), cfg, w)
+    prompts = [random_tokens(cfg, n, seed=500 + n) for n in (3, 20, 7, 12, 5, 9, 16, 4, 11, 8)]
+    sp = SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True)
+    calls = {"split": 0}
+    from minivllm_amd.kernels.library import KernelLibrary
+    real_call = KernelLibrary.call
+
+    def counting_call(self, name, *args):
+        if name == "mv_add_rmsnorm_split":
+            calls["split"] += 1
+        return real_call(self, name, *args)
+
+    monkeypatch.setattr(KernelLibrary, "call", counting_call)
+    results = {}
+    for name in ("deferred", "added up"):
+        if name == "added up":
+            real_has = KernelLibrary.has
+            monkeypatch.setattr(KernelLibrary, "has", lambda self, n: n != "mv_add_rmsnorm_split" and real_has(self, n))
+        llm = LLM(model=path, dtype="bfloat16", kv_cache_block_size=16, kv_cache_num_blocks=64, max_model_len=64,
+                  max_num_batched_tokens=256, max_num_batched_seqs=16, use_cuda_graph=(name == "deferred"))
+        outs = llm.generate(prompts, sp, use_tqdm=False)
+        results[name] = [o.token_ids for o in outs]
+        if name == "deferred":
+            assert calls["split"] > 0, "no product left its sums to a norm"
+            check_against_plain(cfg, w, outs[:3], [sp] * 3, "bfloat16")
+            seen = calls["split"]
+        else:
+            assert calls["split"] == seen
+        del llm
+        torch.cuda.empty_cache()
+    assert results["deferred"] == results["added up"]

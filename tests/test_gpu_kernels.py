@@ -833,3 +833,45 @@ def test_norm_is_not_deferred_for_many_rows():
     stream = HiddenStream(torch.randn(17, 128, device="cuda"), torch.empty(17, 128, device="cuda"))
     assert isinstance(norm.pending(stream, None), torch.Tensor)
     assert not ops_for(torch.float32).can_fuse_norm(4, 128)
+
+
+@pytest.mark.parametrize("M,N,K,with_bias,with_rows", [(12, 4096, 4096, False, False), (33, 3080, 4096, True, False),
+                                                      (64, 2048, 8192, False, True), (2, 5120, 25600, False, False)])
+def test_partial_sums_of_a_product_go_straight_into_the_norm(M, N, K, with_bias, with_rows):
+    """A product whose K was split leaves its partial sums to the residual add + norm that follows
+    (``defer_sum``): the new residual and the normalised rows are bit for bit those of the path that
+    adds the sums up in a kernel of its own first; asking for the tensor instead gives the same
+    product; and the next product of the kind adds an unused one up before it takes the work area."""
+    from minivllm_amd.kernels.ops import SplitSum
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(29)
+    a = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
+    w = dev((torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16))
+    b = dev(torch.randn(N, generator=g).to(torch.bfloat16)) if with_bias else None
+    nw = dev((1 + 0.1 * torch.randn(N, generator=g)).to(torch.bfloat16))
+    resid0 = dev(torch.randn(M, N, generator=g))
+    rows = dev(torch.tensor([M - 1, 0], dtype=torch.int32)) if with_rows else None
+    n_out = 2 if with_rows else M
+
+    plain = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    assert ops.gemm(a, w, plain, b) is None
+    resid_a, out_a = resid0.clone(), torch.full((n_out, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.add_rmsnorm(resid_a, plain, nw, 1e-6, out_a, rows=rows)
+
+    target = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    split = ops.gemm(a, w, target, b, defer_sum=True)
+    assert isinstance(split, SplitSum), "the shape was left to another kernel"
+    resid_b, out_b = resid0.clone(), torch.full((n_out, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.add_rmsnorm(resid_b, split, nw, 1e-6, out_b, rows=rows)
+    assert torch.equal(out_a, out_b) and torch.equal(resid_a, resid_b)
+    assert split.done != with_rows          # with rows the delta stays pending in the stream
+    if with_rows:
+        assert torch.isnan(target.float()).all()
+        assert torch.equal(split.materialize(), plain)
+
+    # an unused one is added up when the next product needs the work area
+    first = ops.gemm(a, w, target, b, defer_sum=True)
+    other = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    second = ops.gemm(a, w, other, b, defer_sum=True)
+    assert first.done and torch.equal(target, plain)
+    assert torch.equal(second.materialize(), plain) and second.done and ops._split_pending is None
