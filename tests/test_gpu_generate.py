@@ -256,6 +256,29 @@ def test_graphs_of_many_sequences_use_rehearsed_library_products(models):
     assert all(verdicts.values()), f"a library product did not replay faithfully: {verdicts}"
 
 
+D128 = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 256,
+        "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 512,
+        "vocab_size": 1000, "max_position_embeddings": 4096, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+        "tie_word_embeddings": True, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
+
+
+@pytest.mark.parametrize("page_size", [64, 256])
+def test_generation_with_large_pages(tmp_path, page_size):
+    """Pages of 64 and of 256 slots (the reference's default block size) with the MFMA attention
+    kernels: prompts that end inside a page, cross a page's edge while decoding, and share the step."""
+    from minivllm_amd import LLM, SamplingParams
+    cfg = D128
+    w = make_weights(cfg, seed=78, stored=torch.bfloat16, qk_gain=1.5)
+    path = write_model_dir(str(tmp_path / "d128p"), cfg, w)
+    prompts = [random_tokens(cfg, n, seed=700 + n) for n in (250, 40, 7, 300, 129)]
+    sp = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    llm = LLM(model=path, dtype="bfloat16", kv_cache_block_size=page_size, kv_cache_num_blocks=4096 // page_size,
+              max_model_len=512, max_num_batched_tokens=192, max_num_batched_seqs=8)
+    outs = llm.generate(prompts, sp, use_tqdm=False)
+    check_against_plain(cfg, w, outs, [sp] * len(prompts), "bfloat16")
+    llm.manager.check_invariants()
+
+
 def test_generation_with_head_size_128(tmp_path):
     """A small model with the head size the MFMA kernels serve (128; hidden 256, two kv heads, K =
     256/512): decode steps take the fused attention and products, alone, in graphs and four in a
