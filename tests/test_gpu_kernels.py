@@ -875,3 +875,41 @@ def test_partial_sums_of_a_product_go_straight_into_the_norm(M, N, K, with_bias,
     second = ops.gemm(a, w, other, b, defer_sum=True)
     assert first.done and torch.equal(target, plain)
     assert torch.equal(second.materialize(), plain) and second.done and ops._split_pending is None
+
+
+def test_kernels_that_load_straight_into_lds_repeat_their_results():
+    """The K-splitting product and the prompt attention bring operands into LDS with loads whose
+    completion they wait for by count. A wait that came too early would show as results that differ
+    from call to call; here many calls in a row give the same bits."""
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(31)
+    for M, N, K in ((64, 4096, 4096), (9, 3100, 8192), (33, 12288, 2048)):
+        a = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
+        w = dev((torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16))
+        ops._mid_work = None
+        first = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        ops.gemm(a, w, first)
+        assert ops._mid_work is not None
+        for _ in range(30):
+            again = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+            ops.gemm(a, w, again)
+            assert torch.equal(first, again)
+    # prompt attention: one long portion over scrambled pages, both walks of the keys
+    H, Hkv, D, ps = 16, 8, 128, 16
+    for T in (700, 2048):
+        k_all = [torch.randn(T, Hkv, D, generator=g)]
+        v_all = [torch.randn(T, Hkv, D, generator=g)]
+        pages = -(-T // ps)
+        order = torch.randperm(pages + 3, generator=g)[:pages].tolist()
+        kp, vp = fill_pages(k_all, v_all, [order], ps, Hkv, D, pages + 3, torch.bfloat16)
+        bt = dev(torch.tensor([order], dtype=torch.int32))
+        q = dev(torch.randn(T, H * D, generator=g).to(torch.bfloat16))
+        pos = dev(torch.arange(T, dtype=torch.int32))
+        tseq = dev(torch.zeros(T, dtype=torch.int32))
+        plan = make_plan([T], [T])
+        first = torch.empty(T, H * D, dtype=torch.bfloat16, device="cuda")
+        ops.attention(q, first, kp, vp, bt, ps, pos, tseq, H, Hkv, D, D ** -0.5, None, plan=plan)
+        for _ in range(20):
+            again = torch.empty(T, H * D, dtype=torch.bfloat16, device="cuda")
+            ops.attention(q, again, kp, vp, bt, ps, pos, tseq, H, Hkv, D, D ** -0.5, None, plan=plan)
+            assert torch.equal(first, again)
