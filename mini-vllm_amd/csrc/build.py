@@ -29,7 +29,13 @@ ARCH = "gfx950"
 COMMON_SOURCES = ["runtime.hip", "elementwise.hip", "gemm_ref.hip", "attention_ref.hip", "sampling.hip"]
 VARIANT_SOURCES: Dict[str, List[str]] = {
     "f32": COMMON_SOURCES,
-    "bf16": COMMON_SOURCES + ["gemm_skinny.hip", "gemm_mid.hip", "attention_fast.hip", "attention_prefill.hip"],
+    "bf16": COMMON_SOURCES + ["gemm_skinny.hip", "gemm_mid.hip", "gemm_lt.hip", "attention_fast.hip",
+                              "attention_prefill.hip"],
+}
+# libraries a variant links against
+VARIANT_LIBS: Dict[str, List[str]] = {
+    "f32": [],
+    "bf16": ["-lhipblaslt"],
 }
 VARIANT_DEFINES: Dict[str, List[str]] = {
     "f32": ["-DMV_WITH_F32"],
@@ -60,7 +66,7 @@ def _sources(variant: str) -> List[str]:
 
 def source_hash(variant: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(BASE_FLAGS + VARIANT_DEFINES[variant]).encode())
+    h.update(" ".join(BASE_FLAGS + VARIANT_DEFINES[variant] + VARIANT_LIBS[variant]).encode())
     names = sorted(set(_sources(variant)) | {f for f in os.listdir(CSRC) if f.endswith(".h")})
     for name in names:
         h.update(name.encode())
@@ -161,7 +167,7 @@ def build(variant: str, force: bool = False, jobs: Optional[int] = None) -> str:
                 _log(f"  [{done}/{len(sources)}] {futs[fut]} ({dt:.1f} s)")
     lib = os.path.join(out_dir, library_name(variant))
     tmp = lib + f".tmp{os.getpid()}"
-    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp] + objs
+    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp] + objs + VARIANT_LIBS[variant]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"linking {lib} failed:\n{' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")

@@ -53,6 +53,10 @@ _OPTIONAL_SIGNATURES = {
     "mv_gemm_skinny_swiglu": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_skinny_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
                                     c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "mv_gemm_lt_workspace": (c_long, []),
+    # A, lda, W, bias, C, ldc, M, N, K, workspace, workspace_bytes, stream
+    "mv_gemm_lt": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_long,
+                           c_void_p]),
     "mv_gemm_mid_workspace": (c_long, [c_int, c_int, c_int]),
     "mv_gemm_mid_splits": (c_int, [c_int, c_int]),
     # A, lda, W, M, N, K, work, work_floats, stream

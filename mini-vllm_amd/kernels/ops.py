@@ -113,6 +113,7 @@ class Ops:
         self.stream_handle: Optional[int] = None
         self._transposed = {}
         self._mid_work: Optional[torch.Tensor] = None
+        self._lt_work: Optional[torch.Tensor] = None        # the library's workspace
         self._split_pending: Optional[SplitSum] = None     # partial sums in the work area nobody has used yet
         self._mid_retired: list = []
         self._sample_work: Optional[torch.Tensor] = None
@@ -349,16 +350,35 @@ class Ops:
                                   self._stream())
                 return
         if fast and out.dtype == self.dtype and M > SKINNY_MAX_M and self._library_allowed(M, N, K, bias is not None):
-            wt = self._transposed.get(w.data_ptr())
-            if wt is None or wt.shape != (K, N):
-                wt = self._transposed[w.data_ptr()] = w.t()      # the view is made once per weight
-            if bias is None:
-                torch.mm(a, wt, out=out)
-            else:
-                torch.addmm(bias, a, wt, out=out)
+            self._library_product(a, w, bias, out)
             return
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
+
+    def _library_product(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> None:
+        """out = a @ w^T (+ bias) by the library (hipBLASLt), bf16 in and out. It is called directly
+        where the kernel library was built with it (a call costs a third of the host time of the
+        tensor library's dispatcher, which matters for prompt steps of small models); else through
+        ``torch.mm``."""
+        M, K = a.shape
+        N = w.shape[0]
+        if self.lib.has("mv_gemm_lt") and a.stride(1) == 1 and out.stride(1) == 1 and a.data_ptr() % 16 == 0 \
+                and out.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
+            if self._lt_work is None:
+                if torch.cuda.is_current_stream_capturing():
+                    raise KernelLibraryError("the library's workspace must be made before a capture")
+                self._lt_work = torch.empty(int(self.lib.dll.mv_gemm_lt_workspace()), dtype=torch.uint8, device=a.device)
+            self.lib.call("mv_gemm_lt", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias),
+                          out.data_ptr(), out.stride(0) if M > 1 else N, M, N, K, self._lt_work.data_ptr(),
+                          self._lt_work.numel(), self._stream())
+            return
+        wt = self._transposed.get(w.data_ptr())
+        if wt is None or wt.shape != (K, N):
+            wt = self._transposed[w.data_ptr()] = w.t()      # the view is made once per weight
+        if bias is None:
+            torch.mm(a, wt, out=out)
+        else:
+            torch.addmm(bias, a, wt, out=out)
 
     def _library_allowed(self, M: int, N: int, K: int, with_bias: bool) -> bool:
         """Whether the library's matrix product may serve this shape now. Outside graphs: whenever it
@@ -382,16 +402,15 @@ class Ops:
     def _rehearse_library_product(self, M: int, N: int, K: int, with_bias: bool) -> bool:
         dev = torch.device("cuda", torch.cuda.current_device())
         a = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
-        wt = (torch.randn(N, K, device=dev, dtype=torch.bfloat16) * 0.05).t()
+        w = torch.randn(N, K, device=dev, dtype=torch.bfloat16) * 0.05
         bias = torch.randn(N, device=dev, dtype=torch.bfloat16) if with_bias else None
         out = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
 
         def product(dst):
-            if bias is None:
-                torch.mm(a, wt, out=dst)
-            else:
-                torch.addmm(bias, a, wt, out=dst)
+            self._library_product(a, w, bias, dst)
 
+        bound = self.stream_handle
+        self.stream_handle = None                          # the rehearsal runs on torch's current stream
         try:
             product(out)                                   # loads the kernel, makes the library's handles
             torch.cuda.synchronize()
@@ -412,6 +431,8 @@ class Ops:
             return ok
         except RuntimeError:
             return False
+        finally:
+            self.stream_handle = bound
 
     def _gemm_mid(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   ldc: int, M: int, N: int, K: int, swiglu: bool, defer_sum: bool = False):
