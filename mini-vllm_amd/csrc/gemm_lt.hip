@@ -53,6 +53,14 @@ const char* lt_status(hipblasStatus_t s) {
         if (st_ != HIPBLAS_STATUS_SUCCESS) return mv_fail("gemm_lt: %s: %s", #call, lt_status(st_)); \
     } while (0)
 
+void drop_plan(LtPlan& p) {
+    if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    if (p.w) hipblasLtMatrixLayoutDestroy(p.w);
+    if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+    if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+    p = LtPlan{};
+}
+
 int make_plan(LtPlan& p, int M, int N, int K, long lda, long ldc, bool with_bias, size_t workspace_bytes) {
     LT_CHECK(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
     const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
@@ -71,22 +79,30 @@ int make_plan(LtPlan& p, int M, int N, int K, long lda, long ldc, bool with_bias
     LT_CHECK(hipblasLtMatmulPreferenceCreate(&pref));
     LT_CHECK(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
                                                    sizeof(workspace_bytes)));
-    hipblasLtMatmulHeuristicResult_t found[1];
+    // The heuristic's list is in its order of preference; it may hold algorithms that want more
+    // workspace than the preference names, so the first that fits is taken.
+    constexpr int kAsk = 8;
+    hipblasLtMatmulHeuristicResult_t found[kAsk];
     int n_found = 0;
-    const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.w, p.a, p.c, p.c, pref, 1, found,
+    const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.w, p.a, p.c, p.c, pref, kAsk, found,
                                                                &n_found);
     hipblasLtMatmulPreferenceDestroy(pref);
     if (st != HIPBLAS_STATUS_SUCCESS || n_found < 1)
         return mv_fail("gemm_lt: the library has no algorithm for M=%d N=%d K=%d (%s)", M, N, K, lt_status(st));
-    p.algo = found[0].algo;
-    p.workspace = found[0].workspaceSize;
-    return 0;
+    for (int i = 0; i < n_found; ++i) {
+        if (found[i].workspaceSize > workspace_bytes) continue;
+        p.algo = found[i].algo;
+        p.workspace = found[i].workspaceSize;
+        return 0;
+    }
+    return mv_fail("gemm_lt: every algorithm the library offers for M=%d N=%d K=%d wants more than the %zu bytes of "
+                   "workspace brought (the first %zu)", M, N, K, workspace_bytes, found[0].workspaceSize);
 }
 
 }  // namespace
 
 // Bytes of workspace the caller should bring (plans are made for at most this much).
-extern "C" long mv_gemm_lt_workspace() { return 32L << 20; }
+extern "C" long mv_gemm_lt_workspace() { return 128L << 20; }
 
 extern "C" int mv_gemm_lt(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N,
                           int K, void* workspace, long workspace_bytes, hipStream_t stream) {
@@ -101,7 +117,10 @@ extern "C" int mv_gemm_lt(const void* A, long lda, const void* W, const void* bi
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
         LtPlan p;
-        if (int rc = make_plan(p, M, N, K, lda, ldc, bias != nullptr, (size_t)workspace_bytes)) return rc;
+        if (int rc = make_plan(p, M, N, K, lda, ldc, bias != nullptr, (size_t)workspace_bytes)) {
+            drop_plan(p);
+            return rc;
+        }
         it = g_plans.emplace(key, p).first;
     }
     LtPlan& p = it->second;
