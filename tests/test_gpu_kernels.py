@@ -706,6 +706,92 @@ def test_gemm_swiglu_fused(M, I, K):
     assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_pages_beyond_two_to_the_31_elements(dtype):
+    """A pool whose key and value tensors each hold more than 2^31 elements (what a small model gets
+    when the device's memory is left to the cache): requests whose pages lie at the far end, among
+    them the very last page, are written and read like any other. Three steps through every
+    cache-writing and attention kernel: a prompt alone; a whole prompt beside a decoded token; both
+    requests decoding (in bfloat16 also from the raw rows, by the kernel that writes the cache itself)."""
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(71)
+    H, Hkv, D, ps = 16, 8, 128, 16
+    page_elems = Hkv * ps * D
+    num_pages = (1 << 31) // page_elems + 1500
+    assert num_pages * page_elems > (1 << 31) + 1000 * page_elems
+    kp = torch.empty(num_pages, Hkv, ps, D, dtype=dtype, device="cuda")
+    vp = torch.empty(num_pages, Hkv, D, ps, dtype=dtype, device="cuda")
+    ctx = [203, 302]                                        # lengths at the end
+    pages_per = [-(-c // ps) for c in ctx]
+    # pages from the top of the pool, the last one included, in scrambled order, and one low page each
+    top = (num_pages - 2 - torch.randperm(1400, generator=g)[:sum(pages_per)]).tolist()
+    top[3] = num_pages - 1
+    tables = [top[:pages_per[0]], top[pages_per[0]:]]
+    tables[0][5], tables[1][7] = 4, 11
+    assert len(set(tables[0] + tables[1])) == sum(pages_per)
+    for t in tables:                                        # what the kernels must not rely on
+        idx = torch.tensor(t, device="cuda")
+        kp[idx] = float("nan"); vp[idx] = float("nan")
+    bt = torch.full((2, max(pages_per)), -1, dtype=torch.int32)
+    for s_, t in enumerate(tables):
+        bt[s_, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    bt = dev(bt)
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype) for c in ctx]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype) for c in ctx]
+    scale = 1.0 / math.sqrt(D)
+    tol = 2 * max(OP_TOL[dtype], 5e-6)
+
+    def run_step(spans, fused=False):
+        """spans: (sequence, first position, tokens). Writes the tokens' keys and values, runs
+        attention for them and compares with the reference over the sequences' whole prefixes."""
+        positions, token_seq, rows_k, rows_v = [], [], [], []
+        for s_, start, cnt in spans:
+            positions += list(range(start, start + cnt)); token_seq += [s_] * cnt
+            rows_k.append(k_all[s_][start:start + cnt]); rows_v.append(v_all[s_][start:start + cnt])
+        n = len(positions)
+        q = torch.randn(n, H, D, generator=g)
+        for i in range(n):          # a key of the sequence's first page stands out for its last query
+            if i + 1 == n or token_seq[i + 1] != token_seq[i]:
+                q[i] = 6.0 * k_all[token_seq[i]][2].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
+        q = q.to(dtype)
+        qkv = dev(torch.cat([q.view(n, -1), torch.cat(rows_k).view(n, -1), torch.cat(rows_v).view(n, -1)], dim=1))
+        pos_t = torch.tensor(positions, dtype=torch.int32); seq_t = torch.tensor(token_seq, dtype=torch.int32)
+        out = torch.full((n, H * D), float("nan"), dtype=dtype, device="cuda")
+        q_lens = [cnt for _, _, cnt in spans]
+        plan = make_plan(q_lens, [start + cnt for _, start, cnt in spans])
+        plan_seq = dev(torch.tensor(sum(([i] * c for i, c in enumerate(q_lens)), []), dtype=torch.int32))
+        step_bt = bt[[s_ for s_, _, _ in spans]].contiguous()
+        if fused:
+            assert ops.attention_decode_fused(qkv, out, kp, vp, step_bt, ps, dev(pos_t), plan_seq, H, Hkv, D, scale,
+                                              None, plan, None, None, 1e-6, None, False, True)
+        else:
+            ops.qk_norm_rope_store(qkv, H, Hkv, D, dev(pos_t), plan_seq, None, None, 1e-6, None, False, kp, vp,
+                                   step_bt, ps)
+            ops.attention(qkv[:, :H * D], out, kp, vp, step_bt, ps, dev(pos_t), plan_seq, H, Hkv, D, scale, None,
+                          plan=plan)
+        torch.cuda.synchronize()
+        want = reference_attention(q.double(), [k.double() for k in k_all], [v.double() for v in v_all], pos_t, seq_t,
+                                   H, Hkv, scale, None)
+        got = out.float().cpu().view(n, H, D)
+        assert not torch.isnan(got).any()
+        assert rel_err(got.numpy(), want.numpy()) <= tol
+
+    run_step([(1, 0, 300)])                                 # a prompt alone (values go tile by tile)
+    run_step([(0, 0, 201), (1, 300, 1)])                    # a whole prompt beside a decoded token
+    run_step([(0, 201, 1), (1, 301, 1)])                    # both decode
+    if dtype == torch.bfloat16:
+        run_step([(0, 202, 1)], fused=True)                 # from the raw rows, one request
+    # the pages hold exactly what was written, the last page of the pool included
+    for s_, c in enumerate(ctx):
+        upto = c if (dtype == torch.bfloat16 or s_ == 1) else c - 1
+        for pos in (0, 1, 50, 3 * ps + 1, upto - 1):
+            page, slot = tables[s_][pos // ps], pos % ps
+            assert torch.equal(kp[page, :, slot, :].cpu(), k_all[s_][pos]), (s_, pos)
+            assert torch.equal(vp[page, :, :, slot].cpu(), v_all[s_][pos]), (s_, pos)
+    del kp, vp
+    torch.cuda.empty_cache()
+
+
 def test_attention_reduces_to_library_softmax():
     """One head, no window, whole sequence: equals torch's scaled_dot_product_attention."""
     ops = ops_for(torch.float32)
