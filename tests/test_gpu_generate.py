@@ -136,6 +136,25 @@ def test_prefix_reuse_gives_the_same_tokens(models):
     assert llm.metrics.prefill_tokens < plain_llm.metrics.prefill_tokens      # the shared page was not run again
 
 
+def test_pool_sized_from_the_memory_left(models):
+    """Without a page count the pool is what the memory share leaves after a dry step of a full
+    token budget, never more than every request at full length can use; a share below what is
+    already in use is refused with the numbers."""
+    from minivllm_amd import LLM, SamplingParams
+    cfg, w, path = models["B"]
+    llm = LLM(model=path, dtype="bfloat16", kv_cache_block_size=8, max_model_len=96, max_num_batched_tokens=256,
+              max_num_batched_seqs=6, gpu_memory_utilization=0.3)
+    assert llm.executor.num_pages == 6 * 12 and llm.manager.pools[0].num_pages == 72
+    assert all(k.shape[0] == 72 and v.shape[0] == 72 for k, v in llm.executor.kv_pages.values())
+    prompts = [random_tokens(cfg, n, seed=70 + n) for n in (30, 3, 11)]
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    outs = llm.generate(prompts, sp, use_tqdm=False)
+    check_against_plain(cfg, w, outs, [sp] * 3, "bfloat16")
+    with pytest.raises(RuntimeError, match="no memory left for the cache"):
+        LLM(model=path, dtype="bfloat16", max_model_len=96, max_num_batched_tokens=64, max_num_batched_seqs=4,
+            gpu_memory_utilization=1e-6)
+
+
 def test_eos_and_max_model_len(models):
     from minivllm_amd import LLM, SamplingParams
     cfg, w, path = models["A"]
