@@ -345,15 +345,14 @@ def test_attention_general(dtype, with_plan, H, Hkv, D, ps, window):
 
 
 @pytest.mark.parametrize("H,Hkv,D,ps,window", [(4, 2, 128, 16, None), (8, 2, 64, 32, 300), (8, 1, 128, 16, None)])
-def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window):
-    """Prompt portions over more than a thousand keys (the MFMA kernel then walks the keys with two
-    wave groups per workgroup and merges them): a whole long prompt, a late portion of another, and
-    a single token, with a far key (or the one at the window's edge) made to stand out."""
+@pytest.mark.parametrize("ctx_lens,q_lens", [([1203, 1170, 1050], [1203, 70, 1]), ([5003, 6100, 2050], [5003, 650, 1])])
+def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window, ctx_lens, q_lens):
+    """Prompt portions over thousands of keys (the MFMA kernel then walks the keys with two wave
+    groups per workgroup and merges them): a whole long prompt, a late portion of another, and a
+    single token, with a far key (or the one at the window's edge) made to stand out."""
     ops = ops_for(torch.bfloat16)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(61)
-    ctx_lens = [1203, 1170, 1050]
-    q_lens = [1203, 70, 1]
     k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
     v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
     pages_per = [-(-c // ps) for c in ctx_lens]
@@ -377,7 +376,7 @@ def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window):
     positions = torch.tensor(positions, dtype=torch.int32)
     token_seq = torch.tensor(token_seq, dtype=torch.int32)
     q = torch.randn(n, H, D, generator=g)
-    for row, s in ((1202, 0), (1203 + 69, 1), (n - 1, 2)):      # the last query of every sequence
+    for row, s in ((q_lens[0] - 1, 0), (q_lens[0] + q_lens[1] - 1, 1), (n - 1, 2)):      # the last query of every sequence
         far = 3 if window is None else ctx_lens[s] - 1 - window
         q[row] = 6.0 * k_all[s][far].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
     q = q.to(dtype)
@@ -387,8 +386,11 @@ def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window):
     assert plan.max_context_len >= 1024
     ops.attention(dev(q.view(n, H * D)), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale,
                   window, plan=plan)
-    # the reference for a sample of the rows (every row of the short sequences, a spread of the long one)
-    rows = sorted(set(list(range(0, 1203, 37)) + list(range(1180, n))))
+    # the reference for a sample of the rows: a spread of each sequence, every row around the seam between
+    # the first two, and the last ones
+    first = q_lens[0]
+    rows = sorted(set(list(range(0, first, max(37, first // 40))) + list(range(first - 23, first + 40)) +
+                      list(range(first + 40, n, 31)) + list(range(n - 5, n))))
     want = reference_attention(q[rows].double(), k_all, v_all, positions[rows], token_seq[rows], H, Hkv, scale, window)
     got = out.float().cpu().view(n, H, D)
     assert not torch.isnan(got).any()
