@@ -133,6 +133,38 @@ def test_long_decoding(cases):
         assert worst <= tol[dtype]
 
 
+@pytest.mark.parametrize("head_dim,page_size", [(128, 16), (64, 32), (48, 16)])
+def test_contexts_beyond_a_thousand_tokens(tmp_path, head_dim, page_size):
+    """Requests of 1100 to 2300 tokens: prompts in portions of up to 400 tokens, then a hundred and
+    more decoded one by one across the lengths at which the decode graphs and the prompt kernel
+    change their launch (1024, 2048), three live at a time beside each other. Sharp attention: a
+    far key that is lost shows."""
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 96,
+           "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": head_dim, "intermediate_size": 160,
+           "vocab_size": 211, "max_position_embeddings": 4096, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+           "tie_word_embeddings": False, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
+    weights = make_weights(cfg, seed=head_dim, stored=torch.bfloat16, qk_gain=2.5)
+    path = write_model_dir(str(tmp_path / "long"), cfg, weights)
+    lengths = {"a": 1100, "b": 2300, "c": 1290, "d": 2100}
+    reqs = {rid: random_tokens(cfg, n, seed=n) for rid, n in lengths.items()}
+    want = {rid: plain_logits(cfg, weights, toks) for rid, toks in reqs.items()}
+    emulated = {rid: plain_logits_bf16(cfg, weights, toks) for rid, toks in reqs.items()}
+    bf16_err = max(rel_err(emulated[r][p], want[r][p]) for r, t in reqs.items() for p in range(len(t)))
+    prompt_lens = {"a": 960, "b": 2000, "c": 1280, "d": 1900}
+    steps = trace_tools.mixed(reqs, prompt_lens, max_live=3, seed=head_dim, max_portion=400)
+    from minivllm_amd.engine.trace import TraceRunner
+    for dtype in ("float32", "bfloat16"):
+        runner = TraceRunner(path, dtype, trace_tools.max_live_tokens(steps), page_size=page_size)
+        got = trace_tools.collect(steps, runner.run_step)
+        assert len(got) == sum(lengths.values())
+        worst = max(rel_err(row, want[rid][pos]) for (rid, pos), row in got.items())
+        tol = TOL_F32 if dtype == "float32" else bf16_tolerance(bf16_err)
+        print(f"long contexts, head size {head_dim} [{dtype}]: worst relative error {worst:.3e} (allowed {tol:.3e})")
+        assert worst <= tol
+        runner.manager.check_invariants()
+        assert all(pool.num_free == pool.num_pages for pool in runner.manager.pools)
+
+
 def test_trace_run_program(cases, tmp_path):
     """bin/trace_run as a user calls it: steps on standard input, logits in files."""
     case = cases["A"]
