@@ -140,13 +140,14 @@ def measure_prefill(llm, vocab, tokens, repeats, seed):
     return min(times[1:]) if repeats else times[0]
 
 
-def measure_serve(llm, vocab, requests, gen_len, seed):
+def measure_serve(llm, vocab, requests, gen_len, seed, prompt_min=128, prompt_max=2048):
     """All requests submitted at once; returns (seconds, generated tokens, prompt tokens, steps, preemptions)."""
     import numpy as np
     import torch
     from minivllm_amd import SamplingParams
     rng = np.random.default_rng(seed)
-    prompts = [[int(t) for t in rng.integers(0, vocab, size=int(n))] for n in rng.integers(128, 2049, size=requests)]
+    prompts = [[int(t) for t in rng.integers(0, vocab, size=int(n))]
+               for n in rng.integers(prompt_min, prompt_max + 1, size=requests)]
     # a few requests through every kind of step first (graphs are captured on first use)
     llm.generate(prompts[:4], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
     torch.cuda.synchronize()
@@ -188,6 +189,9 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=256, help="requests of the serve workload")
     ap.add_argument("--gen-len", type=int, default=256, help="generated tokens per request of the serve workload")
     ap.add_argument("--token-budget", type=int, default=8192, help="tokens per step of the serve workload")
+    ap.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the serve workload")
+    ap.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the serve workload")
+    ap.add_argument("--max-seqs", type=int, default=256, help="most requests in one step of the serve workload")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -201,21 +205,24 @@ def main() -> int:
     layers_full = shape["num_hidden_layers"]
     layers = args.layers or layers_full
     if args.only == "serve":
-        if 2048 + args.gen_len > args.context:
-            print(f"bench.py: prompts of up to 2048 tokens + {args.gen_len} generated exceed the context {args.context}")
+        if not 1 <= args.prompt_min <= args.prompt_max or args.prompt_max + args.gen_len > args.context:
+            print(f"bench.py: prompts of {args.prompt_min}..{args.prompt_max} tokens + {args.gen_len} generated "
+                  f"do not fit the context {args.context}")
             return 2
-        pages = args.requests * (-(-(2048 + args.gen_len) // args.block_size) + 1) + 64
-        llm, cfg = build_llm(args, shape, layers, max_seqs=min(256, args.requests), token_budget=args.token_budget,
-                             num_pages=pages)
-        dt, gen, prompt, steps, preempted = measure_serve(llm, cfg.vocab_size, args.requests, args.gen_len, args.seed)
+        live = min(args.max_seqs, args.requests)
+        pages = live * (-(-(args.prompt_max + args.gen_len) // args.block_size) + 1) + 64
+        llm, cfg = build_llm(args, shape, layers, max_seqs=live, token_budget=args.token_budget, num_pages=pages)
+        dt, gen, prompt, steps, preempted = measure_serve(llm, cfg.vocab_size, args.requests, args.gen_len, args.seed,
+                                                          args.prompt_min, args.prompt_max)
         print(json.dumps({
-            "metric": "generated tok/s, continuous batching (%d requests, prompts 128..2048, %d generated each)"
-                      % (args.requests, args.gen_len),
+            "metric": "generated tok/s, continuous batching (%d requests, prompts %d..%d, %d generated each)"
+                      % (args.requests, args.prompt_min, args.prompt_max, args.gen_len),
             "value": round(gen / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 0,
             "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
             "config": {"model": f"qwen3-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
                        "requests": args.requests, "gen_len": args.gen_len, "token_budget": args.token_budget,
+                       "max_seqs": live, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max,
                        "seq_len": args.context, "block_size": args.block_size, "graph": not args.no_graph,
                        "scheduler_steps": args.scheduler_steps, "parallelism": "single-gpu"},
             "seconds": round(dt, 3), "prompt_tokens": prompt, "generated_tokens": gen,

@@ -1,6 +1,7 @@
 // The library's matrix product for many rows (prompt portions, decode steps of more than 64
 // sequences), called directly:
-//     C[M, N] = A[M, K] * W[N, K]^T (+ bias),   bf16 in and out, float accumulation (hipBLASLt).
+//     C[M, N] = A[M, K] * W[N, K]^T (+ bias),   bf16 in, bf16 or float out, float accumulation
+//     (hipBLASLt).
 // Going through a tensor library's dispatcher costs about 18 us of host time per product on this
 // machine, a direct call about 5: a prompt step of a small model has four products per layer that
 // take 15 to 30 us each on the device, so the host would be the slower side.
@@ -11,8 +12,10 @@
 // transa = T, transb = N. The bias then runs along the rows of D, which is what its bias epilogue
 // adds.
 //
-// One plan (descriptor, layouts, the heuristic's first algorithm) is kept per shape. The caller
-// brings the workspace; nothing is allocated here after a shape's first call.
+// One plan (descriptor, layouts, the first algorithm of the heuristic's list that fits the
+// workspace) is kept per shape. The caller brings the workspace; nothing is allocated here after a
+// shape's first call. A shape the library has no algorithm for is declined with return code 2
+// (nothing done), every time it comes.
 #include "common.h"
 
 #include <hipblaslt/hipblaslt.h>
@@ -28,11 +31,12 @@ struct LtPlan {
     hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
+    bool served = false;            // the library has an algorithm for the shape that fits the workspace
 };
 
 std::mutex g_lock;
 hipblasLtHandle_t g_handle = nullptr;
-std::map<std::tuple<int, int, int, long, long, int>, LtPlan> g_plans;
+std::map<std::tuple<int, int, int, long, long, int, int>, LtPlan> g_plans;
 
 const char* lt_status(hipblasStatus_t s) {
     switch (s) {
@@ -61,7 +65,8 @@ void drop_plan(LtPlan& p) {
     p = LtPlan{};
 }
 
-int make_plan(LtPlan& p, int M, int N, int K, long lda, long ldc, bool with_bias, size_t workspace_bytes) {
+int make_plan(LtPlan& p, int M, int N, int K, long lda, long ldc, bool with_bias, bool float_out,
+              size_t workspace_bytes) {
     LT_CHECK(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
     const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
     LT_CHECK(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)));
@@ -74,7 +79,7 @@ int make_plan(LtPlan& p, int M, int N, int K, long lda, long ldc, bool with_bias
     }
     LT_CHECK(hipblasLtMatrixLayoutCreate(&p.w, HIP_R_16BF, K, N, K));
     LT_CHECK(hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, K, M, lda));
-    LT_CHECK(hipblasLtMatrixLayoutCreate(&p.c, HIP_R_16BF, N, M, ldc));
+    LT_CHECK(hipblasLtMatrixLayoutCreate(&p.c, float_out ? HIP_R_32F : HIP_R_16BF, N, M, ldc));
     hipblasLtMatmulPreference_t pref = nullptr;
     LT_CHECK(hipblasLtMatmulPreferenceCreate(&pref));
     LT_CHECK(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
@@ -87,16 +92,15 @@ int make_plan(LtPlan& p, int M, int N, int K, long lda, long ldc, bool with_bias
     const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.w, p.a, p.c, p.c, pref, kAsk, found,
                                                                &n_found);
     hipblasLtMatmulPreferenceDestroy(pref);
-    if (st != HIPBLAS_STATUS_SUCCESS || n_found < 1)
-        return mv_fail("gemm_lt: the library has no algorithm for M=%d N=%d K=%d (%s)", M, N, K, lt_status(st));
+    if (st != HIPBLAS_STATUS_SUCCESS || n_found < 1) return 0;      // no algorithm: the plan stays without one
     for (int i = 0; i < n_found; ++i) {
         if (found[i].workspaceSize > workspace_bytes) continue;
         p.algo = found[i].algo;
         p.workspace = found[i].workspaceSize;
+        p.served = true;
         return 0;
     }
-    return mv_fail("gemm_lt: every algorithm the library offers for M=%d N=%d K=%d wants more than the %zu bytes of "
-                   "workspace brought (the first %zu)", M, N, K, workspace_bytes, found[0].workspaceSize);
+    return 0;                                                        // none fits the workspace brought
 }
 
 }  // namespace
@@ -104,8 +108,11 @@ int make_plan(LtPlan& p, int M, int N, int K, long lda, long ldc, bool with_bias
 // Bytes of workspace the caller should bring (plans are made for at most this much).
 extern "C" long mv_gemm_lt_workspace() { return 128L << 20; }
 
-extern "C" int mv_gemm_lt(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N,
-                          int K, void* workspace, long workspace_bytes, hipStream_t stream) {
+extern "C" int mv_gemm_lt(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int c_dtype, int M,
+                          int N, int K, void* workspace, long workspace_bytes, hipStream_t stream) {
+    MV_REQUIRE(c_dtype == MV_BF16 || c_dtype == MV_F32, "gemm_lt: output type %d is neither bf16 nor float",
+               c_dtype);
+    const bool float_out = c_dtype == MV_F32;
     MV_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_lt: bad sizes M=%d N=%d K=%d", M, N, K);
     MV_REQUIRE(lda >= K && ldc >= N, "gemm_lt: lda=%ld / ldc=%ld too small for K=%d / N=%d", lda, ldc, K, N);
     MV_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)C % 16) == 0,
@@ -113,17 +120,22 @@ extern "C" int mv_gemm_lt(const void* A, long lda, const void* W, const void* bi
     MV_REQUIRE(workspace_bytes >= 0 && (workspace != nullptr || workspace_bytes == 0), "gemm_lt: bad workspace");
     std::lock_guard<std::mutex> guard(g_lock);
     if (g_handle == nullptr) LT_CHECK(hipblasLtCreate(&g_handle));
-    const auto key = std::make_tuple(M, N, K, lda, ldc, bias != nullptr ? 1 : 0);
+    const auto key = std::make_tuple(M, N, K, lda, ldc, bias != nullptr ? 1 : 0, float_out ? 1 : 0);
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
         LtPlan p;
-        if (int rc = make_plan(p, M, N, K, lda, ldc, bias != nullptr, (size_t)workspace_bytes)) {
+        if (int rc = make_plan(p, M, N, K, lda, ldc, bias != nullptr, float_out, (size_t)workspace_bytes)) {
             drop_plan(p);
             return rc;
         }
         it = g_plans.emplace(key, p).first;
     }
     LtPlan& p = it->second;
+    if (!p.served) {
+        mv_fail("gemm_lt: the library has no algorithm for M=%d N=%d K=%d (lda %ld, ldc %ld) within %ld bytes of workspace",
+                M, N, K, lda, ldc, workspace_bytes);
+        return 2;
+    }
     MV_REQUIRE((long)p.workspace <= workspace_bytes, "gemm_lt: the plan needs %zu bytes of workspace, %ld were brought",
                p.workspace, workspace_bytes);
     if (bias != nullptr)

@@ -54,9 +54,9 @@ _OPTIONAL_SIGNATURES = {
     "mv_gemm_skinny_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
                                     c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_lt_workspace": (c_long, []),
-    # A, lda, W, bias, C, ldc, M, N, K, workspace, workspace_bytes, stream
-    "mv_gemm_lt": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_long,
-                           c_void_p]),
+    # A, lda, W, bias, C, ldc, c_dtype, M, N, K, workspace, workspace_bytes, stream
+    "mv_gemm_lt": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p,
+                           c_long, c_void_p]),
     "mv_gemm_mid_workspace": (c_long, [c_int, c_int, c_int]),
     "mv_gemm_mid_splits": (c_int, [c_int, c_int]),
     # A, lda, W, M, N, K, work, work_floats, stream
@@ -123,6 +123,17 @@ class KernelLibrary:
         if rc != 0:
             msg = self.dll.mv_last_error()
             raise KernelLibraryError(msg.decode("utf-8", "replace") if msg else f"{name} failed")
+
+    def offer(self, name: str, *args) -> bool:
+        """Calls an entry point that may decline its arguments (return code 2, nothing done):
+        False then, True when it ran; any other failure raises."""
+        rc = getattr(self.dll, name)(*args)
+        if rc == 0:
+            return True
+        if rc == 2:
+            return False
+        msg = self.dll.mv_last_error()
+        raise KernelLibraryError(msg.decode("utf-8", "replace") if msg else f"{name} failed")
 
 
 _LOCK = threading.Lock()

@@ -341,25 +341,34 @@ class Ops:
                                   defer_sum=defer_sum and out.dtype == self.dtype and out.is_contiguous())
             if done:
                 return done if isinstance(done, SplitSum) else None
-            if M <= SKINNY_MAX_M or out.dtype == torch.float32 or not self._library_allowed(M, N, K, bias is not None):
-                # more rows than one workgroup takes are dealt out to groups of workgroups by the kernel
-                for m0 in range(0, M, SKINNY_LAUNCH_ROWS):
-                    m = min(SKINNY_LAUNCH_ROWS, M - m0)
-                    self.lib.call("mv_gemm_skinny", a.data_ptr() + m0 * lda * 2, lda, w.data_ptr(), K, _ptr(bias),
-                                  out.data_ptr() + m0 * ldc * out.element_size(), ldc, _CODES[out.dtype], m, N, K,
-                                  self._stream())
+            if M > SKINNY_MAX_M and self._library_serves(out) and \
+                    self._library_allowed(M, N, K, bias is not None, out.dtype) and self._library_product(a, w, bias, out):
                 return
-        if fast and out.dtype == self.dtype and M > SKINNY_MAX_M and self._library_allowed(M, N, K, bias is not None):
-            self._library_product(a, w, bias, out)
+            # more rows than one workgroup takes are dealt out to groups of workgroups by the kernel
+            for m0 in range(0, M, SKINNY_LAUNCH_ROWS):
+                m = min(SKINNY_LAUNCH_ROWS, M - m0)
+                self.lib.call("mv_gemm_skinny", a.data_ptr() + m0 * lda * 2, lda, w.data_ptr(), K, _ptr(bias),
+                              out.data_ptr() + m0 * ldc * out.element_size(), ldc, _CODES[out.dtype], m, N, K,
+                              self._stream())
+            return
+        if fast and M > SKINNY_MAX_M and self._library_serves(out) and \
+                self._library_allowed(M, N, K, bias is not None, out.dtype) and self._library_product(a, w, bias, out):
             return
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
 
-    def _library_product(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> None:
-        """out = a @ w^T (+ bias) by the library (hipBLASLt), bf16 in and out. It is called directly
-        where the kernel library was built with it (a call costs a third of the host time of the
-        tensor library's dispatcher, which matters for prompt steps of small models); else through
-        ``torch.mm``."""
+    def _library_serves(self, out: torch.Tensor) -> bool:
+        """The library's product writes the activation type; called directly it also writes float32
+        (the logits of a step of more than 64 rows)."""
+        return out.dtype == self.dtype or (out.dtype == torch.float32 and self.lib.has("mv_gemm_lt")
+                                           and out.data_ptr() % 16 == 0)
+
+    def _library_product(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> bool:
+        """out = a @ w^T (+ bias) by the library (hipBLASLt), bf16 in, bf16 or float32 out. It is
+        called directly where the kernel library was built with it (a call costs a third of the host
+        time of the tensor library's dispatcher, which matters for prompt steps of small models);
+        else, for bf16 output, through ``torch.mm``. False, with nothing done, when the library has
+        no algorithm for the shape."""
         M, K = a.shape
         N = w.shape[0]
         if self.lib.has("mv_gemm_lt") and a.stride(1) == 1 and out.stride(1) == 1 and a.data_ptr() % 16 == 0 \
@@ -368,10 +377,11 @@ class Ops:
                 if torch.cuda.is_current_stream_capturing():
                     raise KernelLibraryError("the library's workspace must be made before a capture")
                 self._lt_work = torch.empty(int(self.lib.dll.mv_gemm_lt_workspace()), dtype=torch.uint8, device=a.device)
-            self.lib.call("mv_gemm_lt", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias),
-                          out.data_ptr(), out.stride(0) if M > 1 else N, M, N, K, self._lt_work.data_ptr(),
-                          self._lt_work.numel(), self._stream())
-            return
+            return self.lib.offer("mv_gemm_lt", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias),
+                                  out.data_ptr(), out.stride(0) if M > 1 else N, _CODES[out.dtype], M, N, K,
+                                  self._lt_work.data_ptr(), self._lt_work.numel(), self._stream())
+        if out.dtype != self.dtype:
+            return False                 # float32 comes only from the direct call
         wt = self._transposed.get(w.data_ptr())
         if wt is None or wt.shape != (K, N):
             wt = self._transposed[w.data_ptr()] = w.t()      # the view is made once per weight
@@ -379,8 +389,9 @@ class Ops:
             torch.mm(a, wt, out=out)
         else:
             torch.addmm(bias, a, wt, out=out)
+        return True
 
-    def _library_allowed(self, M: int, N: int, K: int, with_bias: bool) -> bool:
+    def _library_allowed(self, M: int, N: int, K: int, with_bias: bool, out_dtype: torch.dtype = torch.bfloat16) -> bool:
         """Whether the library's matrix product may serve this shape now. Outside graphs: whenever it
         is switched on. For a graph: only when a graph holding just this product, replayed several
         times with other work and synchronisations in between, gave the eager result every time
@@ -391,23 +402,25 @@ class Ops:
             return False
         if not self.for_graph:
             return True
-        key = (M, N, K, with_bias)
+        key = (M, N, K, with_bias) if out_dtype == torch.bfloat16 else (M, N, K, with_bias, out_dtype)
         ok = self._library_in_graph.get(key)
         if ok is None:
             if torch.cuda.is_current_stream_capturing():
                 return False
-            ok = self._library_in_graph[key] = self._rehearse_library_product(M, N, K, with_bias)
+            ok = self._library_in_graph[key] = self._rehearse_library_product(M, N, K, with_bias, out_dtype)
         return ok
 
-    def _rehearse_library_product(self, M: int, N: int, K: int, with_bias: bool) -> bool:
+    def _rehearse_library_product(self, M: int, N: int, K: int, with_bias: bool,
+                                  out_dtype: torch.dtype = torch.bfloat16) -> bool:
         dev = torch.device("cuda", torch.cuda.current_device())
         a = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
         w = torch.randn(N, K, device=dev, dtype=torch.bfloat16) * 0.05
         bias = torch.randn(N, device=dev, dtype=torch.bfloat16) if with_bias else None
-        out = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+        out = torch.empty(M, N, device=dev, dtype=out_dtype)
 
         def product(dst):
-            self._library_product(a, w, bias, dst)
+            if not self._library_product(a, w, bias, dst):
+                raise RuntimeError("the library has no algorithm for the shape")
 
         bound = self.stream_handle
         self.stream_handle = None                          # the rehearsal runs on torch's current stream

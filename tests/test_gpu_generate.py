@@ -271,7 +271,7 @@ def test_graphs_of_many_sequences_use_rehearsed_library_products(models):
         del r
     assert rel_err(runs[True], runs[False]) <= 2e-2
     verdicts = get_ops(torch.bfloat16)._library_in_graph
-    assert verdicts and all(m > 64 for (m, _, _, _) in verdicts), verdicts
+    assert verdicts and all(key[0] > 64 for key in verdicts), verdicts
     assert all(verdicts.values()), f"a library product did not replay faithfully: {verdicts}"
 
 

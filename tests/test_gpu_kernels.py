@@ -674,24 +674,36 @@ def test_gemm_weight_streaming_many_rows(M, N, K):
         ops.use_library_gemm = library
 
 
-@pytest.mark.parametrize("M,N,K,with_bias", [(65, 1024, 2048, True), (200, 336, 1024, False), (2048, 6144, 1024, False),
-                                             (300, 4096, 12288, True), (2048, 51200, 5120, False)])
-def test_gemm_many_rows_through_the_library(M, N, K, with_bias):
-    """More than 64 rows outside graphs: the library's product, called directly. The largest shape
-    is one for which the library's first choice wants more workspace than a small one would hold."""
+@pytest.mark.parametrize("M,N,K,with_bias,out_dtype", [
+    (65, 1024, 2048, True, torch.bfloat16), (200, 336, 1024, False, torch.bfloat16),
+    (2048, 6144, 1024, False, torch.bfloat16), (300, 4096, 12288, True, torch.bfloat16),
+    (2048, 51200, 5120, False, torch.bfloat16), (128, 151936, 1024, False, torch.float32),
+    (70, 1001, 96, True, torch.float32), (400, 50021, 4096, False, torch.float32)])
+def test_gemm_many_rows_through_the_library(M, N, K, with_bias, out_dtype):
+    """More than 64 rows outside graphs: the library's product, called directly, into the activation
+    type or into float32 (the logits of many rows). The largest bf16 shape is one for which the
+    library's first choice wants more workspace than a small one would hold."""
     ops = ops_for(torch.bfloat16)
     assert ops.lib.has("mv_gemm_lt")
     g = torch.Generator(device="cuda").manual_seed(29)
     a = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
     w = (torch.randn(N, K, generator=g, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
     b = torch.randn(N, generator=g, device="cuda").to(torch.bfloat16) if with_bias else None
-    out = torch.full((M, N + 8), float("nan"), dtype=torch.bfloat16, device="cuda")[:, :N]   # rows in a wider buffer
-    ops.gemm(a, w, out, b)
+    out = torch.full((M, N + 8), float("nan"), dtype=out_dtype, device="cuda")[:, :N]   # rows in a wider buffer
+    calls = []
+    real = ops._library_product
+    ops._library_product = lambda *args: (calls.append(1), real(*args))[1]
+    try:
+        ops.gemm(a, w, out, b)
+    finally:
+        del ops._library_product
+    assert calls, "the shape was left to another kernel"
     cols = torch.arange(0, N, max(1, N // 512), device="cuda")
     want = a.double() @ w[cols].double().T
     if with_bias:
         want = want + b[cols].double()
-    assert rel_err(out[:, cols].float().cpu().numpy(), want.cpu().numpy()) <= OP_TOL[torch.bfloat16]
+    tol = OP_TOL[torch.bfloat16] if out_dtype == torch.bfloat16 else 3e-6
+    assert rel_err(out[:, cols].float().cpu().numpy(), want.cpu().numpy()) <= tol
     assert bool(torch.isfinite(out.float()).all())
 
 
