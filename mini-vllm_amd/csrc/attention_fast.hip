@@ -127,8 +127,9 @@ __device__ __forceinline__ void norm_rotate(const Frag (&raw)[DS], int g, const 
         for (int e = 0; e < 8; ++e) dst[s].s[e] = f32_to_bf16_bits(x[s][e]);
 }
 
-template <int D, int W, bool FUSED>
-__global__ void __launch_bounds__(64 * W)
+// OCC workgroups are to share a compute unit (W / 4 waves of each on every SIMD): the register budget.
+template <int D, int W, bool FUSED, int OCC>
+__global__ void __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(OCC * W / 4, OCC * W / 4)))
 attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                       const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                       const int* __restrict__ block_table, int bt_width, int page_size,
@@ -524,12 +525,12 @@ __global__ void attention_merge_kernel(const float* __restrict__ partials, bf16*
     }
 }
 
-template <int D, int W, bool FUSED>
+template <int D, int W, bool FUSED, int OCC>
 static void launch_decode(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                           int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv,
                           float scale, int window, float* partials, int nsplit, const FusedInput& fz) {
-    hipLaunchKernelGGL((attention_decode_kernel<D, W, FUSED>), grid, dim3(64 * W), 0, stream, (const bf16*)q, q_stride,
+    hipLaunchKernelGGL((attention_decode_kernel<D, W, FUSED, OCC>), grid, dim3(64 * W), 0, stream, (const bf16*)q, q_stride,
                        (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,
                        page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit, fz);
 }
@@ -558,9 +559,25 @@ static int decode_common(bool fused, const FusedInput& fz, const void* q, long q
     if (n_seqs <= 0) return 0;
     dim3 grid(n_seqs, Hkv, nsplit);
     float* part = nsplit > 1 ? partials : nullptr;
+    // With more workgroups than compute units, two of them share a unit (the kernel is then held to
+    // 256 registers a lane, which costs it three spilled ones at head size 128): one's set-up and
+    // tail overlap the other's stream of keys, 4-6 % on a step of 64 to 256 sequences. A grid that
+    // fits the chip at once keeps all registers.
+    const int occ = (long)n_seqs * Hkv * nsplit > 256 ? 2 : 1;
 #define AF_LAUNCH(DD, WW, FF)                                                                                     \
-    launch_decode<DD, WW, FF>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,  \
-                              page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, part, nsplit, fz)
+    do {                                                                                                          \
+        if constexpr (WW == 4) {                                                                                  \
+            if (occ == 2) {                                                                                       \
+                launch_decode<DD, WW, FF, 2>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages,        \
+                                             block_table, bt_width, page_size, positions, cu_seqlens, n_seqs, H,  \
+                                             Hkv, scale, window, part, nsplit, fz);                               \
+                break;                                                                                            \
+            }                                                                                                     \
+        }                                                                                                         \
+        launch_decode<DD, WW, FF, 1>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,   \
+                                     bt_width, page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window,   \
+                                     part, nsplit, fz);                                                           \
+    } while (0)
     if (fused) {
         MV_REQUIRE(waves == 4, "attention_decode_fused: %d waves per workgroup (4 only)", waves);
         if (D == 128) AF_LAUNCH(128, 4, true);

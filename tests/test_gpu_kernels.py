@@ -443,6 +443,62 @@ def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
     assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
 
 
+@pytest.mark.parametrize("H,Hkv,D", [(16, 8, 128), (8, 8, 64)])
+@pytest.mark.parametrize("fused", [False, True])
+def test_attention_decode_with_more_workgroups_than_compute_units(H, Hkv, D, fused):
+    """Forty sequences of eight kv heads: more workgroups than the chip has compute units, for
+    which the kernel is built with half the registers so that two workgroups share a unit. Both
+    forms: finished queries against a finished cache, and raw rows whose key and value the kernel
+    writes itself."""
+    ops = ops_for(torch.bfloat16)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(44)
+    ps, n = 16, 40
+    assert n * Hkv > 256
+    ctx_lens = [int(c) for c in torch.randint(1, 400, (n,), generator=g)]
+    ctx_lens[3], ctx_lens[17] = 1, 16
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    pages_per = [-(-c // ps) for c in ctx_lens]
+    num_pages = sum(pages_per) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, cur = [], 0
+    for n_p in pages_per:
+        tables.append(perm[cur:cur + n_p]); cur += n_p
+    kp, vp = fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype)
+    bt = torch.full((n, max(pages_per)), -1, dtype=torch.int32)
+    for s_, t in enumerate(tables):
+        bt[s_, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    positions = torch.tensor([c - 1 for c in ctx_lens], dtype=torch.int32)
+    token_seq = torch.arange(n, dtype=torch.int32)
+    q = torch.randn(n, H, D, generator=g)
+    for s_ in range(n):
+        if ctx_lens[s_] > 40:           # a far key stands out
+            q[s_] = 6.0 * k_all[s_][3].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
+    q = q.to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.full((n, H * D), float("nan"), dtype=dtype, device="cuda")
+    plan = make_plan([1] * n, ctx_lens, decode_only=True)
+    if fused:
+        raw = torch.cat([q.view(n, -1)] + [torch.stack([x[c - 1] for x, c in zip(kv, ctx_lens)]).to(dtype).view(n, -1)
+                                           for kv in (k_all, v_all)], dim=1)
+        for s_, c in enumerate(ctx_lens):        # the new slots are not written yet
+            kp[tables[s_][(c - 1) // ps], :, (c - 1) % ps, :] = float("nan")
+            vp[tables[s_][(c - 1) // ps], :, :, (c - 1) % ps] = float("nan")
+        assert ops.attention_decode_fused(dev(raw), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D,
+                                          scale, None, plan, None, None, 1e-6, None, False, True)
+    else:
+        ops.attention(dev(q.view(n, H * D)), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale,
+                      None, plan=plan)
+    want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, None)
+    assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+    if fused:
+        for s_, c in enumerate(ctx_lens):
+            page, slot = tables[s_][(c - 1) // ps], (c - 1) % ps
+            assert torch.equal(kp[page, :, slot, :].float().cpu().double(), k_all[s_][c - 1])
+            assert torch.equal(vp[page, :, :, slot].float().cpu().double(), v_all[s_][c - 1])
+
+
 def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
     """One workgroup walks 18,000 keys (1,125 pages of 16): more page ids than it keeps in LDS, the
     rest are read from the block table as it goes."""
