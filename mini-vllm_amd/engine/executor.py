@@ -69,6 +69,21 @@ class _Staging:
         ev.record()
 
 
+class RepeatedRun:
+    """Decode steps in a row that were launched and may still be running."""
+
+    def __init__(self, host: torch.Tensor, done: torch.cuda.Event, device_tokens: torch.Tensor, repeat: int,
+                 bucket: int, count: int):
+        self.host, self.done, self.device_tokens = host, done, device_tokens
+        self.repeat, self.bucket, self.count = repeat, bucket, count
+
+    def tokens(self) -> np.ndarray:
+        """Waits for the launch; the drawn tokens, int32 [repeat, sequences]."""
+        self.done.synchronize()
+        n = self.repeat * self.bucket
+        return self.host[:n].numpy().reshape(self.repeat, self.bucket)[:, :self.count].copy()
+
+
 class Executor:
     def __init__(self, config: EngineConfig, model: Optional[Tuple[Architecture, object, TensorSource]] = None,
                  device: str = "cuda:0"):
@@ -126,6 +141,9 @@ class Executor:
         self._graph_pool = None
         self._repeat_graphs: Dict[Tuple[int, int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
         self._graph_workspace: Optional[Workspace] = None
+        # pinned buffers for the tokens of launches in flight, used in turn (two launches at most are)
+        self._token_buffers: List[Optional[torch.Tensor]] = [None] * 4
+        self._next_token_buffer = 0
         self.kv_pages: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
         self.state_tensors: Dict[int, torch.Tensor] = {}
         self.num_pages = 0
@@ -419,14 +437,41 @@ class Executor:
     def can_repeat(self, num_seqs: int) -> bool:
         return bool(self.config.use_cuda_graph) and self.model.graph_safe and num_seqs <= GRAPH_BUCKETS[-1]
 
-    @torch.inference_mode()
     def step_repeated(self, seqs: Sequence[SeqStep], repeat: int, temperature: np.ndarray, top_k: np.ndarray,
                       top_p: np.ndarray, seeds: np.ndarray, counters: np.ndarray) -> np.ndarray:
+        """``launch_repeated`` and the wait for its tokens, int32 [repeat, len(seqs)]."""
+        return self.launch_repeated(seqs, repeat, temperature, top_k, top_p, seeds, counters).tokens()
+
+    def repeat_ready(self, seqs: Sequence[SeqStep], repeat: int, lookahead: int = 0) -> bool:
+        """Whether the graph that ``launch_repeated`` would replay for these sequences, ``lookahead``
+        positions further on, exists already (its first use captures it, which waits for the device)."""
+        S = len(seqs)
+        if not self.can_repeat(S):
+            return False
+        bucket = next(b for b in GRAPH_BUCKETS if b >= S)
+        return (bucket, self._repeat_cap(seqs, repeat + lookahead), repeat) in self._repeat_graphs
+
+    def _repeat_cap(self, seqs: Sequence[SeqStep], span: int) -> int:
+        longest = max(s.start + span for s in seqs)
+        cap = 1024
+        while cap < longest:
+            cap *= 2
+        return min(cap, max(self.config.max_model_len, 1))
+
+    @torch.inference_mode()
+    def launch_repeated(self, seqs: Sequence[SeqStep], repeat: int, temperature: np.ndarray, top_k: np.ndarray,
+                        top_p: np.ndarray, seeds: np.ndarray, counters: np.ndarray,
+                        after: Optional["RepeatedRun"] = None) -> "RepeatedRun":
         """Runs a step of single decoded tokens ``repeat`` times in a row, as one graph: every run
         draws a token per sequence (per-sequence sampling arrays of length len(seqs); ``counters``
         is the index of the first token each sequence draws) and the next run takes it as its
         input at the next position. The sequences must hold pages for all ``repeat`` positions.
-        Returns the drawn tokens, int32 [repeat, len(seqs)]."""
+        Returns at once; the handle's ``tokens()`` waits for the drawn tokens.
+
+        With ``after`` (the launch before, of the same sequences in the same order, possibly still
+        running) the input tokens are not the ones in ``seqs`` but the last ones that launch drew,
+        taken on the device: the host has not seen them yet. ``seqs`` then says where they go
+        (``start`` = the position after that launch's last)."""
         S = len(seqs)
         if not self.can_repeat(S) or repeat < 1 or any(len(s.tokens) != 1 or list(s.want) != [0] for s in seqs):
             raise ValueError("a repeated step takes graph-sized batches of single tokens, each wanted")
@@ -437,11 +482,9 @@ class Executor:
                     for t in self.state_tensors.values():
                         t[s.state_slot].zero_()
         bucket = next(b for b in GRAPH_BUCKETS if b >= S)
-        longest = max(s.start + repeat for s in seqs)
-        cap = 1024
-        while cap < longest:
-            cap *= 2
-        cap = min(cap, max(self.config.max_model_len, 1))
+        cap = self._repeat_cap(seqs, repeat)
+        if after is not None and (after.bucket != bucket or after.count != S):
+            raise ValueError("a launch that follows another takes the same sequences")
         widths = [self.max_pages_per_seq] * len(self.groups)
         # sampling arrays behind the step's integers: temperature, top_k, top_p, (seed, counter) pairs
         arr, off, facts = self._fill(seqs, pad_to=bucket, bt_widths=widths, lookahead=repeat - 1,
@@ -462,8 +505,20 @@ class Executor:
             entry = self._capture_repeated(key, arr, off, facts, seqs)
         graph, meta, tokens = entry
         self._upload(arr, dst=meta)
+        if after is not None:
+            o_tok = off["token_ids"][0]
+            meta[o_tok:o_tok + bucket].copy_(after.device_tokens[after.repeat - 1])
         graph.replay()
-        return tokens[:, :S].cpu().numpy()
+        # the tokens go to pinned memory at once, before a later launch of the same graph overwrites them
+        host = self._token_buffers[self._next_token_buffer]
+        if host is None or host.numel() < tokens.numel():
+            host = torch.empty(max(tokens.numel(), 4096), dtype=torch.int32, pin_memory=True)
+            self._token_buffers[self._next_token_buffer] = host
+        self._next_token_buffer = (self._next_token_buffer + 1) % len(self._token_buffers)
+        host[:tokens.numel()].copy_(tokens.view(-1), non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return RepeatedRun(host, done, tokens, repeat, bucket, S)
 
     def _capture_repeated(self, key, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
         bucket, cap, repeat = key
