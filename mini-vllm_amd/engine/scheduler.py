@@ -213,6 +213,31 @@ class Scheduler:
             self.manager.reserve(s.request.id, k)
         return k
 
+    def schedule_ahead(self, prev: ScheduledStep) -> Optional[ScheduledStep]:
+        """The step after ``prev`` while ``prev`` is still running and its tokens are unknown: the
+        same requests, ``prev.repeat`` positions further on, again ``prev.repeat`` runs in a row.
+        Only when that is what ``schedule`` would decide whatever the tokens turn out to be, short of
+        a request ending on an end-of-sequence token: nobody waits, ``prev`` holds every running
+        request as a decoded token, every request has the tokens of both steps to go, and the pages
+        for them are free (they are reserved here). None otherwise; nothing is changed then.
+        What such a step computes for a request that ``prev`` ends is dropped by ``update``."""
+        k = prev.repeat
+        if k <= 1 or k != self.max_decode_repeat or self.waiting or len(prev.seqs) != len(self.running):
+            return None
+        for s in prev.seqs:
+            r = s.request
+            if r.state != RequestState.RUNNING or not s.is_decode or not s.sample:
+                return None
+            if min(r.sampling_params.max_tokens - r.num_completion_tokens, self.max_model_len - len(r.tokens)) < 2 * k:
+                return None
+        extra = [self.manager.pages_needed(s.request.id, 2 * k) for s in prev.seqs]
+        for g in range(len(self.manager.groups)):
+            if sum(e[g] for e in extra) > self.manager.pools[g].num_free:
+                return None
+        for s in prev.seqs:
+            self.manager.reserve(s.request.id, 2 * k)
+        return ScheduledStep([ScheduledSeq(s.request, s.start + k, 1, sample=True) for s in prev.seqs], repeat=k)
+
     def schedule(self) -> Optional[ScheduledStep]:
         """The next step, or None when nothing is left to do."""
         while True:
@@ -237,6 +262,8 @@ class Scheduler:
         now = time.perf_counter()
         for seq, drawn in zip(step.seqs, sampled):
             req = seq.request
+            if req.state == RequestState.FINISHED:
+                continue          # a step scheduled ahead ran on for a request that the step before ended
             if not seq.sample:
                 self.manager.commit(req.id, seq.num_tokens, req.tokens)
                 continue

@@ -46,33 +46,15 @@ class FakeEngine:
         step = self.sched.schedule()
         if step is None:
             return None
+        return self.run_scheduled(step)
+
+    def run_scheduled(self, step):
         assert step.num_tokens <= self.sched.max_num_batched_tokens
         assert len(step.seqs) <= self.sched.max_num_batched_seqs
         assert len({s.request.id for s in step.seqs}) == len(step.seqs)
         sampled = []
         if step.repeat > 1:
-            # the device's part: every run writes the newest token and draws the next from the cache
-            assert not self.sched.waiting and all(s.is_decode and s.sample for s in step.seqs)
-            for s in step.seqs:
-                r = s.request
-                seq = self.manager.sequence(r.id)
-                assert s.start == seq.num_computed == len(r.tokens) - 1
-                assert r.num_completion_tokens + step.repeat <= r.sampling_params.max_tokens
-                toks, drawn = list(r.tokens), []
-                for j in range(step.repeat):
-                    pos = s.start + j
-                    contexts = []
-                    for g, spec in enumerate(self.groups):
-                        table = seq.pages[g]
-                        assert table[pos // self.ps] >= 0
-                        self.mem[g][(table[pos // self.ps], pos % self.ps)] = toks[pos]
-                        lo = 0 if spec.retention == "full" else max(0, pos - spec.window)
-                        ctx = [self.mem[g][(table[p // self.ps], p % self.ps)] for p in range(lo, pos + 1)]
-                        assert ctx == toks[lo:pos + 1], "the cache does not hold the request's tokens"
-                        contexts.append(ctx)
-                    t = next_token(contexts[0])
-                    toks.append(t); drawn.append(t)
-                sampled.append(drawn)
+            sampled = self.device_runs(step)
             self.steps.append(step)
             done = self.sched.update(step, sampled)
             self.manager.check_invariants()
@@ -105,6 +87,61 @@ class FakeEngine:
         done = self.sched.update(step, sampled)
         self.manager.check_invariants()
         return step, done
+
+    def device_runs(self, step, before=None):
+        """The device's part of a step that runs several times in a row: every run writes the
+        newest token and draws the next from the cache. ``before``: what the launch before drew for
+        the same requests, which the host has not recorded yet (a step scheduled ahead)."""
+        assert not self.sched.waiting and all(s.is_decode and s.sample for s in step.seqs)
+        sampled = []
+        for i, s in enumerate(step.seqs):
+            r = s.request
+            seq = self.manager.sequence(r.id)
+            toks, drawn = list(r.tokens) + (before[i] if before else []), []
+            assert s.start == len(toks) - 1 and seq.num_computed == len(r.tokens) - 1
+            assert r.num_completion_tokens + len(toks) - len(r.tokens) + step.repeat <= r.sampling_params.max_tokens
+            for j in range(step.repeat):
+                pos = s.start + j
+                contexts = []
+                for g, spec in enumerate(self.groups):
+                    table = seq.pages[g]
+                    assert table[pos // self.ps] >= 0
+                    self.mem[g][(table[pos // self.ps], pos % self.ps)] = toks[pos]
+                    lo = 0 if spec.retention == "full" else max(0, pos - spec.window)
+                    ctx = [self.mem[g][(table[p // self.ps], p % self.ps)] for p in range(lo, pos + 1)]
+                    assert ctx == toks[lo:pos + 1], "the cache does not hold the request's tokens"
+                    contexts.append(ctx)
+                t = next_token(contexts[0])
+                toks.append(t); drawn.append(t)
+            sampled.append(drawn)
+        return sampled
+
+    def run_all_launching_ahead(self, limit=100000):
+        """As an engine that launches the next step of decoded tokens before it has read the
+        tokens of the one that runs. Returns how many steps were scheduled ahead."""
+        ahead_count = n = 0
+        in_flight = None                                   # (step, what the device drew)
+        while in_flight is not None or not self.sched.finished:
+            n += 1
+            assert n < limit, "the scheduler does not terminate"
+            if in_flight is None:
+                step = self.sched.schedule()
+                assert step is not None
+                if step.repeat == 1:
+                    self.run_scheduled(step)
+                    continue
+                in_flight = (step, self.device_runs(step))
+            step, drawn = in_flight
+            in_flight = None
+            nxt = self.sched.schedule_ahead(step)
+            if nxt is not None:
+                ahead_count += 1
+                assert nxt.repeat == step.repeat and [s.request for s in nxt.seqs] == [s.request for s in step.seqs]
+                in_flight = (nxt, self.device_runs(nxt, before=drawn))
+            self.steps.append(step)
+            self.sched.update(step, drawn)
+            self.manager.check_invariants()
+        return ahead_count
 
     def run_all(self, limit=100000):
         n = 0
@@ -305,3 +342,51 @@ def test_repeat_with_a_window_group():
         assert r.completion_tokens == expected_output(r.prompt_tokens, 19)
     assert max(st.repeat for st in e.steps) == 4
     assert all(p.num_free == p.num_pages for p in e.manager.pools)
+
+
+@pytest.mark.parametrize("use_eos", [False, True])
+@pytest.mark.parametrize("seed", range(6))
+def test_steps_scheduled_ahead_give_the_same_tokens(seed, use_eos):
+    """The next step of decoded tokens is launched before the tokens of the running one are known:
+    the same tokens as step by step; what ran on for a request that ended on an end token is
+    dropped with its pages; near max_tokens, max_model_len or the pool's end nothing is launched
+    ahead."""
+    rng = random.Random(100 + seed)
+    prompts = [[rng.randrange(VOCAB) for _ in range(rng.randrange(1, 30))] for _ in range(7)]
+    limits = [rng.randrange(1, 60) for _ in prompts]
+    e = FakeEngine(num_pages=rng.choice([40, 64, 200]), page_size=4, max_tokens=32, max_seqs=rng.choice([2, 4, 8]),
+                   repeat=rng.choice([2, 4]), max_model_len=rng.choice([50, 4096]))
+    reqs = [submit(e, p, max_tokens=m, ignore_eos=not use_eos) for p, m in zip(prompts, limits)]
+    ahead = e.run_all_launching_ahead()
+    for r, m in zip(reqs, limits):
+        want = expected_output(r.prompt_tokens, min(m, 50 - len(r.prompt_tokens)) if e.sched.max_model_len == 50 else m,
+                               ignore_eos=not use_eos)
+        assert r.completion_tokens == want, (r.id, ahead)
+        assert r.state == RequestState.FINISHED
+    assert all(p.num_free == p.num_pages for p in e.manager.pools)
+    assert e.manager.slots.num_free == e.manager.slots.num_slots if hasattr(e.manager.slots, "num_slots") else True
+
+
+def test_steps_are_scheduled_ahead_when_nothing_can_change():
+    e = FakeEngine(num_pages=64, page_size=4, max_tokens=32, max_seqs=4, repeat=4)
+    rng = random.Random(5)
+    reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=41, ignore_eos=True) for n in (3, 9)]
+    ahead = e.run_all_launching_ahead()
+    assert ahead >= 7                        # 41 tokens = 1 + 10 steps of 4, all but the last launched ahead
+    for r in reqs:
+        assert r.completion_tokens == expected_output(r.prompt_tokens, 41)
+    # fewer tokens to go than both steps draw, or fewer free pages than both need: nothing is
+    # launched ahead and nothing is reserved
+    for pages, limit in ((64, 7), (5, 9)):
+        e = FakeEngine(num_pages=pages, page_size=4, max_tokens=32, max_seqs=2, repeat=4)
+        a = submit(e, [1, 2, 3], max_tokens=limit, ignore_eos=True)
+        b = submit(e, [4, 5, 6], max_tokens=limit, ignore_eos=True)
+        e.run_scheduled(e.sched.schedule())      # the prompts
+        step = e.sched.schedule()
+        assert step.repeat == 4 and not e.sched.waiting
+        free = [p.num_free for p in e.manager.pools]
+        assert e.sched.schedule_ahead(step) is None and [p.num_free for p in e.manager.pools] == free
+        e.sched.update(step, e.device_runs(step))
+        e.run_all()
+        assert a.completion_tokens == expected_output(a.prompt_tokens, limit)
+        assert b.completion_tokens == expected_output(b.prompt_tokens, limit)
