@@ -48,6 +48,10 @@ class EngineConfig:
     # decode-only steps run this many times in a row on the device before the host looks at the
     # tokens (1: every step comes back to the host)
     num_scheduler_steps: int = 4
+    # such a row of steps is launched before the tokens of the row that runs have been read, where
+    # nothing but an end-of-sequence token could change what it holds (what ran on for a request
+    # that ended is dropped)
+    launch_ahead: bool = False
     seed: int = 0
 
     def __post_init__(self) -> None:

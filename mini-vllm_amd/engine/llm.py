@@ -21,7 +21,7 @@ from ..config.sampling_params import SamplingParams
 from ..sampling.sampler import Sampler, request_seed
 from .executor import Executor
 from .metrics import Metrics
-from .request import Request, RequestOutput
+from .request import Request, RequestOutput, RequestState
 from .scheduler import ScheduledStep, Scheduler
 from .step import SeqStep
 
@@ -65,6 +65,9 @@ class LLM:
         self.sampler = Sampler(self.executor.ops, self.executor.device)
         self.metrics = Metrics()
         self._seeds: Dict[int, int] = {}
+        # a row of decode steps that was launched ahead and is waited for by the next step():
+        # (scheduled step, the executor's handle, the seeds of its requests)
+        self._in_flight = None
 
     # ---- the reference's streaming interface ---------------------------------------------
     def submit(self, tokens: Sequence[int], sampling_params: Optional[SamplingParams] = None) -> Request:
@@ -88,18 +91,25 @@ class LLM:
     def step(self) -> Optional[ScheduledStep]:
         """One step of the engine: schedule, run the batch, draw tokens, record them."""
         t0 = time.perf_counter()
-        step = self.scheduler.schedule()
-        if step is None:
-            return None
-        groups = range(len(self.manager.groups))
-        seqs = []
-        for s in step.seqs:
-            r = s.request
-            cache = self.manager.sequence(r.id)
-            seqs.append(SeqStep(tokens=r.tokens[s.start:s.start + s.num_tokens], start=s.start,
-                                block_tables=[cache.table(g) for g in groups], state_slot=cache.state_slot,
-                                want=[s.num_tokens - 1] if s.sample else []))
-        if step.repeat > 1:
+        run = None
+        if self._in_flight is not None:
+            step, run = self._in_flight
+            self._in_flight = None
+            if all(r.state == RequestState.FINISHED for r in step.requests):
+                run.tokens()                         # everything it ran for has ended: wait and forget it
+                run = None
+        if run is None:
+            step = self.scheduler.schedule()
+            if step is None:
+                return None
+            seqs = self._seq_steps(step)
+            if step.repeat > 1 and self.executor.can_repeat(len(seqs)):
+                run = self.executor.launch_repeated(seqs, step.repeat, *self._sampling_arrays(step))
+        if run is not None:
+            self._launch_ahead(step, run)
+            drawn = run.tokens()
+            sampled = [[int(t) for t in drawn[:, i]] for i in range(len(step.seqs))]
+        elif step.repeat > 1:
             sampled = self._run_repeated(step, seqs)
         else:
             logits = self.executor.step(seqs)
@@ -109,7 +119,6 @@ class LLM:
                                          [r.num_completion_tokens for r in drawing])
             it = iter(tokens)
             sampled = [next(it) if s.sample else None for s in step.seqs]
-        preempted_before = self.scheduler.num_preemptions
         done = self.scheduler.update(step, sampled)
         for r in done:
             self._seeds.pop(r.id, None)
@@ -118,17 +127,50 @@ class LLM:
         step.finished = done
         return step
 
+    def _seq_steps(self, step: ScheduledStep, further: int = 0) -> List[SeqStep]:
+        """What the executor runs for a scheduled step. ``further``: the step was scheduled ahead of
+        one that draws that many tokens per request first; its own input tokens are on the device."""
+        groups = range(len(self.manager.groups))
+        seqs = []
+        for s in step.seqs:
+            r = s.request
+            cache = self.manager.sequence(r.id)
+            tokens = [0] * s.num_tokens if further else r.tokens[s.start:s.start + s.num_tokens]
+            seqs.append(SeqStep(tokens=tokens, start=s.start, block_tables=[cache.table(g) for g in groups],
+                                state_slot=cache.state_slot, want=[s.num_tokens - 1] if s.sample else []))
+        return seqs
+
+    def _sampling_arrays(self, step: ScheduledStep, further: int = 0):
+        reqs = step.requests
+        return Sampler.arrays([r.sampling_params for r in reqs], [self._seeds[r.id] for r in reqs],
+                              [r.num_completion_tokens + further for r in reqs])
+
+    def _launch_ahead(self, step: ScheduledStep, run) -> None:
+        """While ``run`` (the decode steps of ``step``) is on the device and its tokens are unknown:
+        launches the steps after it, if the scheduler can tell what they hold and their graph
+        exists; the next ``step()`` waits for them."""
+        if not self.config.launch_ahead:
+            return
+        probe = [SeqStep(tokens=[0], start=s.start + step.repeat, block_tables=[], state_slot=0, want=[0])
+                 for s in step.seqs]
+        if not self.executor.repeat_ready(probe, step.repeat):
+            return                                   # its first use captures the graph, which waits for the device
+        ahead = self.scheduler.schedule_ahead(step)
+        if ahead is None:
+            return
+        seqs = self._seq_steps(ahead, further=step.repeat)
+        nxt = self.executor.launch_repeated(seqs, ahead.repeat, *self._sampling_arrays(ahead, further=step.repeat),
+                                            after=run)
+        self._in_flight = (ahead, nxt)
+
     def _run_repeated(self, step: ScheduledStep, seqs: List[SeqStep]) -> List[List[int]]:
-        """A step of decoded tokens that runs ``step.repeat`` times in a row: as one graph on the
-        device where the executor offers that, else run by run from here. Returns the tokens each
-        sequence drew, in order."""
-        reqs = [s.request for s in step.seqs]
+        """A step of decoded tokens that runs ``step.repeat`` times in a row where the executor
+        offers no graph for it: run by run from here. Returns the tokens each sequence drew, in
+        order."""
+        reqs = step.requests
         params = [r.sampling_params for r in reqs]
         seeds = [self._seeds[r.id] for r in reqs]
         counters = [r.num_completion_tokens for r in reqs]
-        if self.executor.can_repeat(len(seqs)):
-            drawn = self.executor.step_repeated(seqs, step.repeat, *Sampler.arrays(params, seeds, counters))
-            return [[int(t) for t in drawn[:, i]] for i in range(len(seqs))]
         out: List[List[int]] = [[] for _ in seqs]
         for j in range(step.repeat):
             if j:

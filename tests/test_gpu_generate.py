@@ -247,6 +247,51 @@ def test_decode_steps_in_a_row_give_the_same_tokens(models, dtype):
     assert cut == ref and why_cut == why_ref and "stop" in why_cut
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_launching_ahead_gives_the_same_tokens(models, dtype):
+    """Rows of decode steps launched before the tokens of the running row are read: the same tokens
+    as without, for greedy and drawn tokens, requests that end on an end token in the middle of a
+    row (what ran on for them is dropped), different lengths, and a late arrival."""
+    from minivllm_amd import LLM, SamplingParams
+    cfg, w, path = models["B"]
+    prompts = [random_tokens(cfg, n, seed=300 + n) for n in (5, 21, 40, 3, 17, 9)]
+    params = [SamplingParams(temperature=0.0, max_tokens=37, ignore_eos=True),
+              SamplingParams(temperature=0.8, top_k=20, max_tokens=50, ignore_eos=True, seed=11),
+              SamplingParams(temperature=0.0, max_tokens=64),
+              SamplingParams(temperature=1.0, top_p=0.9, max_tokens=29, seed=12),
+              SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True),
+              SamplingParams(temperature=0.7, max_tokens=45, seed=13)]
+
+    def run(ahead, eos_ids):
+        llm = LLM(model=path, dtype=dtype, kv_cache_block_size=8, kv_cache_num_blocks=64, max_model_len=128,
+                  max_num_batched_tokens=64, max_num_batched_seqs=8, num_scheduler_steps=4, launch_ahead=ahead,
+                  eos_token_ids=eos_ids, seed=5)
+        reqs = [llm.submit(p, sp) for p, sp in zip(prompts[:5], params[:5])]
+        steps = launched = 0
+        while not llm.finished:
+            llm.step()
+            steps += 1
+            launched += llm._in_flight is not None
+            if steps == 7:
+                reqs.append(llm.submit(prompts[5], params[5]))
+        assert ahead == (launched > 0)
+        llm.step()                                    # a row that may still be in flight is waited for
+        assert llm._in_flight is None
+        llm.manager.check_invariants()
+        assert all(p.num_free == p.num_pages for p in llm.manager.pools)
+        return [list(r.completion_tokens) for r in reqs]
+
+    never = (cfg["vocab_size"] - 1,)
+    base = run(False, never)
+    assert base == run(True, never)
+    # an end token that the greedy request 2 meets in the middle of a row of four
+    stop = base[2][13]
+    ends_at = base[2].index(stop)
+    off = run(False, (stop,))
+    assert off == run(True, (stop,))
+    assert off[2] == base[2][:ends_at + 1] and off[0] == base[0]      # request 0 ignores end tokens
+
+
 def test_graphs_of_many_sequences_use_rehearsed_library_products(models):
     """Decode steps of more than 64 sequences: inside a graph the library's matrix product serves
     the shapes that passed a rehearsal (a graph of just that product, replayed against eager runs);
