@@ -81,6 +81,8 @@ def build_llm(args, shape, layers, max_seqs=None, token_budget=None, num_pages=N
                       kv_cache_block_size=args.block_size,
                       kv_cache_num_blocks=num_pages or max(64, args.batch) * pages_per_seq + 16,
                       use_cuda_graph=not args.no_graph, num_scheduler_steps=args.scheduler_steps, seed=args.seed)
+    if getattr(args, "launch_ahead", None) is not None:
+        ec.launch_ahead = bool(args.launch_ahead)
     return LLM(config=ec, model_source=(arch, cfg, source)), cfg
 
 
@@ -181,6 +183,8 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--scheduler-steps", type=int, default=4,
                     help="decode steps run in a row on the device before the host looks at the tokens")
+    ap.add_argument("--launch-ahead", type=int, choices=[0, 1], default=None,
+                    help="launch the next decode steps before the running ones' tokens are read (default: the engine's)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", "--mode", dest="only", choices=["all", "decode", "prefill", "serve"], default="all",

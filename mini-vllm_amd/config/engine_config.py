@@ -51,7 +51,7 @@ class EngineConfig:
     # such a row of steps is launched before the tokens of the row that runs have been read, where
     # nothing but an end-of-sequence token could change what it holds (what ran on for a request
     # that ended is dropped)
-    launch_ahead: bool = False
+    launch_ahead: bool = True
     seed: int = 0
 
     def __post_init__(self) -> None:

@@ -43,6 +43,8 @@ def add_engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--no-cuda-graph", action="store_true", help="run decode steps eagerly (no HIP graph)")
     ap.add_argument("--num-scheduler-steps", type=int, default=4,
                     help="decode-only steps run this many times in a row on the device (1: one token per step)")
+    ap.add_argument("--no-launch-ahead", action="store_true",
+                    help="read the tokens of a row of decode steps before the next row is launched")
     ap.add_argument("--seed", type=int, default=0)
 
 
@@ -63,7 +65,7 @@ def engine_config_from(args):
                         kv_cache_block_size=args.kv_cache_block_size, kv_cache_num_blocks=args.kv_cache_num_blocks,
                         gpu_memory_utilization=args.gpu_memory_utilization,
                         enable_prefix_caching=args.enable_prefix_caching, use_cuda_graph=not args.no_cuda_graph,
-                        num_scheduler_steps=args.num_scheduler_steps,
+                        num_scheduler_steps=args.num_scheduler_steps, launch_ahead=not args.no_launch_ahead,
                         seed=args.seed)
 
 
