@@ -663,7 +663,7 @@ def test_gemm_weight_streaming(out_dtype, M, N, K):
     (17, 3100, 4096, False, torch.bfloat16), (64, 4096, 3072, False, torch.bfloat16),
     (40, 6144, 2048, False, torch.float32), (64, 6144, 2048, True, torch.bfloat16),
     (33, 2 * 1571, 4096, True, torch.bfloat16), (20, 151936 // 4, 1024, False, torch.float32),
-    (9, 3100, 4096, False, torch.bfloat16), (1, 151936 // 4, 4096, False, torch.float32),
+    (9, 3100, 4096, False, torch.bfloat16), (1, 151936 // 4, 4096, False, torch.bfloat16),
     (3, 2 * 12032, 5120, True, torch.bfloat16)])
 def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dtype):
     """9 to 64 rows against a weight of tens of megabytes, any number of rows up to 64 against one
@@ -734,11 +734,12 @@ def test_gemm_weight_streaming_many_rows(M, N, K):
     (65, 1024, 2048, True, torch.bfloat16), (200, 336, 1024, False, torch.bfloat16),
     (2048, 6144, 1024, False, torch.bfloat16), (300, 4096, 12288, True, torch.bfloat16),
     (2048, 51200, 5120, False, torch.bfloat16), (128, 151936, 1024, False, torch.float32),
+    (1, 151936, 1024, False, torch.float32), (8, 151936, 1024, False, torch.float32), (40, 151936, 1024, True, torch.float32),
     (70, 1001, 96, True, torch.float32), (400, 50021, 4096, False, torch.float32)])
-def test_gemm_many_rows_through_the_library(M, N, K, with_bias, out_dtype):
-    """More than 64 rows outside graphs: the library's product, called directly, into the activation
-    type or into float32 (the logits of many rows). The largest bf16 shape is one for which the
-    library's first choice wants more workspace than a small one would hold."""
+def test_gemm_through_the_library(M, N, K, with_bias, out_dtype):
+    """More than 64 rows outside graphs, and any number of rows into float32 against a very large
+    weight (the logits): the library's product, called directly. The largest bf16 shape is one for
+    which the library's first choice wants more workspace than a small one would hold."""
     ops = ops_for(torch.bfloat16)
     assert ops.lib.has("mv_gemm_lt")
     g = torch.Generator(device="cuda").manual_seed(29)
