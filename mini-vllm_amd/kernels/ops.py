@@ -28,11 +28,17 @@ MID_MIN_M = 9
 MID_MIN_WEIGHT = 12 * 1024 * 1024
 MID_ALWAYS_WEIGHT = 120 * 1000 * 1000
 MID_ALWAYS_K = 2048
-# float32 output against a weight of at least this many elements (the output head of a model with a
-# large vocabulary) goes to the library's product at any number of rows: it streams such a weight
-# at the memory's speed (0.6B-sized head: 51 against 65 us at one row, 83 against 136 at 64 rows;
-# 8B-sized: 240 against 273 and 267 against 357)
-LIBRARY_FLOAT_OUT_WEIGHT = 120 * 1000 * 1000
+# A weight with at least four times as many rows as columns and this many elements (gate/up of a large
+# model, the output head of a large vocabulary) goes to the library's product at any number of rows:
+# it streams such a weight at the memory's speed, 5.0 to 5.9 TB/s, where the engine's kernels reach
+# 3.5 to 5 (0.6B-sized head: 51 against 65 us at one row, 83 against 136 at 64 rows; 32B-sized gate/up:
+# 89 against 105 and 98 against 153). Weights with long rows it serves badly (32B-sized down: 134 us
+# against 56).
+LIBRARY_TALL_WEIGHT = 96 * 1000 * 1000
+# The gated pair in one pass (no [M, 2I] intermediate, no second kernel) keeps the smaller of these
+# weights for fewer than 16 rows (8B-sized: 44 against 46 us at 8 rows, 49 against 46 at 16); from
+# this size on the library and a separate activation kernel win at every number of rows
+LIBRARY_TALL_WEIGHT_GATED = 240 * 1000 * 1000
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
@@ -341,8 +347,8 @@ class Ops:
         lda = a.stride(0) if M > 1 else K
         ldc = out.stride(0) if M > 1 else N
         fast = self.use_fast_kernels and not exact and wcode == DTYPE_BF16
-        if (fast and out.dtype == torch.float32 and N * K >= LIBRARY_FLOAT_OUT_WEIGHT and self.lib.has("mv_gemm_lt")
-                and self._library_serves(out) and self._library_allowed(M, N, K, bias is not None, out.dtype)
+        if (fast and self.prefers_library(M, N, K) and self._library_serves(out)
+                and self._library_allowed(M, N, K, bias is not None, out.dtype)
                 and self._library_product(a, w, bias, out)):
             return None
         if fast and K % 32 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.lib.has("mv_gemm_skinny"):
@@ -365,6 +371,13 @@ class Ops:
             return
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
+
+    def prefers_library(self, M: int, N: int, K: int, gated: bool = False) -> bool:
+        """Whether a product of few rows against this weight is left to the library (see
+        LIBRARY_TALL_WEIGHT); ``gated``: the alternative is the gated pair in one pass."""
+        if not (self.use_library_gemm and self.lib.has("mv_gemm_lt")) or N < 4 * K or N * K < LIBRARY_TALL_WEIGHT:
+            return False
+        return not gated or N * K >= LIBRARY_TALL_WEIGHT_GATED or M >= 16
 
     def _library_serves(self, out: torch.Tensor) -> bool:
         """The library's product writes the activation type; called directly it also writes float32
@@ -518,6 +531,8 @@ class Ops:
             return False
         if self.wants_mid(M, w.shape[0], K) and self.lib.has("mv_gemm_mid"):
             return False    # the norm as a kernel of its own and the K-splitting product are faster here
+        if self.prefers_library(M, w.shape[0], K, gated=swiglu):
+            return False    # as are the norm and the library's product
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N):
             return False
         resid_in, delta, resid_out = pending.fused()
@@ -542,6 +557,8 @@ class Ops:
             return False
         M, K = a.shape
         two_i = w_gate_up.shape[0]
+        if self.prefers_library(M, two_i, K, gated=True) and self._library_allowed(M, two_i, K, False):
+            return False
         # with the library's product at hand, more rows than one workgroup takes go there
         if (M > SKINNY_LAUNCH_ROWS or M == 0 or (M > SKINNY_MAX_M and self._library_allowed(M, two_i, K, False))
                 or w_gate_up.dtype != torch.bfloat16 or K % 32 or two_i % 2

@@ -663,7 +663,7 @@ def test_gemm_weight_streaming(out_dtype, M, N, K):
     (17, 3100, 4096, False, torch.bfloat16), (64, 4096, 3072, False, torch.bfloat16),
     (40, 6144, 2048, False, torch.float32), (64, 6144, 2048, True, torch.bfloat16),
     (33, 2 * 1571, 4096, True, torch.bfloat16), (20, 151936 // 4, 1024, False, torch.float32),
-    (9, 3100, 4096, False, torch.bfloat16), (1, 151936 // 4, 4096, False, torch.bfloat16),
+    (9, 3100, 4096, False, torch.bfloat16), (1, 5120, 25600, False, torch.bfloat16),
     (3, 2 * 12032, 5120, True, torch.bfloat16)])
 def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dtype):
     """9 to 64 rows against a weight of tens of megabytes, any number of rows up to 64 against one
