@@ -9,7 +9,9 @@ has them (``model``, ``max_model_len``, ``max_num_batched_tokens``, ``max_num_ba
 * ``kv_cache_num_blocks`` None sizes the cache from free device memory, a number is taken
   as given (the reference treats it as an upper cap, executor.py:46);
 * ``use_cuda_graph`` keeps its name; the decode step is captured in a HIP graph;
-* the executor never writes into this object (the reference's does, executor.py:49).
+* the executor never writes into this object (the reference's does, executor.py:49);
+* ``prefill_chunk``, ``enable_prefix_caching``, ``num_scheduler_steps``, ``launch_ahead`` and ``seed`` have no
+  counterpart there (its scheduler runs whole prompts and one decoded token a step, scheduler.py:26-89).
 """
 from __future__ import annotations
 

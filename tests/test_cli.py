@@ -23,6 +23,8 @@ def test_run_options_map_to_the_engine_config():
     assert (ec.model, ec.max_num_batched_tokens, ec.max_num_batched_seqs) == ("/m", 2048, 128)
     assert ec.gpu_memory_utilization == 0.4 and ec.kv_cache_block_size == 32 and ec.use_cuda_graph is False
     assert ec.prefill_chunk == 256 and ec.enable_prefix_caching is True
+    assert ec.launch_ahead is True
+    assert run.engine_config_from(ap.parse_args(["--model", "/m", "--no-launch-ahead"])).launch_ahead is False
     sp = run.sampling_params_from(args)
     assert (sp.temperature, sp.top_k, sp.top_p, sp.max_tokens, sp.ignore_eos) == (0.5, 7, 0.9, 33, True)
     # the reference's defaults (run.py:12,36)

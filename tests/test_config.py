@@ -102,6 +102,7 @@ def test_engine_config_and_sampling_params():
         EngineConfig(model="x", gpu_memory_utilization=0.0)
     # ours: decode-only steps may run several times in a row on the device
     assert ec.num_scheduler_steps >= 1 and EngineConfig(model="x", num_scheduler_steps=1).num_scheduler_steps == 1
+    assert ec.launch_ahead is True and EngineConfig(model="x", launch_ahead=False).launch_ahead is False
     with pytest.raises(ValueError):
         EngineConfig(model="x", num_scheduler_steps=0)
     sp = SamplingParams()
