@@ -92,12 +92,10 @@ class LLM:
         """One step of the engine: schedule, run the batch, draw tokens, record them."""
         t0 = time.perf_counter()
         run = None
+        self.drain()                                 # a row whose requests have all ended is waited for and forgotten
         if self._in_flight is not None:
             step, run = self._in_flight
             self._in_flight = None
-            if all(r.state == RequestState.FINISHED for r in step.requests):
-                run.tokens()                         # everything it ran for has ended: wait and forget it
-                run = None
         if run is None:
             step = self.scheduler.schedule()
             if step is None:
@@ -126,6 +124,13 @@ class LLM:
         self.metrics.preemptions = self.scheduler.num_preemptions
         step.finished = done
         return step
+
+    def drain(self) -> None:
+        """Waits for decode steps that were launched ahead for requests that have all ended since
+        (their tokens are dropped). ``step()`` does the same when it is called again."""
+        if self._in_flight is not None and all(r.state == RequestState.FINISHED for r in self._in_flight[0].requests):
+            self._in_flight[1].tokens()
+            self._in_flight = None
 
     def _seq_steps(self, step: ScheduledStep, further: int = 0) -> List[SeqStep]:
         """What the executor runs for a scheduled step. ``further``: the step was scheduled ahead of
@@ -219,6 +224,7 @@ class LLM:
                 pbar.update(s.finished_requests - finished_before - pbar.n)
         if pbar is not None:
             pbar.close()
+        self.drain()
         return [self._output(r) for r in sorted(requests, key=lambda r: r.id)]
 
     def _output(self, r: Request) -> RequestOutput:

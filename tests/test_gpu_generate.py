@@ -275,7 +275,7 @@ def test_launching_ahead_gives_the_same_tokens(models, dtype):
             if steps == 7:
                 reqs.append(llm.submit(prompts[5], params[5]))
         assert ahead == (launched > 0)
-        llm.step()                                    # a row that may still be in flight is waited for
+        llm.drain()                                   # a row that may still be in flight is waited for
         assert llm._in_flight is None
         llm.manager.check_invariants()
         assert all(p.num_free == p.num_pages for p in llm.manager.pools)
