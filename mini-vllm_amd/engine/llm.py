@@ -6,7 +6,9 @@ Reference: minivllm/engine/engine.py — ``Engine(config)`` with ``submit`` / ``
 submission, one record per request with the keys ``prompt``, ``completion`` and ``tokens``
 (engine.py:40-90). Those names are kept (``RequestOutput`` also answers to them); prompts may
 also be strings when the model folder holds a tokenizer. ``step`` runs one mixed batch:
-schedule, execute, sample, update.
+schedule, execute, sample, update. A batch of decoded tokens only may run several times in a row
+on the device, and the row after it may be launched while it runs (``EngineConfig.launch_ahead``);
+``step`` still returns one finished step per call, in order.
 """
 from __future__ import annotations
 
