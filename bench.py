@@ -102,12 +102,21 @@ def measure_decode(llm, vocab, batch, prompt_len, steps, warmup, seed):
     reqs = [llm.submit(random_prompt(vocab, prompt_len, seed + i), sp) for i in range(batch)]
     while any(r.num_completion_tokens == 0 for r in reqs):          # prompts in, first token drawn
         llm.step()
+    ahead = llm.config.launch_ahead
+
     def run(n):
         target = min(r.num_completion_tokens for r in reqs) + n
-        while min(r.num_completion_tokens for r in reqs) < target:
-            if llm.step() is None or any(r.finished for r in reqs):
-                raise RuntimeError("a request of the benchmark ended before the timed steps were over; "
-                                   "give it a longer --context")
+        try:
+            while min(r.num_completion_tokens for r in reqs) < target:
+                # the steps that reach the target are not followed by steps launched ahead: the timed
+                # region then holds exactly n steps and nothing runs on when its clock is read
+                to_go = target - min(r.num_completion_tokens for r in reqs)
+                llm.config.launch_ahead = ahead and to_go > llm.config.num_scheduler_steps
+                if llm.step() is None or any(r.finished for r in reqs):
+                    raise RuntimeError("a request of the benchmark ended before the timed steps were over; "
+                                       "give it a longer --context")
+        finally:
+            llm.config.launch_ahead = ahead
     run(warmup)
     torch.cuda.synchronize()
     before = sum(r.num_completion_tokens for r in reqs)
@@ -228,7 +237,8 @@ def main() -> int:
                        "requests": args.requests, "gen_len": args.gen_len, "token_budget": args.token_budget,
                        "max_seqs": live, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max,
                        "seq_len": args.context, "block_size": args.block_size, "graph": not args.no_graph,
-                       "scheduler_steps": args.scheduler_steps, "parallelism": "single-gpu"},
+                       "scheduler_steps": args.scheduler_steps, "launch_ahead": bool(llm.config.launch_ahead),
+                       "parallelism": "single-gpu"},
             "seconds": round(dt, 3), "prompt_tokens": prompt, "generated_tokens": gen,
             "total_tok_s": round((gen + prompt) / dt, 1), "preemptions": preempted}))
         return 0
@@ -267,7 +277,7 @@ def main() -> int:
               "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
               "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch, "seq_len": args.context,
               "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
-              "scheduler_steps": args.scheduler_steps,
+              "scheduler_steps": args.scheduler_steps, "launch_ahead": bool(llm.config.launch_ahead),
               "parallelism": "single-gpu"}
     line = {"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
             "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1, "steps": ran if ran else args.steps, "warmup": args.warmup,
