@@ -116,14 +116,17 @@ class FakeEngine:
             sampled.append(drawn)
         return sampled
 
-    def run_all_launching_ahead(self, limit=100000):
+    def run_all_launching_ahead(self, limit=100000, each_round=None):
         """As an engine that launches the next step of decoded tokens before it has read the
-        tokens of the one that runs. Returns how many steps were scheduled ahead."""
+        tokens of the one that runs. Returns how many steps were scheduled ahead.
+        ``each_round(n)`` is called before round n (to submit requests meanwhile)."""
         ahead_count = n = 0
         in_flight = None                                   # (step, what the device drew)
         while in_flight is not None or not self.sched.finished:
             n += 1
             assert n < limit, "the scheduler does not terminate"
+            if each_round is not None:
+                each_round(n)
             if in_flight is None:
                 step = self.sched.schedule()
                 assert step is not None
@@ -390,3 +393,27 @@ def test_steps_are_scheduled_ahead_when_nothing_can_change():
         e.run_all()
         assert a.completion_tokens == expected_output(a.prompt_tokens, limit)
         assert b.completion_tokens == expected_output(b.prompt_tokens, limit)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_requests_that_arrive_while_a_step_is_in_flight(seed):
+    """New requests come in while a step launched ahead is running: it is read first, then they are
+    admitted; every request still gets the tokens of a run step by step."""
+    rng = random.Random(200 + seed)
+    e = FakeEngine(num_pages=120, page_size=4, max_tokens=24, max_seqs=6, repeat=4)
+    first = [submit(e, [rng.randrange(VOCAB) for _ in range(rng.randrange(2, 20))], max_tokens=rng.randrange(20, 50),
+                    ignore_eos=seed % 2 == 0) for _ in range(2)]
+    late = []
+    arrivals = {4: 1, 5: 2, 9: 1}
+
+    def each_round(n):
+        for _ in range(arrivals.get(n, 0)):
+            late.append(submit(e, [rng.randrange(VOCAB) for _ in range(rng.randrange(1, 25))],
+                               max_tokens=rng.randrange(1, 40), ignore_eos=seed % 2 == 0))
+
+    ahead = e.run_all_launching_ahead(each_round=each_round)
+    assert ahead > 0 and len(late) == 4
+    for r in first + late:
+        assert r.completion_tokens == expected_output(r.prompt_tokens, r.sampling_params.max_tokens,
+                                                      ignore_eos=seed % 2 == 0)
+    assert all(p.num_free == p.num_pages for p in e.manager.pools)
