@@ -19,6 +19,22 @@ from dataclasses import dataclass, field
 from typing import Optional, Tuple
 
 
+COMPUTE_DTYPES = ("bfloat16", "float32")
+
+
+def compute_dtype_name(engine_dtype: Optional[str], model_dtype: Optional[str], where: str = "config.json") -> str:
+    """The precision the engine computes in: the engine option when it is given, else what the
+    model's config.json names. The engine computes in bfloat16 or float32 only; a model that
+    names anything else (float16) is served only when the caller states which of the two to use
+    (the reference takes whatever config.json says, minivllm/executor/executor.py:17)."""
+    from .model_config import ConfigError
+    name = engine_dtype or model_dtype or "bfloat16"
+    if name not in COMPUTE_DTYPES:
+        raise ConfigError(f"{where}: the model names the dtype {name!r}; the engine computes in bfloat16 or float32 "
+                          f"and picks neither silently: state dtype='bfloat16' or dtype='float32' (--dtype)")
+    return name
+
+
 @dataclass
 class EngineConfig:
     # ---- model -------------------------------------------------------------------------

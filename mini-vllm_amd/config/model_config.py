@@ -75,11 +75,14 @@ class ModelConfig:
 class Qwen3Config(ModelConfig):
     """Qwen3 dense decoder (reference: minivllm/models/models/qwen3.py).
 
-    ``sliding_window`` follows the reference's attention layer, whose window is the
-    number of tokens to the left of a query that it may attend to besides itself
-    (minivllm/models/layers/attention.py:56-60, minivllm/models/models/gemma3.py:69).
-    The reference's Qwen3 never passes a window; here ``use_sliding_window`` turns it on
-    for the layers with index >= ``max_window_layers`` and leaves the others full.
+    The reference's Qwen3 never passes a window to its attention layer (qwen3.py:66-71), so
+    there every layer sees all keys whatever ``use_sliding_window`` says. Here the key is
+    honoured with the meaning it has where it comes from: with ``use_sliding_window`` the
+    layers with index >= ``max_window_layers`` see ``sliding_window`` keys, the query's own
+    among them (key position > query position - sliding_window); the other layers see all.
+    No file of the reference pins this: parity unpinned. The attention part counts a window as
+    tokens to the left of the query besides itself (the reference's attention layer,
+    minivllm/models/layers/attention.py:56-60), which is ``sliding_window - 1``.
     """
 
     architecture: ClassVar[str] = "Qwen3ForCausalLM"
@@ -112,9 +115,10 @@ class Qwen3Config(ModelConfig):
         return self.num_key_value_heads * self.head_dim
 
     def layer_window(self, layer: int) -> Optional[int]:
-        """Window (tokens to the left) of ``layer``, or None for full attention."""
+        """How many tokens to the left of a query ``layer`` sees besides the query itself
+        (``sliding_window`` keys in all, the query's own included), or None for all."""
         if self.use_sliding_window and layer >= self.max_window_layers:
-            return self.sliding_window
+            return self.sliding_window - 1
         return None
 
     @classmethod
@@ -159,8 +163,9 @@ class Qwen3Config(ModelConfig):
             if window is None:
                 raise ConfigError(f"{where}: use_sliding_window is true but 'sliding_window' is missing")
             window = _typed(window, "sliding_window", int, where)
-            if window < 0:
-                raise ConfigError(f"{where}: sliding_window must be >= 0, got {window}")
+            if window < 1:
+                raise ConfigError(f"{where}: sliding_window counts the keys a query sees, its own included, "
+                                  f"and must be >= 1, got {window}")
             max_window_layers = layers if max_window_layers is None else _typed(
                 max_window_layers, "max_window_layers", int, where)
         else:

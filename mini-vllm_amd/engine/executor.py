@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, GroupSpec, groups_from_needs
-from ..config.engine_config import EngineConfig
+from ..config.engine_config import EngineConfig, compute_dtype_name
 from ..kernels.ops import dtype_from_name, get_ops
 from ..models.causal_lm import CausalLM, expected_tensors
 from ..models.registry import Architecture, load_config
@@ -102,10 +102,7 @@ class Executor:
             arch, model_config, source = model
             where = "the given tensors"
         self.arch, self.model_config = arch, model_config
-        dtype_name = config.dtype or getattr(model_config, "dtype", "bfloat16")
-        if dtype_name == "float16":
-            dtype_name = "bfloat16"
-        self.dtype = dtype_from_name(dtype_name)
+        self.dtype = dtype_from_name(compute_dtype_name(config.dtype, getattr(model_config, "dtype", None), where))
         self.page_size = config.kv_cache_block_size
 
         plan = arch.plan(model_config)
@@ -114,6 +111,13 @@ class Executor:
                              f"max_position_embeddings {plan.max_positions}")
         check_tensors(source, expected_tensors(arch, model_config, plan), arch.ignorable(model_config), where)
 
+        if self.dtype == torch.bfloat16:
+            wide = [n for n, d in expected_tensors(arch, model_config, plan).items()
+                    if len(d.shape) == 2 and not d.integer and source.stored_type(n) != "BF16"]
+            if wide:
+                logger.warning("%d matrices of %s are stored in 32-bit and stay so: products with them run on the "
+                               "exact kernel, not on the MFMA kernels (first: %s); store the model in bfloat16 for "
+                               "serving speed", len(wide), where, wide[0])
         self.ops = get_ops(self.dtype)
         self.rt = Runtime(device=self.device, dtype=self.dtype, ops=self.ops, workspace=Workspace(self.device),
                           max_positions=config.max_model_len)

@@ -27,6 +27,11 @@ class DeviceRandomSource(TensorSource):
     def is_integer(self, name: str) -> bool:
         return self.expected[name].integer
 
+    def stored_type(self, name: str) -> str:
+        if self.expected[name].integer:
+            return "I32"
+        return {torch.bfloat16: "BF16", torch.float32: "F32"}.get(self.dtype, str(self.dtype))
+
     def read(self, name: str) -> torch.Tensor:
         decl = self.expected[name]
         gen = torch.Generator(device=self.device)

@@ -3,8 +3,9 @@
 Reference: minivllm/models/loader.py:24-29 and qwen3.py:223-245. The reference raises a bare
 ``KeyError`` for an unknown tensor name, does not notice missing tensors and leaves a wrong
 shape to ``copy_``. Here every problem of a folder is found before any data is read and is
-reported in one ``WeightError`` that lists missing tensors, unexpected tensors and wrong
-shapes.
+reported in one ``WeightError`` that lists missing tensors, unexpected tensors, wrong
+shapes, wrong kinds (integer against floating) and stored types the engine does not keep
+(float16, 8-bit floats: it converts nothing silently).
 """
 from __future__ import annotations
 
@@ -13,14 +14,15 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..parts.base import TensorDecl
-from .source import DeviceTensors, SafetensorsSource, TensorSource
+from .source import KEPT_FLOAT_TYPES, DeviceTensors, SafetensorsSource, TensorSource
 
 
 class WeightError(ValueError):
     def __init__(self, where: str, missing: List[str], unexpected: List[str],
                  wrong_shape: List[Tuple[str, Tuple[int, ...], Tuple[int, ...]]],
-                 wrong_type: List[Tuple[str, str]]):
+                 wrong_type: List[Tuple[str, str]], unsupported_dtype: Optional[List[Tuple[str, str]]] = None):
         self.missing, self.unexpected, self.wrong_shape, self.wrong_type = missing, unexpected, wrong_shape, wrong_type
+        self.unsupported_dtype = unsupported_dtype = list(unsupported_dtype or [])
         lines = [f"the weights in {where} do not fit the model:"]
         if missing:
             lines.append(f"  missing tensors ({len(missing)}):")
@@ -34,6 +36,11 @@ class WeightError(ValueError):
         if wrong_type:
             lines.append(f"  wrong kinds ({len(wrong_type)}):")
             lines += [f"    {n}: {why}" for n, why in wrong_type]
+        if unsupported_dtype:
+            kinds = sorted({t for _, t in unsupported_dtype})
+            lines.append(f"  unsupported dtype {', '.join(kinds)} ({len(unsupported_dtype)} tensors; the engine keeps "
+                         f"bfloat16 and float32 as stored and converts nothing else):")
+            lines += [f"    {n}: {t}" for n, t in unsupported_dtype]
         super().__init__("\n".join(lines))
 
 
@@ -42,7 +49,7 @@ def check_tensors(source: TensorSource, expected: Dict[str, TensorDecl], ignorab
     have = set(source.names())
     missing = sorted(n for n in expected if n not in have)
     unexpected = sorted(n for n in have if n not in expected and n not in ignorable)
-    wrong_shape, wrong_type = [], []
+    wrong_shape, wrong_type, unsupported = [], [], []
     for name, decl in expected.items():
         if name not in have:
             continue
@@ -52,8 +59,10 @@ def check_tensors(source: TensorSource, expected: Dict[str, TensorDecl], ignorab
         if source.is_integer(name) != decl.integer:
             wrong_type.append((name, "integer tensor where a floating one is expected" if not decl.integer
                                else "floating tensor where an integer table is expected"))
-    if missing or unexpected or wrong_shape or wrong_type:
-        raise WeightError(where, missing, unexpected, sorted(wrong_shape), sorted(wrong_type))
+        elif not decl.integer and source.stored_type(name) not in KEPT_FLOAT_TYPES:
+            unsupported.append((name, source.stored_type(name)))
+    if missing or unexpected or wrong_shape or wrong_type or unsupported:
+        raise WeightError(where, missing, unexpected, sorted(wrong_shape), sorted(wrong_type), sorted(unsupported))
 
 
 def open_model_folder(model_dir: str) -> TensorSource:

@@ -5,8 +5,10 @@ and yields ``(name, tensor)``; it does not use an index file. Here the files are
 (sorted), their headers give names, shapes and dtypes without reading data, and tensors are
 read one at a time by name.
 
-Storage rule: floating tensors are kept in bfloat16, except that a tensor stored in 32-bit
-(or wider) stays float32; integer tensors become int32.
+Storage rule: a tensor stored in bfloat16 stays bfloat16, one stored in 32-bit (or wider)
+floating point stays float32, integer tensors become int32. Any other stored type (float16,
+8-bit floats) is refused: the engine computes in bfloat16 or float32 and converts nothing
+behind the user's back.
 """
 from __future__ import annotations
 
@@ -30,12 +32,21 @@ class TensorSource:
     def is_integer(self, name: str) -> bool:
         raise NotImplementedError
 
+    def stored_type(self, name: str) -> str:
+        """The stored element type by its safetensors name ("BF16", "F32", "F16", "I64", ...)."""
+        raise NotImplementedError
+
     def read(self, name: str) -> torch.Tensor:
         """The tensor on the CPU, as stored."""
         raise NotImplementedError
 
 
 _INT_DTYPES = {"I8", "I16", "I32", "I64", "U8", "U16", "U32", "U64", "BOOL"}
+# stored floating types the engine keeps (bfloat16 as it is, the wide ones as float32)
+KEPT_FLOAT_TYPES = {"BF16", "F32", "F64"}
+_TORCH_TYPE_NAMES = {torch.bfloat16: "BF16", torch.float32: "F32", torch.float64: "F64", torch.float16: "F16",
+                     torch.int8: "I8", torch.int16: "I16", torch.int32: "I32", torch.int64: "I64",
+                     torch.uint8: "U8", torch.bool: "BOOL"}
 
 
 class SafetensorsSource(TensorSource):
@@ -68,6 +79,9 @@ class SafetensorsSource(TensorSource):
     def is_integer(self, name: str) -> bool:
         return self._dtypes[name].upper() in _INT_DTYPES
 
+    def stored_type(self, name: str) -> str:
+        return self._dtypes[name].upper()
+
     def read(self, name: str) -> torch.Tensor:
         return self._handles[self._where[name]].get_tensor(name)
 
@@ -86,6 +100,10 @@ class DictSource(TensorSource):
         t = self._tensors[name]
         return not (t.is_floating_point() or t.is_complex())
 
+    def stored_type(self, name: str) -> str:
+        dt = self._tensors[name].dtype
+        return _TORCH_TYPE_NAMES.get(dt, str(dt).replace("torch.", "").upper())
+
     def read(self, name: str) -> torch.Tensor:
         return self._tensors[name]
 
@@ -96,7 +114,9 @@ def storage_dtype(t: torch.Tensor) -> torch.dtype:
         return torch.int32
     if t.dtype in (torch.float32, torch.float64):
         return torch.float32
-    return torch.bfloat16
+    if t.dtype == torch.bfloat16:
+        return torch.bfloat16
+    raise TypeError(f"tensors stored as {t.dtype} are not supported (bfloat16 and float32 are)")
 
 
 class DeviceTensors:

@@ -80,11 +80,14 @@ def swiglu_mlp(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w
 
 
 def layer_window(cfg: Dict, layer: int) -> Optional[int]:
-    """Window of a layer from config.json: with ``use_sliding_window`` the layers from
-    ``max_window_layers`` on see ``sliding_window`` tokens to the left (the convention of
-    minivllm/models/layers/attention.py:56-60); the reference's Qwen3 itself never sets one."""
+    """Window of a layer from config.json, as ``causal_attention`` counts it (tokens to the left
+    besides the query, minivllm/models/layers/attention.py:56-60). With ``use_sliding_window`` the
+    layers from ``max_window_layers`` on see ``sliding_window`` keys, the query's own among them
+    (the meaning of the key where it comes from), hence ``sliding_window - 1`` to the left. The
+    reference's Qwen3 never hands a window to its attention (minivllm/models/models/qwen3.py:66-71):
+    no file of the reference pins this rule."""
     if cfg.get("use_sliding_window") and layer >= cfg.get("max_window_layers", cfg["num_hidden_layers"]):
-        return cfg["sliding_window"]
+        return cfg["sliding_window"] - 1
     return None
 
 

@@ -4,7 +4,7 @@ import json
 import pytest
 
 from helpers import TINY_A, TINY_B
-from minivllm_amd.config import ConfigError, EngineConfig, Qwen3Config, SamplingParams
+from minivllm_amd.config import ConfigError, EngineConfig, Qwen3Config, SamplingParams, compute_dtype_name
 from minivllm_amd.models import config_from_dict, get_architecture, load_config, registered_architectures
 
 
@@ -17,7 +17,8 @@ def test_qwen3_keys_are_read():
     assert cfg.attention_bias is True and cfg.tie_word_embeddings is False
     assert cfg.eos_token_ids == (3, 5)
     assert cfg.q_dim == 256 and cfg.kv_dim == 64
-    assert [cfg.layer_window(i) for i in range(3)] == [None, 21, 21]
+    # sliding_window 21 = 21 keys with the query's own: 20 to its left
+    assert [cfg.layer_window(i) for i in range(3)] == [None, 20, 20]
     assert cfg.dtype == "bfloat16"
 
 
@@ -58,6 +59,7 @@ def test_missing_size_is_an_error(key):
     ({"vocab_size": "256"}, "integer"),
     ({"rms_norm_eps": 0.0}, "rms_norm_eps"),
     ({"use_sliding_window": True, "sliding_window": None}, "sliding_window"),
+    ({"use_sliding_window": True, "sliding_window": 0}, "sliding_window"),
     ({"torch_dtype": "int8"}, "dtype"),
 ])
 def test_unsupported_values_are_refused(patch, needle):
@@ -82,7 +84,7 @@ def test_plan_is_data():
     arch, cfg = config_from_dict(dict(TINY_B))
     plan = arch.plan(cfg)
     assert len(plan.layers) == 3 and [c.layer for c in plan.calls] == [0, 1, 2]
-    assert plan.layers[0].mixer.window is None and plan.layers[2].mixer.window == 21
+    assert plan.layers[0].mixer.window is None and plan.layers[2].mixer.window == 20
     assert plan.layers[1].mixer.num_heads == 8 and plan.layers[1].mixer.scale == 32 ** -0.5
     assert plan.layers[1].ffn.intermediate_size == 168
     assert plan.head.tied is False and plan.final_norm.eps == 1e-5
@@ -111,3 +113,15 @@ def test_engine_config_and_sampling_params():
     for bad in (dict(temperature=-1.0), dict(max_tokens=0), dict(top_k=-1), dict(top_p=0.0), dict(top_p=1.5)):
         with pytest.raises(ValueError):
             SamplingParams(**bad)
+
+
+def test_float16_models_need_a_stated_dtype():
+    """config.json may name float16; the engine computes in bfloat16 or float32 and picks neither
+    silently (the reference computes in whatever config.json names, executor.py:17)."""
+    _, cfg = config_from_dict({**TINY_A, "torch_dtype": "float16"})
+    assert cfg.dtype == "float16"
+    with pytest.raises(ConfigError, match="float16.*state dtype"):
+        compute_dtype_name(None, cfg.dtype, "m/config.json")
+    assert compute_dtype_name("float32", cfg.dtype) == "float32"
+    assert compute_dtype_name("bfloat16", cfg.dtype) == "bfloat16"
+    assert compute_dtype_name(None, "float32") == "float32" and compute_dtype_name(None, None) == "bfloat16"

@@ -131,7 +131,7 @@ def test_attention_part_and_block(dtype, layer):
     mixer_cls = MIXERS.get(spec.kind)
     mixer = mixer_cls(spec, tensors("mixer", mixer_cls.tensors(spec)), rt, position=rope)
     need = mixer_cls.cache_need(spec)
-    assert need.retention == ("full" if layer == 0 else "window") and need.window == (None if layer == 0 else 21)
+    assert need.retention == ("full" if layer == 0 else "window") and need.window == (None if layer == 0 else 20)
 
     g = torch.Generator().manual_seed(2)
     lens = [50, 44]

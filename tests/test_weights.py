@@ -62,11 +62,12 @@ def test_untied_model_needs_its_head(tmp_path):
 
 def test_kept_dtypes():
     assert storage_dtype(torch.zeros(1, dtype=torch.bfloat16)) == torch.bfloat16
-    assert storage_dtype(torch.zeros(1, dtype=torch.float16)) == torch.bfloat16
+    with pytest.raises(TypeError, match="float16"):                                  # never converted silently
+        storage_dtype(torch.zeros(1, dtype=torch.float16))
     assert storage_dtype(torch.zeros(1, dtype=torch.float32)) == torch.float32      # 32-bit stays 32-bit
     assert storage_dtype(torch.zeros(1, dtype=torch.float64)) == torch.float32
     assert storage_dtype(torch.zeros(1, dtype=torch.int64)) == torch.int32           # integer tables
-    src = DictSource({"a": torch.ones(3, dtype=torch.float16), "b": torch.ones(3), "c": torch.arange(3)})
+    src = DictSource({"a": torch.ones(3, dtype=torch.bfloat16), "b": torch.ones(3), "c": torch.arange(3)})
     dev = DeviceTensors(src, torch.device("cpu"))
     assert dev.get("a").dtype == torch.bfloat16 and dev.get("b").dtype == torch.float32
     assert dev.get("c").dtype == torch.int32
@@ -94,3 +95,25 @@ def test_random_model_folder(tmp_path, raw, stored):
     d3 = write_model_folder(str(tmp_path / "rand3"), cfg, seed=4, dtype=stored)
     assert torch.equal(open_model_folder(d2).read("model.norm.weight"), src.read("model.norm.weight"))
     assert not torch.equal(open_model_folder(d3).read("model.norm.weight"), src.read("model.norm.weight"))
+
+
+def test_float16_tensors_are_refused_not_converted(tmp_path):
+    """A tensor stored in float16 is named in the one error; nothing is converted silently."""
+    w = make_weights(TINY_A, 0, stored=torch.bfloat16)
+    w["model.layers.1.mlp.down_proj.weight"] = w["model.layers.1.mlp.down_proj.weight"].to(torch.float16)
+    w["model.norm.weight"] = w["model.norm.weight"].to(torch.float16)
+    del w["model.layers.0.mlp.up_proj.weight"]
+    d = write_model_dir(str(tmp_path / "m"), TINY_A, w)
+    arch, cfg = load_config(d)
+    with pytest.raises(WeightError) as ei:
+        check_tensors(open_model_folder(d), expected_tensors(arch, cfg), arch.ignorable(cfg), d)
+    e = ei.value
+    assert e.unsupported_dtype == [("model.layers.1.mlp.down_proj.weight", "F16"), ("model.norm.weight", "F16")]
+    assert e.missing == ["model.layers.0.mlp.up_proj.weight"]
+    assert "unsupported dtype F16 (2 tensors" in str(e)
+    with pytest.raises(TypeError, match="float16"):
+        storage_dtype(torch.zeros(2, dtype=torch.float16))
+    # the same through a dictionary of tensors
+    with pytest.raises(WeightError, match="unsupported dtype F16"):
+        check_tensors(DictSource({**make_weights(TINY_A, 0), "model.norm.weight": torch.ones(64, dtype=torch.float16)}),
+                      expected_tensors(arch, cfg), arch.ignorable(cfg))
