@@ -36,7 +36,31 @@ TINY_C = {
     "rope_theta": 50000.0, "rms_norm_eps": 3e-6, "tie_word_embeddings": False, "attention_bias": False,
     "hidden_act": "silu", "torch_dtype": "bfloat16", "eos_token_id": 1,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# The second tiny configuration exactly as the benchmark description states it: no bias and no
+# window, so every layer keeps all keys and prefix reuse can be on (cache pages of 8, portions of 7).
+TINY_B0 = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 3, "hidden_size": 96, "num_attention_heads": 8, "num_key_value_heads": 2,
+    "head_dim": 32, "intermediate_size": 160, "vocab_size": 384, "max_position_embeddings": 2048,
+    "rope_theta": 1000000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "attention_bias": False,
+    "hidden_act": "silu", "torch_dtype": "float32", "eos_token_id": 2,
+}
+# Head sizes the MFMA attention kernels serve (128 and 64), widths the MFMA products serve.
+TINY_D128 = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 2, "hidden_size": 256, "num_attention_heads": 4, "num_key_value_heads": 2,
+    "head_dim": 128, "intermediate_size": 512, "vocab_size": 1000, "max_position_embeddings": 4096,
+    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "attention_bias": False,
+    "hidden_act": "silu", "torch_dtype": "bfloat16", "eos_token_id": 0,
+}
+TINY_D64 = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 3, "hidden_size": 192, "num_attention_heads": 6, "num_key_value_heads": 1,
+    "head_dim": 64, "intermediate_size": 320, "vocab_size": 777, "max_position_embeddings": 4096,
+    "rope_theta": 50000.0, "rms_norm_eps": 2e-6, "tie_word_embeddings": False, "attention_bias": True,
+    "hidden_act": "silu", "torch_dtype": "bfloat16", "eos_token_id": 0,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "B0": TINY_B0, "D128": TINY_D128, "D64": TINY_D64}
 
 
 def tensor_shapes(cfg: Dict) -> Dict[str, tuple]:

@@ -119,3 +119,4 @@ def collect(steps: List[dict], run_step: Callable[[dict], Optional[np.ndarray]])
         for rid in st["end"]:
             pos.pop(rid, None)
     return out
+
