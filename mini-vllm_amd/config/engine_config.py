@@ -10,7 +10,7 @@ has them (``model``, ``max_model_len``, ``max_num_batched_tokens``, ``max_num_ba
   as given (the reference treats it as an upper cap, executor.py:46);
 * ``use_cuda_graph`` keeps its name; the decode step is captured in a HIP graph;
 * the executor never writes into this object (the reference's does, executor.py:49);
-* ``prefill_chunk``, ``enable_prefix_caching``, ``num_scheduler_steps``, ``launch_ahead`` and ``seed`` have no
+* ``prefill_chunk``, ``enable_prefix_caching``, ``num_scheduler_steps``, ``launch_ahead``, ``seed`` have no
   counterpart there (its scheduler runs whole prompts and one decoded token a step, scheduler.py:26-89).
 """
 from __future__ import annotations
@@ -70,6 +70,10 @@ class EngineConfig:
     # nothing but an end-of-sequence token could change what it holds (what ran on for a request
     # that ended is dropped)
     launch_ahead: bool = True
+    # record every decode graph the configuration can ask for when the engine starts (the
+    # reference does, minivllm/executor/graph.py:24-58) instead of at a graph's first use, which
+    # makes that step wait for the recording
+    capture_graphs_at_start: bool = False
     seed: int = 0
 
     def __post_init__(self) -> None:

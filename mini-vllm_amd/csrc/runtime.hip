@@ -1,5 +1,6 @@
 // Host-side support of the C entry points: the error channel and a few queries.
 #include "common.h"
+#include <stdlib.h>
 #include <string.h>
 
 static thread_local char g_error[512] = "";
@@ -33,3 +34,36 @@ extern "C" int mv_built_dtypes() {
 }
 
 extern "C" int mv_abi_version() { return 1; }
+
+// What a captured graph holds, by kind of node: out[0] kernels, out[1] memsets, out[2] copies,
+// out[3] anything else. The engine admits no memset node in a graph it replays (such nodes have
+// given wrong results on replays after the first); a library call that records one is found here.
+extern "C" int mv_graph_census(void* graph, int* out) {
+    MV_REQUIRE(graph != nullptr && out != nullptr, "mv_graph_census: null argument");
+    size_t n = 0;
+    hipError_t e = hipGraphGetNodes((hipGraph_t)graph, nullptr, &n);
+    if (e != hipSuccess) return mv_fail("mv_graph_census: hipGraphGetNodes: %s", hipGetErrorString(e));
+    out[0] = out[1] = out[2] = out[3] = 0;
+    if (n == 0) return 0;
+    hipGraphNode_t* nodes = (hipGraphNode_t*)malloc(n * sizeof(hipGraphNode_t));
+    MV_REQUIRE(nodes != nullptr, "mv_graph_census: out of host memory");
+    e = hipGraphGetNodes((hipGraph_t)graph, nodes, &n);
+    if (e != hipSuccess) {
+        free(nodes);
+        return mv_fail("mv_graph_census: hipGraphGetNodes: %s", hipGetErrorString(e));
+    }
+    for (size_t i = 0; i < n; ++i) {
+        hipGraphNodeType t;
+        e = hipGraphNodeGetType(nodes[i], &t);
+        if (e != hipSuccess) {
+            free(nodes);
+            return mv_fail("mv_graph_census: hipGraphNodeGetType: %s", hipGetErrorString(e));
+        }
+        if (t == hipGraphNodeTypeKernel) out[0]++;
+        else if (t == hipGraphNodeTypeMemset) out[1]++;
+        else if (t == hipGraphNodeTypeMemcpy) out[2]++;
+        else out[3]++;
+    }
+    free(nodes);
+    return 0;
+}

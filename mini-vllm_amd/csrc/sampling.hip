@@ -128,11 +128,32 @@ sample_partial_kernel(const float* __restrict__ logits, long ld, int V, const fl
     }
 }
 
+// What a row's drawn token is written to. Besides the output, a decode step that runs again at
+// once on the device takes the token as its next input: ``next_ids[row]`` receives it, the row's
+// position and context length move on by one and its random stream's counter by one. Null
+// pointers leave all that out.
+struct Advance {
+    int* next_ids;
+    int* positions;
+    int* context_lens;
+    unsigned long long* rng;
+};
+
+__device__ __forceinline__ void deliver(int row, int token, int* out, const Advance& adv) {
+    out[row] = token;
+    if (adv.next_ids != nullptr) {
+        adv.next_ids[row] = token;
+        adv.positions[row] += 1;
+        adv.context_lens[row] += 1;
+        if (adv.rng != nullptr) adv.rng[2 * (size_t)row + 1] += 1;
+    }
+}
+
 __global__ void __launch_bounds__(SP_THREADS)
 sample_kernel(const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
               const int* __restrict__ top_k, const float* __restrict__ top_p,
-              const unsigned long long* __restrict__ rng, int* __restrict__ out,
-              const Best* __restrict__ partial, int chunks) {
+              const unsigned long long* rng, int* __restrict__ out,
+              const Best* __restrict__ partial, int chunks, Advance adv) {
     __shared__ Best shb[17];
     __shared__ float scratch[17];
     __shared__ int hcount[256];
@@ -151,14 +172,14 @@ sample_kernel(const float* __restrict__ logits, long ld, int V, const float* __r
         Best b{-INFINITY, NEG_I};
         for (int c = tid; c < chunks; c += SP_THREADS) b = better(b, partial[(size_t)row * chunks + c]);
         b = block_argmax(b, shb);
-        if (tid == 0) out[row] = b.i;
+        if (tid == 0) deliver(row, b.i, out, adv);
         return;
     }
     if (!(T > 0.f)) {
         Best b{-INFINITY, NEG_I};
         for (int i = tid; i < V; i += SP_THREADS) b = better(b, Best{x[i], i});
         b = block_argmax(b, shb);
-        if (tid == 0) out[row] = b.i;
+        if (tid == 0) deliver(row, b.i, out, adv);
         return;
     }
 
@@ -252,17 +273,17 @@ sample_kernel(const float* __restrict__ logits, long ld, int V, const float* __r
         const float g = -logf(-logf(u));
         best = better(best, Best{z + g, i});
     }
-    best = block_argmax(best, shb);
-    if (tid == 0) out[row] = best.i;
+    best = block_argmax(best, shb);        // (its barriers lie between every lane's read of the counter and the write)
+    if (tid == 0) deliver(row, best.i, out, adv);
 }
 
 // temperature, top_k, top_p: per row, or null for 0 / off / off. rng: [M][2] = (seed, counter).
 // work: 8 * M * chunks bytes of scratch, or null. With it, rows that need no threshold (greedy
 // rows, and drawn rows without top-k and top-p) are served by two short launches in which
 // `chunks` workgroups share a row; the drawn token is the same either way.
-extern "C" int mv_sample(const float* logits, long ld, int M, int V, const float* temperature, const int* top_k,
+static int sample_launch(const float* logits, long ld, int M, int V, const float* temperature, const int* top_k,
                          const float* top_p, const unsigned long long* rng, int* out, void* work, int chunks,
-                         hipStream_t stream) {
+                         Advance adv, hipStream_t stream) {
     MV_REQUIRE(M >= 0 && V > 0 && ld >= V, "sample: bad sizes M=%d V=%d ld=%ld", M, V, ld);
     MV_REQUIRE(temperature == nullptr || rng != nullptr, "sample: temperatures given without random keys");
     MV_REQUIRE(work == nullptr || (chunks >= 1 && chunks <= 65535), "sample: bad chunk count %d", chunks);
@@ -273,6 +294,25 @@ extern "C" int mv_sample(const float* logits, long ld, int M, int V, const float
         if (int rc = mv_check_launch("sample (first pass)")) return rc;
     }
     hipLaunchKernelGGL(sample_kernel, dim3(M), dim3(SP_THREADS), 0, stream, logits, ld, V, temperature, top_k,
-                       top_p, rng, out, (const Best*)work, chunks);
+                       top_p, rng, out, (const Best*)work, chunks, adv);
     return mv_check_launch("sample");
+}
+
+extern "C" int mv_sample(const float* logits, long ld, int M, int V, const float* temperature, const int* top_k,
+                         const float* top_p, const unsigned long long* rng, int* out, void* work, int chunks,
+                         hipStream_t stream) {
+    return sample_launch(logits, ld, M, V, temperature, top_k, top_p, rng, out, work, chunks,
+                         Advance{nullptr, nullptr, nullptr, nullptr}, stream);
+}
+
+// The same, for a decode step that runs again on the device with the drawn tokens: row m's token also
+// goes to next_ids[m], positions[m] and context_lens[m] move on by one, and so does the counter of
+// the row's random stream (rng is written here).
+extern "C" int mv_sample_advance(const float* logits, long ld, int M, int V, const float* temperature,
+                                 const int* top_k, const float* top_p, unsigned long long* rng, int* out, void* work,
+                                 int chunks, int* next_ids, int* positions, int* context_lens, hipStream_t stream) {
+    MV_REQUIRE(next_ids != nullptr && positions != nullptr && context_lens != nullptr,
+               "sample_advance: the next step's token ids, positions and context lengths are needed");
+    return sample_launch(logits, ld, M, V, temperature, top_k, top_p, rng, out, work, chunks,
+                         Advance{next_ids, positions, context_lens, rng}, stream);
 }

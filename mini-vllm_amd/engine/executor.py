@@ -145,6 +145,8 @@ class Executor:
         self._graph_pool = None
         self._repeat_graphs: Dict[Tuple[int, int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
         self._graph_workspace: Optional[Workspace] = None
+        # what each recorded graph holds, by kind of node (see _record)
+        self.graph_census: Dict[Tuple, Dict[str, int]] = {}
         # pinned buffers for the tokens of launches in flight, used in turn (two launches at most are)
         self._token_buffers: List[Optional[torch.Tensor]] = [None] * 4
         self._next_token_buffer = 0
@@ -186,6 +188,8 @@ class Executor:
         self._allocate_pages(num_pages)
         logger.info("allocated %d cache pages of %d tokens (%.2f GiB)", num_pages, self.page_size,
                     num_pages * self.bytes_per_page() / 2 ** 30)
+        if cfg.capture_graphs_at_start and cfg.use_cuda_graph and self.model.graph_safe:
+            self.capture_graphs()
 
     def _allocate_pages(self, num_pages: int) -> None:
         self.kv_pages.clear()
@@ -205,7 +209,8 @@ class Executor:
         buffer reaches its final size before the cache is sized from what is left."""
         ps = self.page_size
         n_seqs = max(1, min(self.config.max_num_batched_seqs, _cdiv(num_tokens, ps)))
-        per_seq = max(1, num_tokens // n_seqs)
+        # (no step holds more tokens of a request than max_model_len)
+        per_seq = max(1, min(num_tokens // n_seqs, self.config.max_model_len))
         pages_per_seq = _cdiv(per_seq, ps)
         self._allocate_pages(n_seqs * pages_per_seq)
         seqs = []
@@ -214,6 +219,9 @@ class Executor:
             seqs.append(SeqStep(tokens=[0] * per_seq, start=0, block_tables=[table] * len(self.groups),
                                 state_slot=s % self.num_state_slots, want=[per_seq - 1]))
         self.step(seqs)
+        if self.config.use_cuda_graph and self.model.graph_safe:
+            # the scratch area that all decode graphs share, at the size of the largest batch they serve
+            self._prepare_graph_workspace()
         torch.cuda.synchronize()
         self.kv_pages.clear()
         torch.cuda.empty_cache()
@@ -253,7 +261,7 @@ class Executor:
                                      f"{s.start + n - 1} needs {last_page + 1}")
 
     def _fill(self, seqs: Sequence[SeqStep], pad_to: Optional[int] = None, bt_widths: Optional[List[int]] = None,
-              lookahead: int = 0, extra_words: int = 0):
+              lookahead: int = 0, extra_words: int = 0, check_pages: bool = True):
         """Packs the step's integers into one int32 array. Returns (array, offsets dict, facts).
         ``lookahead`` extends the check of the block tables to positions that later runs of a
         repeated step touch; ``extra_words`` leaves room at the end (offset "extra", 8-byte aligned)."""
@@ -330,7 +338,7 @@ class Executor:
             idx = np.arange(w, dtype=np.int64)[None, :]
             touched = (idx >= (first_pos // self.page_size)[:, None]) & (idx <= last_page[:, None])
             ids = bt[:S][touched]
-            if ids.size and (ids.min() < 0 or ids.max() >= self.num_pages):
+            if check_pages and ids.size and (ids.min() < 0 or ids.max() >= self.num_pages):
                 raise ValueError(f"cache group {g}: a block table names a page outside the pool of "
                                  f"{self.num_pages} (or one that was given back) where the step reads or writes")
         if N and (tok[:N].min() < 0 or tok[:N].max() >= self.vocab_size):
@@ -549,17 +557,16 @@ class Executor:
             self.ops.sample(logits[:bucket], tokens[0], temps, top_k, top_p, rng)
             torch.cuda.synchronize()
             self._graph_workspace.frozen = True
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
+            advance = (ctx.token_ids, ctx.positions, ctx.context_lens)
+
+            def body():
                 for j in range(repeat):
                     logits = self.model.forward(ctx)
-                    self.ops.sample(logits[:bucket], tokens[j], temps, top_k, top_p, rng)
-                    if j + 1 < repeat:             # the next run: the drawn tokens, one position on
-                        ctx.token_ids.copy_(tokens[j])
-                        ctx.positions.add_(1)
-                        ctx.context_lens.add_(1)
-                        rng[:, 1].add_(1)
-            self._graph_pool = graph.pool()
+                    # the sampler feeds the next run itself: the drawn tokens, one position on
+                    self.ops.sample(logits[:bucket], tokens[j], temps, top_k, top_p, rng,
+                                    advance=advance if j + 1 < repeat else None)
+
+            graph = self._record(body, key)
         finally:
             self._graph_workspace.frozen = False
             self.rt.workspace = eager_workspace
@@ -584,22 +591,109 @@ class Executor:
         self._upload(arr, dst=meta)
         return self._context(meta, off, facts, dummy)
 
+    def _prepare_graph_workspace(self) -> None:
+        """One scratch area for all graphs, sized by a step of padding rows at the largest batch the
+        graphs serve; should a later graph need a larger buffer, the old one stays alive for the
+        graphs that hold it."""
+        if self._graph_workspace is not None:
+            return
+        eager_workspace, was_for_graph = self.rt.workspace, self.ops.for_graph
+        self.ops.for_graph = True
+        try:
+            self._graph_workspace = Workspace(self.device, retain=True)
+            self.rt.workspace = self._graph_workspace
+            largest = next(b for b in GRAPH_BUCKETS if b >= min(self.config.max_num_batched_seqs, GRAPH_BUCKETS[-1]))
+            pad_ctx = self._padding_step(largest)
+            pad_ctx.attention_plan.max_context_len = self.config.max_model_len
+            self.model.forward(pad_ctx)
+            torch.cuda.synchronize()
+        finally:
+            self.rt.workspace = eager_workspace
+            self.ops.for_graph = was_for_graph
+
+    def _record(self, body, key) -> torch.cuda.CUDAGraph:
+        """Records ``body`` into a graph and looks at what was recorded: a graph with a memset node
+        is not kept (such nodes have replayed wrongly on this platform; the engine's own kernels
+        record none, a library product might). It is recorded again with the engine's own products
+        only, and must be clean then."""
+        for library in (True, False):
+            self.ops.library_in_graphs = library
+            try:
+                graph = torch.cuda.CUDAGraph(keep_graph=True)
+                with torch.cuda.graph(graph, pool=self._graph_pool):
+                    body()
+            finally:
+                self.ops.library_in_graphs = True
+            census = self.ops.graph_census(graph.raw_cuda_graph())
+            self.graph_census[key] = census
+            if census["memset"] == 0:
+                graph.instantiate()
+                self._graph_pool = graph.pool()
+                return graph
+            logger.warning("the decode graph %s holds %d memset nodes%s", key, census["memset"],
+                           "; recording it again without library products" if library else "")
+            del graph
+        raise RuntimeError(f"the decode graph {key} holds memset nodes although only the engine's kernels ran")
+
+    def capture_graphs(self) -> int:
+        """Records, ahead of serving, every decode graph the configuration can ask for: batch-size
+        buckets up to ``max_num_batched_seqs``, context caps up to ``max_model_len``, single steps
+        and rows of 2 to ``num_scheduler_steps`` (the reference records its buckets when the engine
+        starts, minivllm/executor/graph.py:24-58). Otherwise a graph is recorded at its first use,
+        which makes that step wait. Returns the number of graphs recorded."""
+        caps, cap = [], 1024
+        while True:
+            caps.append(min(cap, max(self.config.max_model_len, 1)))
+            if cap >= self.config.max_model_len:
+                break
+            cap *= 2
+        limit = min(self.config.max_num_batched_seqs, GRAPH_BUCKETS[-1], self.num_state_slots)
+        buckets = [b for b in GRAPH_BUCKETS if b <= limit]
+        if limit not in buckets:
+            buckets.append(next(b for b in GRAPH_BUCKETS if b >= limit))
+        k = self.config.num_scheduler_steps
+        made = 0
+        tables = [[0]] * len(self.groups)
+        for bucket in sorted(set(buckets), reverse=True):       # the largest first: it sizes the scratch area
+            n = min(bucket, limit)
+            for cap in sorted(set(caps)):
+                # stand-in sequences whose context reaches the cap; the recorded launches depend on the
+                # sizes only, never on these values
+                start = max(0, min(cap, self.config.max_model_len) - max(k, 1))
+                seqs = [SeqStep(tokens=[0], start=start, block_tables=tables, state_slot=i % self.num_state_slots,
+                                want=[0]) for i in range(n)]
+                widths = [self.max_pages_per_seq] * len(self.groups)
+                if (bucket, cap) not in self._graphs:
+                    arr, off, facts = self._fill(seqs, pad_to=bucket, bt_widths=widths, check_pages=False)
+                    self._as_padding(arr, off)
+                    self._capture(bucket, cap, arr, off, facts, seqs)
+                    made += 1
+                for repeat in range(2, k + 1):          # a row is shorter when a request nears its last token
+                    if (bucket, cap, repeat) in self._repeat_graphs:
+                        continue
+                    arr, off, facts = self._fill(seqs, pad_to=bucket, bt_widths=widths, extra_words=7 * bucket,
+                                                 check_pages=False)
+                    self._as_padding(arr, off)
+                    self._capture_repeated((bucket, cap, repeat), arr, off, facts, seqs)
+                    made += 1
+        logger.info("recorded %d decode graphs ahead of serving", made)
+        return made
+
+    @staticmethod
+    def _as_padding(arr: np.ndarray, off) -> None:
+        """Turns the rows of a packed step into padding rows: every kernel runs, none touches the cache."""
+        for name, value in (("token_seq", -1), ("logit_rows", -1), ("cu_seqlens", 0), ("context_lens", 0)):
+            o, size = off[name]
+            arr[o:o + size] = value
+        o, size = off["positions"]
+        arr[o:o + size] = 0
+
     def _capture(self, bucket: int, cap: int, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
         logger.info("capturing the decode graph for %d sequences, contexts up to %d", bucket, cap)
         eager_workspace = self.rt.workspace
-        self.ops.for_graph = True                  # library products only where a rehearsal allows them
+        self.ops.for_graph = True
         try:
-            if self._graph_workspace is None:
-                # one scratch area for all graphs, sized for the largest bucket; should a later
-                # graph need a larger buffer, the old one stays alive for the graphs that hold it
-                self._graph_workspace = Workspace(self.device, retain=True)
-                self.rt.workspace = self._graph_workspace
-                largest = next(b for b in GRAPH_BUCKETS
-                               if b >= min(self.config.max_num_batched_seqs, GRAPH_BUCKETS[-1]))
-                pad_ctx = self._padding_step(largest)
-                pad_ctx.attention_plan.max_context_len = self.config.max_model_len
-                self.model.forward(pad_ctx)
-                torch.cuda.synchronize()
+            self._prepare_graph_workspace()
             self.rt.workspace = self._graph_workspace
             meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
             self._upload(arr, dst=meta)
@@ -609,10 +703,9 @@ class Executor:
             self.model.forward(ctx)                # loads every kernel before the capture
             torch.cuda.synchronize()
             self._graph_workspace.frozen = True    # the eager run above sized everything: nothing is allocated now
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                logits = self.model.forward(ctx)
-            self._graph_pool = graph.pool()
+            result = []
+            graph = self._record(lambda: result.append(self.model.forward(ctx)), (bucket, cap))
+            logits = result[-1]
         finally:
             self._graph_workspace.frozen = False
             self.rt.workspace = eager_workspace

@@ -24,6 +24,7 @@ _SIGNATURES = {
     "mv_last_error": (ctypes.c_char_p, []),
     "mv_built_dtypes": (c_int, []),
     "mv_abi_version": (c_int, []),
+    "mv_graph_census": (c_int, [c_void_p, c_void_p]),
     "mv_embedding": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "mv_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
                                c_int, c_int, c_int, c_void_p]),
@@ -44,6 +45,9 @@ _SIGNATURES = {
                                  c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
     "mv_sample": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_int, c_void_p]),
+    # ... as mv_sample up to chunks, then next_ids, positions, context_lens, stream
+    "mv_sample_advance": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
 }
 
 # entry points that only the bfloat16 library has

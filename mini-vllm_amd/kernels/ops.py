@@ -117,10 +117,10 @@ class Ops:
         self.lib = library.load(library.variant_of(_NAMES[dtype]))
         self.use_fast_kernels = dtype == torch.bfloat16
         self.use_library_gemm = dtype == torch.bfloat16
-        # set by the executor while it rehearses and captures a graph: the library's product then
-        # runs only for shapes that passed a rehearsal of their own (see _library_allowed)
+        # set by the executor while it records a graph; library products take part in a recording
+        # while ``library_in_graphs`` holds (see _library_allowed)
         self.for_graph = False
-        self._library_in_graph: dict = {}
+        self.library_in_graphs = True
         self.stream_handle: Optional[int] = None
         self._transposed = {}
         self._mid_work: Optional[torch.Tensor] = None
@@ -414,60 +414,18 @@ class Ops:
         return True
 
     def _library_allowed(self, M: int, N: int, K: int, with_bias: bool, out_dtype: torch.dtype = torch.bfloat16) -> bool:
-        """Whether the library's matrix product may serve this shape now. Outside graphs: whenever it
-        is switched on. For a graph: only when a graph holding just this product, replayed several
-        times with other work and synchronisations in between, gave the eager result every time
-        (a library may record nodes that do not replay faithfully). The rehearsal happens in the
-        eager run that precedes every capture; a shape that was never rehearsed stays with the
-        engine's own kernels."""
-        if not self.use_library_gemm:
-            return False
-        if not self.for_graph:
-            return True
-        key = (M, N, K, with_bias) if out_dtype == torch.bfloat16 else (M, N, K, with_bias, out_dtype)
-        ok = self._library_in_graph.get(key)
-        if ok is None:
-            if torch.cuda.is_current_stream_capturing():
-                return False
-            ok = self._library_in_graph[key] = self._rehearse_library_product(M, N, K, with_bias, out_dtype)
-        return ok
+        """Whether the library's matrix product may serve this shape now: whenever it is switched
+        on, and while a graph is being recorded only as long as ``library_in_graphs`` holds. The
+        executor looks at every graph it has recorded (``graph_census``) and records it again
+        without library products should one of them have left a memset node in it."""
+        return self.use_library_gemm and (self.library_in_graphs or not self.for_graph)
 
-    def _rehearse_library_product(self, M: int, N: int, K: int, with_bias: bool,
-                                  out_dtype: torch.dtype = torch.bfloat16) -> bool:
-        dev = torch.device("cuda", torch.cuda.current_device())
-        a = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
-        w = torch.randn(N, K, device=dev, dtype=torch.bfloat16) * 0.05
-        bias = torch.randn(N, device=dev, dtype=torch.bfloat16) if with_bias else None
-        out = torch.empty(M, N, device=dev, dtype=out_dtype)
-
-        def product(dst):
-            if not self._library_product(a, w, bias, dst):
-                raise RuntimeError("the library has no algorithm for the shape")
-
-        bound = self.stream_handle
-        self.stream_handle = None                          # the rehearsal runs on torch's current stream
-        try:
-            product(out)                                   # loads the kernel, makes the library's handles
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                product(out)
-            ok = True
-            want = torch.empty_like(out)
-            for _ in range(3):
-                a.normal_()                                # eager work between the replays
-                out.fill_(float("nan"))
-                torch.cuda.synchronize()
-                graph.replay()
-                torch.cuda.synchronize()
-                product(want)
-                ok = ok and bool(torch.equal(out, want))
-            del graph
-            return ok
-        except RuntimeError:
-            return False
-        finally:
-            self.stream_handle = bound
+    def graph_census(self, raw_graph: int) -> dict:
+        """Nodes of a recorded graph by kind: {"kernel", "memset", "copy", "other"}."""
+        import ctypes
+        counts = (ctypes.c_int * 4)()
+        self.lib.call("mv_graph_census", raw_graph, ctypes.addressof(counts))
+        return dict(kernel=counts[0], memset=counts[1], copy=counts[2], other=counts[3])
 
     def _gemm_mid(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   ldc: int, M: int, N: int, K: int, swiglu: bool, defer_sum: bool = False):
@@ -737,11 +695,15 @@ class Ops:
     # ------------------------------------------------------------------------------------
     def sample(self, logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
                top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
-               rng: Optional[torch.Tensor] = None) -> None:
+               rng: Optional[torch.Tensor] = None, advance: Optional[tuple] = None) -> None:
         """One token id per row of float32 ``logits`` into int32 ``out``.
 
         temperature float32 [M] (None or 0: arg-max), top_k int32 [M], top_p float32 [M],
-        rng int64 [M, 2] = (seed, counter) of each row's random stream."""
+        rng int64 [M, 2] = (seed, counter) of each row's random stream.
+
+        ``advance`` = (token_ids, positions, context_lens), int32 [>= M] each, makes the kernel
+        prepare the same step's next run on the device: row m's token also goes to token_ids[m],
+        positions[m] and context_lens[m] grow by one and so does the counter in ``rng``."""
         _dev(logits, "logits"); _dev(out, "sampled ids")
         if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
             raise KernelLibraryError("sample: logits must be float32 [M, V] with a contiguous last dimension")
@@ -768,6 +730,16 @@ class Ops:
                 self._sample_work = torch.empty(SAMPLE_WORK_ROWS * SAMPLE_CHUNKS * 2, dtype=torch.int32,
                                                 device=logits.device)
             work = self._sample_work
+        if advance is not None:
+            for t, what in zip(advance, ("next token ids", "positions", "context lengths")):
+                _dev(t, what)
+                if t.dtype != torch.int32 or t.numel() < M or not t.is_contiguous():
+                    raise KernelLibraryError(f"sample: {what} must be contiguous int32 with at least M elements")
+            self.lib.call("mv_sample_advance", logits.data_ptr(), logits.stride(0) if M > 1 else V, M, V,
+                          _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(rng), out.data_ptr(), _ptr(work),
+                          SAMPLE_CHUNKS, advance[0].data_ptr(), advance[1].data_ptr(), advance[2].data_ptr(),
+                          self._stream())
+            return
         self.lib.call("mv_sample", logits.data_ptr(), logits.stride(0) if M > 1 else V, M, V, _ptr(temperature),
                       _ptr(top_k), _ptr(top_p), _ptr(rng), out.data_ptr(), _ptr(work), SAMPLE_CHUNKS, self._stream())
 

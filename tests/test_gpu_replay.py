@@ -18,15 +18,27 @@ from helpers import (TINY, TOL_F32, bf16_tolerance, make_weights, plain_logits, 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-STORED = {"A": torch.float32, "B": torch.bfloat16, "C": torch.bfloat16}
-LENGTHS = {"A": [70, 5, 33, 17, 1 + 32, 49], "B": [91, 40, 66, 2, 58, 35], "C": [50, 36, 77]}
+STORED = {"A": torch.float32, "B": torch.bfloat16, "C": torch.bfloat16, "D128": torch.bfloat16, "D64": torch.bfloat16}
+LENGTHS = {"A": [70, 5, 33, 17, 1 + 32, 49], "B": [91, 40, 66, 2, 58, 35], "C": [50, 36, 77],
+           "D128": [70, 5, 133, 17, 49], "D64": [91, 40, 66, 2, 158]}
+# D128 and D64 have the head sizes the MFMA attention kernels serve (on pages of 16 and 32) and widths
+# the MFMA products serve: in bfloat16 every cutting below runs the serving kernels with them
+PAGE = {"A": 16, "B": 16, "C": 16, "D128": 16, "D64": 32}
+NAMES = ["A", "B", "C", "D128", "D64"]
+# sharp: the q/k norm weights are scaled so that attention is peaked and one lost or wrong key shows;
+# rounding is amplified with it, so the bfloat16 bound of these cases is wide. mild: the same case with
+# the weights as drawn, where the bfloat16 bound is at most 2e-2 and a small systematic error shows.
+GAINS = {"sharp": 2.5, "mild": 1.0}
+MILD_BF16_BOUND = 2e-2
 
 
 class Case:
-    def __init__(self, name, tmp, qk_gain=1.0):
+    def __init__(self, name, tmp, qk_gain=1.0, kind="sharp"):
+        self.name, self.kind = name, kind
         self.cfg = TINY[name]
+        self.page = PAGE[name]
         self.weights = make_weights(self.cfg, seed=sum(map(ord, name)), stored=STORED[name], qk_gain=qk_gain)
-        self.dir = write_model_dir(str(tmp / f"tiny{name}"), self.cfg, self.weights)
+        self.dir = write_model_dir(str(tmp / f"tiny{name}_{kind}"), self.cfg, self.weights)
         self.reqs = {f"r{i}": random_tokens(self.cfg, n, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
         self.want = {rid: plain_logits(self.cfg, self.weights, toks) for rid, toks in self.reqs.items()}
         emulated = {rid: plain_logits_bf16(self.cfg, self.weights, toks) for rid, toks in self.reqs.items()}
@@ -34,7 +46,10 @@ class Case:
                               for rid, toks in self.reqs.items() for p in range(len(toks)))
 
     def tol(self, dtype):
-        return TOL_F32 if dtype == "float32" else bf16_tolerance(self.bf16_error)
+        if dtype == "float32":
+            return TOL_F32
+        bound = bf16_tolerance(self.bf16_error)
+        return min(bound, MILD_BF16_BOUND) if self.kind == "mild" else bound
 
     def check(self, got, dtype, what):
         worst = 0.0
@@ -49,65 +64,72 @@ class Case:
 @pytest.fixture(scope="module")
 def cases(tmp_path_factory):
     tmp = tmp_path_factory.mktemp("models")
-    return {name: Case(name, tmp, qk_gain=2.5) for name in ("A", "B", "C")}
+    return {(name, kind): Case(name, tmp, qk_gain=gain, kind=kind) for name in NAMES for kind, gain in GAINS.items()}
 
 
-def runner_for(case, dtype, steps, page_size=16, use_graph=True, slack=0):
+def runner_for(case, dtype, steps, page_size=None, use_graph=True, slack=0):
     from minivllm_amd.engine.trace import TraceRunner
-    return TraceRunner(case.dir, dtype, trace_tools.max_live_tokens(steps) + slack, page_size=page_size,
+    return TraceRunner(case.dir, dtype, trace_tools.max_live_tokens(steps) + slack, page_size=page_size or case.page,
                        use_graph=use_graph)
 
 
+def both(cases, name):
+    """The sharp and the mild copy of a configuration."""
+    return [cases[(name, kind)] for kind in GAINS]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", NAMES)
 def test_whole(cases, name, dtype):
-    case = cases[name]
-    steps = trace_tools.whole(case.reqs)
-    got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
-    assert len(got) == case.check(got, dtype, f"tiny {name} whole")
+    for case in both(cases, name):
+        steps = trace_tools.whole(case.reqs)
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+        assert len(got) == case.check(got, dtype, f"tiny {name} {case.kind} whole")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", NAMES)
 @pytest.mark.parametrize("use_graph", [True, False])
 def test_tail_decode(cases, name, dtype, use_graph):
-    case = cases[name]
-    steps = trace_tools.tail_decode(case.reqs, tail=32)
-    got = trace_tools.collect(steps, runner_for(case, dtype, steps, use_graph=use_graph).run_step)
-    case.check(got, dtype, f"tiny {name} last 32 one by one (graph={use_graph})")
-    for rid, toks in case.reqs.items():
-        assert (rid, len(toks) - 1) in got
+    for case in both(cases, name):
+        steps = trace_tools.tail_decode(case.reqs, tail=32)
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps, use_graph=use_graph).run_step)
+        case.check(got, dtype, f"tiny {name} {case.kind} last 32 one by one (graph={use_graph})")
+        for rid, toks in case.reqs.items():
+            assert (rid, len(toks) - 1) in got
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
-@pytest.mark.parametrize("page_size", [16, 4])
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("page_size", ["own", 4])
 def test_portions(cases, name, dtype, page_size):
-    case = cases[name]
-    steps = trace_tools.portions(case.reqs)
-    got = trace_tools.collect(steps, runner_for(case, dtype, steps, page_size=page_size).run_step)
-    assert len(got) == case.check(got, dtype, f"tiny {name} portions (page {page_size})")
+    """(pages of 4 slots send the head sizes 64 and 128 to the general attention kernel)"""
+    for case in both(cases, name):
+        steps = trace_tools.portions(case.reqs)
+        ps = case.page if page_size == "own" else page_size
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps, page_size=ps).run_step)
+        assert len(got) == case.check(got, dtype, f"tiny {name} {case.kind} portions (page {ps})")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", NAMES)
 def test_mixed(cases, name, dtype):
-    case = cases[name]
-    prompt_lens = {rid: max(2, len(t) - 12) if len(t) > 3 else len(t) for rid, t in case.reqs.items()}
-    for seed in (0, 1):
-        steps = trace_tools.mixed(case.reqs, prompt_lens, max_live=4 if name != "C" else 2, seed=seed)
-        runner = runner_for(case, dtype, steps)
-        got = trace_tools.collect(steps, runner.run_step)
-        assert len(got) == case.check(got, dtype, f"tiny {name} mixed seed {seed}")
-        runner.manager.check_invariants()
-        assert not runner.manager.seqs                       # everything was given back
-        for pool in runner.manager.pools:
-            assert pool.num_free == pool.num_pages
+    for case in both(cases, name):
+        prompt_lens = {rid: max(2, len(t) - 12) if len(t) > 3 else len(t) for rid, t in case.reqs.items()}
+        for seed in (0, 1):
+            steps = trace_tools.mixed(case.reqs, prompt_lens, max_live=4 if name != "C" else 2, seed=seed)
+            runner = runner_for(case, dtype, steps)
+            got = trace_tools.collect(steps, runner.run_step)
+            assert len(got) == case.check(got, dtype, f"tiny {name} {case.kind} mixed seed {seed}")
+            runner.manager.check_invariants()
+            assert not runner.manager.seqs                       # everything was given back
+            for pool in runner.manager.pools:
+                assert pool.num_free == pool.num_pages
 
 
 def test_first_tokens_and_single_token_requests(cases):
     """The first positions of a sequence, and requests of one and two tokens."""
-    case = cases["A"]
+    case = cases[("A", "sharp")]
     reqs = {"one": case.reqs["r0"][:1], "two": case.reqs["r0"][:2], "three": case.reqs["r1"][:3]}
     steps = trace_tools.whole(reqs)
     for dtype in ("float32", "bfloat16"):
@@ -119,7 +141,7 @@ def test_first_tokens_and_single_token_requests(cases):
 
 def test_long_decoding(cases):
     """One token after another from the very first, 300 of them, across many pages."""
-    case = cases["B"]
+    case = cases[("B", "sharp")]
     toks = random_tokens(case.cfg, 300, seed=77)
     want = plain_logits(case.cfg, case.weights, toks)
     emulated = plain_logits_bf16(case.cfg, case.weights, toks)
@@ -167,7 +189,7 @@ def test_contexts_beyond_a_thousand_tokens(tmp_path, head_dim, page_size):
 
 def test_trace_run_program(cases, tmp_path):
     """bin/trace_run as a user calls it: steps on standard input, logits in files."""
-    case = cases["A"]
+    case = cases[("A", "sharp")]
     prompt_lens = {rid: max(2, len(t) - 6) for rid, t in case.reqs.items()}
     steps = trace_tools.mixed(case.reqs, prompt_lens, max_live=3, seed=5)
     for dtype in ("float32", "bfloat16"):
@@ -193,8 +215,9 @@ def test_trace_run_program(cases, tmp_path):
 
 def test_layer_sizes_of_the_0_6b_shape(tmp_path):
     """The layer sizes of Qwen3-0.6B (hidden 1024, 16/8 heads of 128, intermediate 3072, vocabulary
-    151936, tied head, theta 1e6) with four layers: portions, decoded tokens and a second request
-    on recycled pages, in float32 and bfloat16, against the plain model. This is the shape the
+    151936, tied head, theta 1e6) with four layers, in all four cuttings (whole, the last 32 tokens
+    one by one, portions down to two tokens, mixed with a second request on recycled pages), in
+    float32 and bfloat16, against the plain model. This is the shape the
     MFMA kernels are tuned for (head size 128, K = 1024/2048/3072)."""
     cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 4, "hidden_size": 1024,
            "num_attention_heads": 16, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 3072,
@@ -208,14 +231,18 @@ def test_layer_sizes_of_the_0_6b_shape(tmp_path):
     emulated = {r: plain_logits_bf16(cfg, w64, t) for r, t in reqs.items()}
     del w64
     bf16_err = max(rel_err(emulated[r][p], want[r][p]) for r, t in reqs.items() for p in range(len(t)))
-    steps = trace_tools.mixed(reqs, {"p": 70, "q": 33}, max_live=2, seed=3, max_portion=40)
+    cuttings = {"whole": trace_tools.whole(reqs), "last 32 one by one": trace_tools.tail_decode(reqs, tail=32),
+                "portions": trace_tools.portions(reqs, sizes=(7, 40, 2, 17, 3, 29)),
+                "mixed": trace_tools.mixed(reqs, {"p": 70, "q": 33}, max_live=2, seed=3, max_portion=40)}
     from minivllm_amd.engine.trace import TraceRunner
     for dtype in ("float32", "bfloat16"):
-        runner = TraceRunner(path, dtype, trace_tools.max_live_tokens(steps), page_size=16)
-        got = trace_tools.collect(steps, runner.run_step)
-        worst = max(rel_err(row, want[rid][pos]) for (rid, pos), row in got.items())
         tol = TOL_F32 if dtype == "float32" else bf16_tolerance(bf16_err)
-        print(f"0.6B layer sizes [{dtype}]: {len(got)} rows, worst relative error {worst:.3e} (allowed {tol:.3e})")
-        assert len(got) == 123 and worst <= tol
-        del runner
-        torch.cuda.empty_cache()
+        for what, steps in cuttings.items():
+            runner = TraceRunner(path, dtype, trace_tools.max_live_tokens(steps), page_size=16)
+            got = trace_tools.collect(steps, runner.run_step)
+            worst = max(rel_err(row, want[rid][pos]) for (rid, pos), row in got.items())
+            print(f"0.6B layer sizes, {what} [{dtype}]: {len(got)} rows, worst relative error {worst:.3e} "
+                  f"(allowed {tol:.3e})")
+            assert len(got) == (123 if what != "last 32 one by one" else 66) and worst <= tol
+            del runner
+            torch.cuda.empty_cache()
