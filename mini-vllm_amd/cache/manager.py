@@ -6,14 +6,16 @@ allocates a whole prompt at once (block_manager.py:54-87) or one page per decode
 (block_manager.py:89-98). Here
 
 * calls (layer executions) whose mixers need the same retention form a *group*; each group has
-  its own pool and each request one block table per group. A "full" group keeps every position;
-  a "window" group gives a page back as soon as every position in it lies more than ``window``
-  tokens behind the next query;
+  its own pool and each request one block table per group. How long a group keeps a position is
+  its ``Retention`` object's business (``parts.base``): the manager asks it only for the first page
+  a request still needs (``KeepAll`` keeps every position; ``KeepWindow`` gives a page back as soon
+  as every position in it lies more than ``window`` tokens behind the next query; a mixer with
+  another rule brings its own class);
 * pages are reserved for the portion of tokens about to run (``reserve``), and the request's
   progress is recorded after the step (``commit``), which also publishes pages that became full
   for prefix reuse and returns pages a window has passed;
 * prefix reuse (``enable_prefix_caching``) is offered when every group keeps all positions
-  and no call carries state, and never covers the whole prompt: at least one token is left to
+  (``Retention.keeps_everything``) and no call carries state, and never covers the whole prompt: at least one token is left to
   compute (in the reference a full hit leaves no query at all);
 * a request holds one state slot from ``admit`` to ``release``.
 
@@ -26,6 +28,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 
+from ..parts.base import Retention
 from .page_pool import OutOfPages, PagePool, page_hash
 from .state_slots import OutOfSlots, StateSlots
 
@@ -33,26 +36,26 @@ from .state_slots import OutOfSlots, StateSlots
 @dataclass(frozen=True)
 class GroupSpec:
     """One cache group: the calls it serves and how long it keeps a position."""
-    retention: str                    # "full" | "window"
-    window: Optional[int]             # tokens to the left of a query that stay visible
+    retention: Retention
     calls: Tuple[int, ...]
 
     def __post_init__(self):
-        if self.retention not in ("full", "window"):
-            raise ValueError(f"unknown retention {self.retention!r}")
-        if self.retention == "window" and (self.window is None or self.window < 0):
-            raise ValueError("a window group needs a window >= 0")
+        if not isinstance(self.retention, Retention):
+            raise TypeError(f"a cache group's retention must be a Retention object, got {self.retention!r}")
 
 
 def groups_from_needs(needs: Sequence[Optional[object]]) -> List[GroupSpec]:
     """Groups the calls by what their mixers need (``CacheNeed.group_key()``); calls without a
     need are in no group."""
     keyed: Dict[Tuple, List[int]] = {}
+    rules: Dict[Tuple, Retention] = {}
     for call, need in enumerate(needs):
         if need is None:
             continue
-        keyed.setdefault(need.group_key(), []).append(call)
-    return [GroupSpec(retention=k[0], window=k[1], calls=tuple(v)) for k, v in keyed.items()]
+        key = need.group_key()
+        keyed.setdefault(key, []).append(call)
+        rules.setdefault(key, need.retention)
+    return [GroupSpec(retention=rules[k], calls=tuple(v)) for k, v in keyed.items()]
 
 
 @dataclass
@@ -106,7 +109,7 @@ class CacheManager:
         self.slots = StateSlots(num_state_slots)
         self.seqs: Dict[Hashable, SequenceCache] = {}
         self.prefix_caching = bool(enable_prefix_caching and self.groups and not has_state
-                                   and all(g.retention == "full" for g in self.groups))
+                                   and all(g.retention.keeps_everything for g in self.groups))
 
     # ---- queries ----------------------------------------------------------------------------
     def __contains__(self, req) -> bool:
@@ -121,11 +124,7 @@ class CacheManager:
     def _first_kept_page(self, g: int, next_position: int) -> int:
         """Index of the first page group ``g`` still needs when the next query stands at
         ``next_position``."""
-        spec = self.groups[g]
-        if spec.retention == "full":
-            return 0
-        lo = max(0, next_position - spec.window)
-        return lo // self.page_size
+        return self.groups[g].retention.first_kept_page(next_position, self.page_size)
 
     def pages_needed(self, req, num_new_tokens: int) -> List[int]:
         """Per group, how many pages must be allocated so that ``num_new_tokens`` more positions
@@ -222,7 +221,7 @@ class CacheManager:
                 seq.hashes.append(h)
         seq.num_computed = new_len
         for g, spec in enumerate(self.groups):
-            if spec.retention != "window":
+            if spec.retention.keeps_everything:
                 continue
             first = min(self._first_kept_page(g, new_len), len(seq.pages[g]))
             pages = seq.pages[g]

@@ -7,9 +7,10 @@ allocation :31-60, input building :81-163, forward :197-214) and minivllm/execut
 * ``step`` takes any mix of prompt portions and decoded tokens and returns float32 logits at
   the wanted positions; sampling is a separate call (the reference returns token ids only);
 * step inputs are packed into one pinned buffer and copied with one transfer;
-* the cache is a pair of page tensors per call, K as [page][kv_head][slot][d] and V as
-  [page][kv_head][d][slot], grouped by retention; the reference holds one
-  [2, layers, blocks, block_size, kv_heads, head_dim] tensor (executor.py:51);
+* the cache is a set of page tensors per call, with the shapes the call's mixer asks for (softmax
+  attention: K as [page][kv_head][slot][d] and V as [page][kv_head][d][slot]), grouped by
+  retention; the reference holds one [2, layers, blocks, block_size, kv_heads, head_dim] tensor
+  (executor.py:51);
 * decode-only steps are replayed from a HIP graph captured per batch-size bucket on first use;
   the block-table width of a graph is ceil(max_model_len / page_size), not the pool size
   (graph.py:20);
@@ -150,7 +151,7 @@ class Executor:
         # pinned buffers for the tokens of launches in flight, used in turn (two launches at most are)
         self._token_buffers: List[Optional[torch.Tensor]] = [None] * 4
         self._next_token_buffer = 0
-        self.kv_pages: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+        self.kv_pages: Dict[int, Dict[str, torch.Tensor]] = {}     # per call with a cache need: its page tensors by name
         self.state_tensors: Dict[int, torch.Tensor] = {}
         self.num_pages = 0
         self._allocate_memory()
@@ -197,10 +198,8 @@ class Executor:
         for call, need in enumerate(self.needs):
             if need is None:
                 continue
-            k_shape, v_shape = need.page_shapes(self.page_size)
-            k = torch.zeros((num_pages,) + k_shape, dtype=self.dtype, device=self.device)
-            v = torch.zeros((num_pages,) + v_shape, dtype=self.dtype, device=self.device)
-            self.kv_pages[call] = (k, v)
+            self.kv_pages[call] = {name: torch.zeros((num_pages,) + tuple(shape), dtype=self.dtype, device=self.device)
+                                   for name, shape in need.page_shapes(self.page_size).items()}
         self._graphs.clear()
         self._repeat_graphs.clear()
 
@@ -334,9 +333,9 @@ class Executor:
                 bt[i, :len(t)] = t
             # every page a kernel may touch must be a page of the pool
             spec = self.groups[g]
-            first_pos = np.zeros(S, dtype=np.int64) if spec.retention == "full" else np.maximum(0, starts - spec.window)
+            first_page = spec.retention.first_kept_pages(starts, self.page_size)
             idx = np.arange(w, dtype=np.int64)[None, :]
-            touched = (idx >= (first_pos // self.page_size)[:, None]) & (idx <= last_page[:, None])
+            touched = (idx >= first_page[:, None]) & (idx <= last_page[:, None])
             ids = bt[:S][touched]
             if check_pages and ids.size and (ids.min() < 0 or ids.max() >= self.num_pages):
                 raise ValueError(f"cache group {g}: a block table names a page outside the pool of "
@@ -374,8 +373,8 @@ class Executor:
             g = self.group_of_call.get(call)
             if g is not None:
                 owner = self.plan.calls[call].cache_from
-                k, v = self.kv_pages[call if owner is None else owner]
-                ctx._kv[call] = KVView(k, v, ctx.block_tables[g], self.page_size)
+                ctx._kv[call] = KVView(self.kv_pages[call if owner is None else owner], ctx.block_tables[g],
+                                       self.page_size)
             if call in self.state_tensors:
                 ctx._state[call] = self.state_tensors[call]
         return ctx
@@ -404,11 +403,7 @@ class Executor:
         if not seqs:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         self._validate(seqs)
-        if self.has_state:
-            for s in seqs:
-                if s.start == 0:
-                    for t in self.state_tensors.values():
-                        t[s.state_slot].zero_()
+        self._zero_new_states(seqs)
         S = len(seqs)
         decode_only = all(len(s.tokens) == 1 for s in seqs)
         if (self.config.use_cuda_graph and self.model.graph_safe and decode_only and S <= GRAPH_BUCKETS[-1]
@@ -418,6 +413,17 @@ class Executor:
         meta = self._upload(arr)
         ctx = self._context(meta, off, facts, seqs)
         return self.model.forward(ctx)
+
+    def _zero_new_states(self, seqs: Sequence[SeqStep]) -> None:
+        """A request that starts at position 0 starts from a cleared state: one indexed fill per
+        state tensor, whatever the number of such requests."""
+        if not self.has_state:
+            return
+        fresh = [s.state_slot for s in seqs if s.start == 0]
+        if fresh:
+            index = torch.tensor(fresh, dtype=torch.int64, device=self.device)
+            for t in self.state_tensors.values():
+                t.index_fill_(0, index, 0)
 
     def _context_cap(self, seqs: Sequence[SeqStep]) -> int:
         """The context length a decode graph is planned for: the next power of two (at least
@@ -488,11 +494,7 @@ class Executor:
         if not self.can_repeat(S) or repeat < 1 or any(len(s.tokens) != 1 or list(s.want) != [0] for s in seqs):
             raise ValueError("a repeated step takes graph-sized batches of single tokens, each wanted")
         self._validate(seqs, lookahead=repeat - 1)
-        if self.has_state:
-            for s in seqs:
-                if s.start == 0:
-                    for t in self.state_tensors.values():
-                        t[s.state_slot].zero_()
+        self._zero_new_states(seqs)
         bucket = next(b for b in GRAPH_BUCKETS if b >= S)
         cap = self._repeat_cap(seqs, repeat)
         if after is not None and (after.bucket != bucket or after.count != S):

@@ -96,11 +96,10 @@ class Scheduler:
                              f"{self.max_model_len} leaves no room to generate")
         longest = min(total, self.max_model_len)
         for g, spec in enumerate(self.manager.groups):
-            if spec.retention == "full":
-                pages = -(-longest // self.manager.page_size)
-                if pages > self.manager.pools[g].num_pages:
-                    raise ValueError(f"the request may reach {longest} tokens = {pages} cache pages, the pool "
-                                     f"has {self.manager.pools[g].num_pages}")
+            pages = spec.retention.most_pages(longest, self.manager.page_size)
+            if pages is not None and pages > self.manager.pools[g].num_pages:
+                raise ValueError(f"the request may reach {longest} tokens = {pages} cache pages, the pool "
+                                 f"has {self.manager.pools[g].num_pages}")
         self.waiting.append(req)
 
     def _computed(self, req: Request) -> int:

@@ -36,11 +36,19 @@ class SeqStep:
 
 @dataclass
 class KVView:
-    """Cache of one call as its mixer sees it."""
-    k_pages: torch.Tensor          # [pages, kv_heads, page_size, head_dim]
-    v_pages: torch.Tensor          # [pages, kv_heads, head_dim, page_size]
+    """Cache of one call as its mixer sees it: the page tensors its ``CacheNeed`` named
+    (``[pages, *page shape]`` each), the block table of its group and the page size."""
+    pages: Dict[str, torch.Tensor]
     block_table: torch.Tensor      # int32 [sequences, width] of the call's group
     page_size: int
+
+    @property
+    def k_pages(self) -> torch.Tensor:      # softmax attention: [pages, kv_heads, page_size, head_dim]
+        return self.pages["k"]
+
+    @property
+    def v_pages(self) -> torch.Tensor:      # [pages, kv_heads, head_dim, page_size]
+        return self.pages["v"]
 
 
 @dataclass

@@ -476,10 +476,11 @@ class Ops:
         """add + RMSNorm + product (or gated pair) in one kernel; False if the shape is not taken
         (nothing has been done then)."""
         M, K = pending.shape
-        norm = pending.norm
-        weight = getattr(norm, "weight", None)
-        spec = getattr(norm, "spec", None)
-        if (weight is None or spec is None or getattr(spec, "kind", "") != "rmsnorm" or not self.can_fuse_norm(M, K)
+        form = pending.norm.as_scaled_rms()     # None: the norm computes something the fused kernel does not
+        if form is None:
+            return False
+        weight, eps, unit_offset = form
+        if (not self.can_fuse_norm(M, K) or weight.numel() != K or not weight.is_contiguous()
                 or weight.data_ptr() % 16
                 or w.dtype != torch.bfloat16 or not w.is_contiguous() or w.shape[1] != K
                 or out.stride(1) != 1 or (swiglu and (w.shape[0] % 2 or out.dtype != torch.bfloat16))):
@@ -497,7 +498,7 @@ class Ops:
         if isinstance(delta, SplitSum):
             delta = delta.materialize()
         self.lib.call("mv_gemm_skinny_norm", resid_in.data_ptr(), _ptr(delta), _ptr(resid_out), weight.data_ptr(),
-                      _weight_code(weight, "norm weight"), float(spec.eps), int(spec.unit_offset), w.data_ptr(),
+                      _weight_code(weight, "norm weight"), float(eps), int(unit_offset), w.data_ptr(),
                       _ptr(bias), out.data_ptr(), out.stride(0) if M > 1 else N, _CODES[out.dtype], M, N, K,
                       int(swiglu), self._stream())
         return True

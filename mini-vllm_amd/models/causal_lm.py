@@ -14,18 +14,20 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from ..parts.base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, HiddenStream,
-                          Runtime, TensorDecl)
+from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed,
+                          HiddenStream, Runtime, TensorDecl)
 from ..parts.plan import ModelPlan, TensorLocation
 from .registry import Architecture
 
 
 def _model_level_decls(plan: ModelPlan) -> List[Tuple[TensorLocation, TensorDecl]]:
-    out = [(TensorLocation(None, "embedding", "weight"),
-            TensorDecl((plan.embedding.vocab_size, plan.embedding.hidden_size)))]
+    out = []
+    for name, decl in EMBEDDINGS.get(plan.embedding.kind).tensors(plan.embedding).items():
+        out.append((TensorLocation(None, "embedding", name), decl))
     for name, decl in NORMS.get(plan.final_norm.kind).tensors(plan.final_norm).items():
         out.append((TensorLocation(None, "final_norm", name), decl))
-    out.append((TensorLocation(None, "head", "weight"), TensorDecl((plan.head.vocab_size, plan.head.hidden_size))))
+    for name, decl in HEADS.get(plan.head.kind).tensors(plan.head).items():
+        out.append((TensorLocation(None, "head", name), decl))
     return out
 
 
@@ -41,10 +43,12 @@ def plan_tensors(plan: ModelPlan) -> List[Tuple[TensorLocation, TensorDecl]]:
         for slot, nspec in layer.norms:
             for name, decl in NORMS.get(nspec.kind).tensors(nspec).items():
                 out.append((TensorLocation(i, f"norm.{slot}", name), decl))
-        for name, decl in MIXERS.get(layer.mixer.kind).tensors(layer.mixer).items():
-            out.append((TensorLocation(i, "mixer", name), decl))
-        for name, decl in FEED_FORWARDS.get(layer.ffn.kind).tensors(layer.ffn).items():
-            out.append((TensorLocation(i, "ffn", name), decl))
+        if layer.mixer is not None:
+            for name, decl in MIXERS.get(layer.mixer.kind).tensors(layer.mixer).items():
+                out.append((TensorLocation(i, "mixer", name), decl))
+        if layer.ffn is not None:
+            for name, decl in FEED_FORWARDS.get(layer.ffn.kind).tensors(layer.ffn).items():
+                out.append((TensorLocation(i, "ffn", name), decl))
     # a position encoding is shared by every mixer that names the same spec: its tensors (a learned
     # table, say) belong to the model, under the role "position.<kind>"
     seen = set()
@@ -80,11 +84,12 @@ class CausalLM:
         def fetch(layer: Optional[int], role: str, decls: Dict[str, TensorDecl]) -> Dict[str, torch.Tensor]:
             return {name: source.get(arch.tensor_name(config, TensorLocation(layer, role, name))) for name in decls}
 
-        self.embedding_table = fetch(None, "embedding", {"weight": None})["weight"]
-        self.embedding_scale = plan.embedding.scale
+        emb_cls = EMBEDDINGS.get(plan.embedding.kind)
+        self.embedding = emb_cls(plan.embedding, fetch(None, "embedding", emb_cls.tensors(plan.embedding)), rt)
         norm_cls = NORMS.get(plan.final_norm.kind)
         self.final_norm = norm_cls(plan.final_norm, fetch(None, "final_norm", norm_cls.tensors(plan.final_norm)), rt)
-        self.head_weight = fetch(None, "head", {"weight": None})["weight"]
+        head_cls = HEADS.get(plan.head.kind)
+        self.head = head_cls(plan.head, fetch(None, "head", head_cls.tensors(plan.head)), rt)
 
         position_parts: Dict[object, object] = {}
         self.graph_safe = True          # every part allows its forward to be captured in a graph
@@ -95,7 +100,6 @@ class CausalLM:
             for slot, nspec in layer.norms:
                 cls = NORMS.get(nspec.kind)
                 norms[slot] = cls(nspec, fetch(i, f"norm.{slot}", cls.tensors(nspec)), rt)
-            mixer_cls = MIXERS.get(layer.mixer.kind)
             kwargs = {}
             pspec = getattr(layer.mixer, "position", None)
             if pspec is not None:
@@ -103,13 +107,19 @@ class CausalLM:
                     pcls = POSITION_ENCODINGS.get(pspec.kind)
                     position_parts[pspec] = pcls(pspec, fetch(None, f"position.{pspec.kind}", pcls.tensors(pspec)), rt)
                 kwargs["position"] = position_parts[pspec]
-            mixer = mixer_cls(layer.mixer, fetch(i, "mixer", mixer_cls.tensors(layer.mixer)), rt, **kwargs)
-            ffn_cls = FEED_FORWARDS.get(layer.ffn.kind)
-            ffn = ffn_cls(layer.ffn, fetch(i, "ffn", ffn_cls.tensors(layer.ffn)), rt)
+            mixer = ffn = None
+            if layer.mixer is not None:
+                mixer_cls = MIXERS.get(layer.mixer.kind)
+                mixer = mixer_cls(layer.mixer, fetch(i, "mixer", mixer_cls.tensors(layer.mixer)), rt, **kwargs)
+            if layer.ffn is not None:
+                ffn_cls = FEED_FORWARDS.get(layer.ffn.kind)
+                ffn = ffn_cls(layer.ffn, fetch(i, "ffn", ffn_cls.tensors(layer.ffn)), rt)
             self.mixers.append(mixer)
             self.blocks.append(BLOCKS.get(layer.block.kind)(layer.block, norms, mixer, ffn))
             parts = [mixer, ffn, kwargs.get("position")] + list(norms.values())
             self.graph_safe = self.graph_safe and all(getattr(p, "graph_safe", True) for p in parts if p is not None)
+        self.graph_safe = self.graph_safe and all(getattr(p, "graph_safe", True)
+                                                  for p in (self.embedding, self.final_norm, self.head))
 
     # ------------------------------------------------------------------------------------
     def cache_needs(self) -> List[Optional[CacheNeed]]:
@@ -118,7 +128,7 @@ class CausalLM:
         needs: List[Optional[CacheNeed]] = []
         for call in self.plan.calls:
             spec = self.plan.layers[call.layer].mixer
-            need = MIXERS.get(spec.kind).cache_need(spec)
+            need = None if spec is None else MIXERS.get(spec.kind).cache_need(spec)
             if call.cache_from is not None:
                 if need is not None:
                     raise ValueError(f"a call reads the cache of call {call.cache_from} but its mixer "
@@ -131,7 +141,7 @@ class CausalLM:
         out = []
         for call in self.plan.calls:
             spec = self.plan.layers[call.layer].mixer
-            out.append(MIXERS.get(spec.kind).state_shape(spec))
+            out.append(None if spec is None else MIXERS.get(spec.kind).state_shape(spec))
         return out
 
     # ------------------------------------------------------------------------------------
@@ -148,21 +158,19 @@ class CausalLM:
         rt, plan = self.rt, self.plan
         n = ctx.n_tokens
         resid = rt.workspace.get("resid", (n, plan.hidden_size), torch.float32)
-        rt.ops.embedding(ctx.token_ids, self.embedding_table, resid, self.embedding_scale)
+        self.embedding.forward(ctx, resid)
         stream = HiddenStream(resid, rt.workspace.get("resid.spare", (n, plan.hidden_size), torch.float32))
         for call_index, call in enumerate(plan.calls):
             self.blocks[call.layer].forward(stream, ctx, call_index)
         m = ctx.n_logit_rows
-        logits = rt.workspace.get("logits", (m, plan.vocab_size), torch.float32)
         if m == 0:
             discard = getattr(stream.delta, "discard", None)
             if discard is not None:
                 discard()
-            return logits
+            return rt.workspace.get("logits", (0, plan.vocab_size), torch.float32)
         h = self.final_norm.forward(stream, ctx, rows=ctx.logit_rows, tag="final_normed")
         # the stream ends here: a last delta that was left as partial sums is not needed again
         discard = getattr(stream.delta, "discard", None)
         if discard is not None:
             discard()
-        rt.ops.gemm(h, self.head_weight, logits)
-        return logits
+        return self.head.forward(h, ctx)

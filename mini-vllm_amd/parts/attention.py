@@ -16,7 +16,8 @@ from typing import Dict, Optional, Tuple
 
 import torch
 
-from .base import (CacheNeed, Mixer, PartSpec, POSITION_ENCODINGS, Runtime, TensorDecl, register_mixer)
+from .base import (CacheNeed, KeepAll, KeepWindow, KeyValueNeed, Mixer, PartSpec, POSITION_ENCODINGS, Runtime,
+                   TensorDecl, register_mixer)
 
 
 @dataclass(frozen=True)
@@ -70,8 +71,8 @@ class Attention(Mixer):
     def cache_need(cls, spec: AttentionSpec) -> Optional[CacheNeed]:
         if spec.shares_kv:
             return None
-        return CacheNeed(retention="full" if spec.window is None else "window", window=spec.window,
-                         num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim)
+        return KeyValueNeed(retention=KeepAll() if spec.window is None else KeepWindow(spec.window),
+                            num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim)
 
     def __init__(self, spec: AttentionSpec, tensors: Dict[str, torch.Tensor], rt: Runtime,
                  position: Optional[object] = None):

@@ -16,7 +16,8 @@ Mixers additionally state what memory they need per request: ``cache_need(spec)`
 of keys and values, ``state_shape(spec)`` for a fixed-size state.
 
 New kinds are added with ``register_mixer`` / ``register_feed_forward`` / ``register_norm`` /
-``register_position_encoding`` / ``register_block``; nothing else in the engine changes.
+``register_position_encoding`` / ``register_block`` / ``register_embedding`` / ``register_head``;
+nothing else in the engine changes.
 """
 from __future__ import annotations
 
@@ -43,26 +44,103 @@ class PartSpec:
     kind: ClassVar[str] = ""
 
 
-@dataclass(frozen=True)
-class CacheNeed:
-    """Paged memory a mixer needs for each token of a request.
+class Retention:
+    """How long a cache group keeps a position of a request. The cache manager and the executor ask
+    only these questions of it, so a mixer with another rule brings a class of its own (frozen
+    dataclasses make good ones: equal rules compare equal and hash alike)."""
 
-    ``retention``: "full" keeps every position; "window" keeps the last ``window`` positions
-    besides the current one, older pages go back to the pool. ``k_shape`` / ``v_shape`` give the
-    per-page tensor shapes as functions of the page size."""
-    retention: str
-    window: Optional[int]
+    # every position stays for the whole life of the request: only then can pages that hold a
+    # prompt's prefix be shared between requests
+    keeps_everything: ClassVar[bool] = False
+
+    def first_kept_page(self, next_position: int, page_size: int) -> int:
+        """Index of the first page the request still needs when its next query stands at
+        ``next_position``; pages before it are given back, and no kernel may touch them."""
+        raise NotImplementedError
+
+    def first_kept_pages(self, next_positions, page_size: int):
+        """The same for an int64 array of positions (one per sequence of a step)."""
+        import numpy as np
+        return np.fromiter((self.first_kept_page(int(p), page_size) for p in next_positions), dtype=np.int64,
+                           count=len(next_positions))
+
+    def most_pages(self, length: int, page_size: int) -> Optional[int]:
+        """Most pages a request of ``length`` tokens holds at one time, if the rule can tell
+        (a request that needs more than its pool has is refused when it is submitted)."""
+        return None
+
+    def key(self) -> Tuple:
+        """Calls whose needs have equal keys share a group: a pool and block tables of their own."""
+        return (type(self).__name__,) + tuple(sorted(vars(self).items()))
+
+
+@dataclass(frozen=True)
+class KeepAll(Retention):
+    keeps_everything: ClassVar[bool] = True
+
+    def first_kept_page(self, next_position: int, page_size: int) -> int:
+        return 0
+
+    def first_kept_pages(self, next_positions, page_size: int):
+        import numpy as np
+        return np.zeros(len(next_positions), dtype=np.int64)
+
+    def most_pages(self, length: int, page_size: int) -> Optional[int]:
+        return -(-length // page_size)
+
+
+@dataclass(frozen=True)
+class KeepWindow(Retention):
+    """The last ``window`` positions besides the query's own stay; older pages go back to the pool."""
+    window: int = 0
+
+    def __post_init__(self):
+        if self.window < 0:
+            raise ValueError(f"a window must be >= 0, got {self.window}")
+
+    def first_kept_page(self, next_position: int, page_size: int) -> int:
+        return max(0, next_position - self.window) // page_size
+
+    def first_kept_pages(self, next_positions, page_size: int):
+        import numpy as np
+        return np.maximum(0, np.asarray(next_positions, dtype=np.int64) - self.window) // page_size
+
+
+class CacheNeed:
+    """Paged memory a mixer needs for each token of a request: which tensors a page consists of
+    and how long positions are kept. The executor allocates ``[pages, *shape]`` per named tensor
+    for every call with this need and hands them to the mixer as ``ctx.kv(call).pages[name]``."""
+
+    retention: Retention
+
+    def page_shapes(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
+        """Name -> shape of one page of ``page_size`` token slots."""
+        raise NotImplementedError
+
+    def group_key(self) -> Tuple:
+        return self.retention.key()
+
+    def bytes_per_token(self, itemsize: int) -> int:
+        total = 0
+        for shape in self.page_shapes(1).values():
+            n = 1
+            for d in shape:
+                n *= int(d)
+            total += n
+        return total * itemsize
+
+
+@dataclass(frozen=True)
+class KeyValueNeed(CacheNeed):
+    """Keys and values of softmax attention: K pages ``[kv_heads, slot, head_dim]`` and V pages
+    transposed, ``[kv_heads, head_dim, slot]``, so that both matrix products of the attention
+    kernels read their first operand straight from a page."""
+    retention: Retention
     num_kv_heads: int
     head_dim: int
 
-    def group_key(self) -> Tuple:
-        return (self.retention, self.window)
-
-    def page_shapes(self, page_size: int) -> Tuple[Tuple[int, ...], Tuple[int, ...]]:
-        return ((self.num_kv_heads, page_size, self.head_dim), (self.num_kv_heads, self.head_dim, page_size))
-
-    def bytes_per_token(self, itemsize: int) -> int:
-        return 2 * self.num_kv_heads * self.head_dim * itemsize
+    def page_shapes(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
+        return {"k": (self.num_kv_heads, page_size, self.head_dim), "v": (self.num_kv_heads, self.head_dim, page_size)}
 
 
 # ---------------------------------------------------------------------------------------
@@ -100,12 +178,16 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("output head")
 
 register_mixer = MIXERS.register
 register_feed_forward = FEED_FORWARDS.register
 register_norm = NORMS.register
 register_position_encoding = POSITION_ENCODINGS.register
 register_block = BLOCKS.register
+register_embedding = EMBEDDINGS.register
+register_head = HEADS.register
 
 
 # ---------------------------------------------------------------------------------------
@@ -249,6 +331,12 @@ class Norm(Part):
     def pending(self, stream: HiddenStream, ctx):
         return self.forward(stream, ctx)
 
+    def as_scaled_rms(self) -> Optional[Tuple[torch.Tensor, float, bool]]:
+        """(weight, eps, unit_offset) when this norm computes ``x / sqrt(mean(x^2) + eps) * w`` (or
+        ``* (1 + w)`` with ``unit_offset``) over the whole row, the form that the fused add + norm +
+        product kernel computes itself; None (the default) keeps the norm a kernel of its own."""
+        return None
+
     def forward(self, stream: HiddenStream, ctx, rows: Optional[torch.Tensor] = None,
                 tag: str = "normed") -> torch.Tensor:
         raise NotImplementedError
@@ -292,6 +380,20 @@ class FeedForward(Part):
     """forward(x, ctx) -> y, token by token."""
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    """forward(ctx, resid): fills the float32 residual stream [tokens, hidden] from ``ctx.token_ids``."""
+
+    def forward(self, ctx, resid: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """forward(h, ctx) -> float32 logits [rows, vocab] from the normalised rows whose logits are wanted."""
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         raise NotImplementedError
 
 

@@ -53,5 +53,8 @@ class RMSNorm(Norm):
             return PendingNorm(self, stream, ctx)
         return self.forward(stream, ctx)
 
+    def as_scaled_rms(self):
+        return self.weight, self.spec.eps, self.spec.unit_offset
+
     def apply(self, x: torch.Tensor, out: torch.Tensor) -> None:
         self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, out, unit_offset=self.spec.unit_offset)

@@ -25,9 +25,11 @@ class TensorLocation:
 
 @dataclass(frozen=True)
 class LayerPlan:
+    """One layer: the block arrangement and the parts it wires. A layer may go without a mixer or
+    without a feed-forward (None); its block arrangement then gets None in that place."""
     block: PartSpec
-    mixer: PartSpec
-    ffn: PartSpec
+    mixer: Optional[PartSpec]
+    ffn: Optional[PartSpec]
     norms: Tuple[Tuple[str, PartSpec], ...]   # (slot, spec) pairs the block arrangement wires
 
     def norm_map(self) -> Dict[str, PartSpec]:
@@ -61,11 +63,11 @@ class ModelPlan:
     hidden_size: int
     vocab_size: int
     max_positions: int
-    embedding: EmbeddingSpec
+    embedding: PartSpec            # EmbeddingSpec, or the spec of another registered embedding
     layers: Tuple[LayerPlan, ...]
     calls: Tuple[Call, ...]
     final_norm: PartSpec
-    head: HeadSpec
+    head: PartSpec                 # HeadSpec, or the spec of another registered head
 
     def validate(self) -> None:
         if not self.layers:

@@ -6,9 +6,24 @@ import random
 import pytest
 
 from minivllm_amd.cache import (CacheManager, GroupSpec, OutOfPages, OutOfSlots, PagePool, StateSlots, page_hash)
+from minivllm_amd.parts import KeepAll, KeepWindow, Retention
 
-FULL = GroupSpec("full", None, (0, 1))
-WIN = GroupSpec("window", 21, (2,))
+from dataclasses import dataclass
+
+
+@dataclass(frozen=True)
+class KeepChunk(Retention):
+    """A third rule, defined here: a query sees the positions of its own chunk of ``chunk`` tokens
+    only, so every page before the chunk of the next query can go."""
+    chunk: int = 1
+
+    def first_kept_page(self, next_position, page_size):
+        return (next_position // self.chunk) * self.chunk // page_size
+
+
+FULL = GroupSpec(KeepAll(), (0, 1))
+WIN = GroupSpec(KeepWindow(21), (2,))
+CHUNK = GroupSpec(KeepChunk(12), (3,))
 
 
 def test_page_hash_is_the_references_chain():
@@ -30,7 +45,7 @@ def test_page_hash_is_the_references_chain():
 
 def test_reference_vectors_with_prefix_caching():
     ps = 256
-    m = CacheManager([GroupSpec("full", None, (0,))], 10240, ps, 512, enable_prefix_caching=True)
+    m = CacheManager([GroupSpec(KeepAll(), (0,))], 10240, ps, 512, enable_prefix_caching=True)
     rng = random.Random(0)
     tokens = [rng.randint(1, 25600) for _ in range(25600)]
     m.admit("big", tokens)
@@ -105,6 +120,29 @@ def test_window_group_gives_pages_back():
     assert m.pools[0].num_free == 64 and m.pools[1].num_free == 64
 
 
+def test_a_retention_rule_defined_outside_the_framework():
+    """The manager asks a group's retention object for the first page still needed and nothing else:
+    a rule defined in this file (the chunk of the next query) gives its pages back like the others."""
+    ps = 8
+    m = CacheManager([FULL, CHUNK], 64, ps, 4)
+    assert [g.retention.key() for g in m.groups] == [("KeepAll",), ("KeepChunk", ("chunk", 12))]
+    m.admit("a")
+    for n in (7, 5, 30, 1, 1, 40, 11):
+        m.reserve("a", n)
+        m.commit("a", n)
+        seq = m.sequence("a")
+        first_kept = (seq.num_computed // 12) * 12 // ps
+        kept = seq.pages[1]
+        assert all(p == -1 for p in kept[:first_kept]) and all(p >= 0 for p in kept[first_kept:])
+        assert all(p >= 0 for p in seq.pages[0])
+        m.check_invariants()
+    assert m.pools[1].num_used <= 3
+    m.release("a")
+    assert all(p.num_free == 64 for p in m.pools)
+    with pytest.raises(TypeError):
+        GroupSpec("full", (0,))                      # a name is not a rule
+
+
 def test_reserve_is_all_or_nothing():
     m = CacheManager([FULL, WIN], [10, 2], 4, 4)
     m.admit("a")
@@ -144,7 +182,7 @@ def test_random_orders(seed, prefix):
     every operation and every page is back at the end."""
     rng = random.Random(seed)
     ps = rng.choice([4, 8, 16])
-    groups = [FULL] if prefix else [FULL, WIN]
+    groups = [FULL] if prefix else [FULL, WIN, CHUNK]
     m = CacheManager(groups, 40, ps, 6, enable_prefix_caching=prefix)
     assert m.prefix_caching == prefix
     shared = [rng.randrange(100) for _ in range(3 * ps)]

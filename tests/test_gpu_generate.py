@@ -159,7 +159,7 @@ def test_pool_sized_from_the_memory_left(models):
     llm = LLM(model=path, dtype="bfloat16", kv_cache_block_size=8, max_model_len=96, max_num_batched_tokens=256,
               max_num_batched_seqs=6, gpu_memory_utilization=0.3)
     assert llm.executor.num_pages == 6 * 12 and llm.manager.pools[0].num_pages == 72
-    assert all(k.shape[0] == 72 and v.shape[0] == 72 for k, v in llm.executor.kv_pages.values())
+    assert all(t.shape[0] == 72 for pages in llm.executor.kv_pages.values() for t in pages.values())
     prompts = [random_tokens(cfg, n, seed=70 + n) for n in (30, 3, 11)]
     sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
     outs = llm.generate(prompts, sp, use_tqdm=False)

@@ -49,7 +49,7 @@ class Ctx:
             bt[i, :len(t)] = torch.tensor(t, dtype=torch.int32)
         self.block_table = bt.to(dev)
         self.attention_plan = None
-        self._kv = KVView(kv[0], kv[1], self.block_table, page_size)
+        self._kv = KVView({"k": kv[0], "v": kv[1]}, self.block_table, page_size)
 
     def kv(self, call):
         return self._kv
@@ -131,7 +131,8 @@ def test_attention_part_and_block(dtype, layer):
     mixer_cls = MIXERS.get(spec.kind)
     mixer = mixer_cls(spec, tensors("mixer", mixer_cls.tensors(spec)), rt, position=rope)
     need = mixer_cls.cache_need(spec)
-    assert need.retention == ("full" if layer == 0 else "window") and need.window == (None if layer == 0 else 20)
+    from minivllm_amd.parts import KeepAll, KeepWindow
+    assert need.retention == (KeepAll() if layer == 0 else KeepWindow(20))
 
     g = torch.Generator().manual_seed(2)
     lens = [50, 44]
@@ -141,7 +142,9 @@ def test_attention_part_and_block(dtype, layer):
     want = [plain.attention_block(cfg, wd, layer, x.double(), torch.arange(x.shape[0])) for x in x_all]
 
     tables, width, n_pages = hand_made_step(rt, [(0, 0, 50), (1, 0, 44)], ps, None)
-    k_shape, v_shape = need.page_shapes(ps)
+    shapes = need.page_shapes(ps)
+    assert list(shapes) == ["k", "v"]
+    k_shape, v_shape = shapes["k"], shapes["v"]
     kv = (torch.full((n_pages,) + k_shape, float("nan"), dtype=rt.dtype, device=dev),
           torch.full((n_pages,) + v_shape, float("nan"), dtype=rt.dtype, device=dev))
     # step 1: the first 30 tokens of sequence 1 alone

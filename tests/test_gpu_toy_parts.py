@@ -443,3 +443,257 @@ def test_toy_routed_feed_forward_and_learned_positions():
     for r in reqs:
         mgr.release(r)
     mgr.check_invariants()
+
+
+def define_chunk_toy():
+    """A third toy architecture. Its mixer caches one tensor per token (the mixer's input itself, no
+    keys and values) and keeps it by a rule of its own: a query sees its own chunk of 12 tokens,
+    every page before that chunk goes back to the pool. Its layers have no feed-forward (a block
+    arrangement defined here wires a norm and a mixer only), its norm centres the row (not an RMS
+    norm, so no kernel may fuse it as one), and its head caps the logits."""
+    from minivllm_amd.config.model_config import ModelConfig
+    from minivllm_amd.models.registry import Architecture, register_architecture
+    from minivllm_amd.parts import (BLOCKS, HEADS, MIXERS, NORMS, Block, CacheNeed, Call, EmbeddingSpec, Head, LayerPlan,
+                                    Mixer, ModelPlan, Norm, PartSpec, Retention, TensorDecl, register_block,
+                                    register_head, register_mixer, register_norm)
+
+    @dataclass(frozen=True)
+    class KeepChunk(Retention):
+        chunk: int = 1
+
+        def first_kept_page(self, next_position, page_size):
+            return (next_position // self.chunk) * self.chunk // page_size
+
+    @dataclass(frozen=True)
+    class InputCacheNeed(CacheNeed):
+        retention: Retention
+        hidden_size: int
+
+        def page_shapes(self, page_size):
+            return {"x": (page_size, self.hidden_size)}
+
+    @dataclass(frozen=True)
+    class ChunkMeanSpec(PartSpec):
+        kind: ClassVar[str] = "toy_chunk_mean"
+        hidden_size: int = 0
+        chunk: int = 1
+
+    class ChunkMean(Mixer):
+        """y_t = W mean(x_s : chunk start <= s <= t), the x_s read back from the paged cache."""
+        graph_safe = False
+
+        @classmethod
+        def tensors(cls, spec):
+            return {"w": TensorDecl((spec.hidden_size, spec.hidden_size))}
+
+        @classmethod
+        def cache_need(cls, spec):
+            return InputCacheNeed(KeepChunk(spec.chunk), spec.hidden_size)
+
+        def __init__(self, spec, tensors, rt):
+            self.spec, self.w = spec, tensors["w"]
+
+        def forward(self, x, ctx, call):
+            view = ctx.kv(call)
+            assert set(view.pages) == {"x"}
+            pages, ps, C = view.pages["x"], view.page_size, self.spec.chunk
+            y = torch.zeros_like(x)
+            base = 0
+            for i, (n, start) in enumerate(zip(ctx.q_lens, ctx.starts)):
+                table = view.block_table[i].long()
+                pos = torch.arange(start, start + n, device=x.device)
+                pages[table[pos // ps], pos % ps] = x[base:base + n]
+                for j in range(n):
+                    p = start + j
+                    seen = torch.arange((p // C) * C, p + 1, device=x.device)
+                    ids = table[seen // ps]
+                    assert int(ids.min()) >= 0, "a page the query needs was given back"
+                    mean = pages[ids, seen % ps].float().mean(dim=0)
+                    y[base + j] = (mean @ self.w.float().T).to(x.dtype)
+                base += n
+            return y
+
+    @dataclass(frozen=True)
+    class CentredNormSpec(PartSpec):
+        kind: ClassVar[str] = "toy_centred_norm"
+        size: int = 0
+        eps: float = 1e-5
+
+    class CentredNorm(Norm):
+        """(x - mean) / sqrt(var + eps) * w: it declares no RMS form, so it always runs by itself."""
+
+        @classmethod
+        def tensors(cls, spec):
+            return {"weight": TensorDecl((spec.size,), init="ones_normal")}
+
+        def __init__(self, spec, tensors, rt):
+            self.spec, self.rt, self.weight = spec, rt, tensors["weight"]
+
+        def forward(self, stream, ctx, rows=None, tag="normed"):
+            delta = stream.delta
+            if delta is not None and not isinstance(delta, torch.Tensor):
+                delta = delta.materialize()
+            x = stream.resid if delta is None else stream.resid + delta.float()
+            if rows is None:
+                stream.resid, stream.delta = x, None
+            else:
+                x = x[rows.long()]
+            c = x - x.mean(-1, keepdim=True)
+            return (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + self.spec.eps) * self.weight.float()).to(self.rt.dtype)
+
+    @dataclass(frozen=True)
+    class MixerOnlySpec(PartSpec):
+        kind: ClassVar[str] = "toy_mixer_only"
+
+    class MixerOnly(Block):
+        """x = x + mixer(norm(x)); the layer has no feed-forward."""
+        norm_slots = ("mixer",)
+
+        def __init__(self, spec, norms, mixer, ffn):
+            assert ffn is None
+            self.norm, self.mixer = norms["mixer"], mixer
+
+        def forward(self, stream, ctx, call):
+            stream.delta = self.mixer.forward(self.norm.forward(stream, ctx), ctx, call)
+
+    @dataclass(frozen=True)
+    class CappedHeadSpec(PartSpec):
+        kind: ClassVar[str] = "toy_capped_head"
+        vocab_size: int = 0
+        hidden_size: int = 0
+        cap: float = 1.0
+
+    class CappedHead(Head):
+        """logits = cap * tanh(h W^T / cap), in float32."""
+
+        @classmethod
+        def tensors(cls, spec):
+            return {"weight": TensorDecl((spec.vocab_size, spec.hidden_size))}
+
+        def __init__(self, spec, tensors, rt):
+            self.spec, self.rt, self.weight = spec, rt, tensors["weight"]
+
+        def forward(self, h, ctx):
+            raw = torch.empty((h.shape[0], self.spec.vocab_size), dtype=torch.float32, device=h.device)
+            self.rt.ops.gemm(h, self.weight, raw)             # the engine's product, then the cap
+            return self.spec.cap * torch.tanh(raw / self.spec.cap)
+
+    for registry, register, spec, cls in ((MIXERS, register_mixer, ChunkMeanSpec, ChunkMean),
+                                          (NORMS, register_norm, CentredNormSpec, CentredNorm),
+                                          (BLOCKS, register_block, MixerOnlySpec, MixerOnly),
+                                          (HEADS, register_head, CappedHeadSpec, CappedHead)):
+        registry.unregister(spec.kind)
+        register(spec.kind, cls)
+
+    @dataclass(frozen=True)
+    class ChunkConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyChunkLM"
+        vocab_size: int = 70
+        hidden_size: int = 64
+        max_position_embeddings: int = 128
+        dtype: str = "float32"
+
+        @classmethod
+        def from_dict(cls, d, where="config.json"):
+            return cls(vocab_size=d["vocab_size"], hidden_size=d["hidden_size"])
+
+    def plan(cfg):
+        h = cfg.hidden_size
+        norm = CentredNormSpec(size=h, eps=1e-5)
+        layer = LayerPlan(MixerOnlySpec(), ChunkMeanSpec(hidden_size=h, chunk=12), None, (("mixer", norm),))
+        return ModelPlan(hidden_size=h, vocab_size=cfg.vocab_size, max_positions=cfg.max_position_embeddings,
+                         embedding=EmbeddingSpec(cfg.vocab_size, h), layers=(layer, layer), calls=(Call(0), Call(1)),
+                         final_norm=norm, head=CappedHeadSpec(cfg.vocab_size, h, cap=3.0))
+
+    def tensor_name(cfg, loc):
+        return f"{loc.role}.{loc.name}" if loc.layer is None else f"layers.{loc.layer}.{loc.role}.{loc.name}"
+
+    arch = Architecture("ToyChunkLM", ChunkConfig, plan, tensor_name)
+    register_architecture(arch, replace=True)
+    return arch, ChunkConfig()
+
+
+def chunk_plain(w: Dict[str, torch.Tensor], tokens, chunk=12, cap=3.0):
+    w = {k: v.double() for k, v in w.items()}
+    x = w["embedding.weight"][torch.tensor(tokens)]
+    n = len(tokens)
+
+    def norm(v, weight):
+        c = v - v.mean(-1, keepdim=True)
+        return c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + 1e-5) * weight
+
+    for layer in range(2):
+        hcur = norm(x, w[f"layers.{layer}.norm.mixer.weight"])
+        y = torch.stack([hcur[(t // chunk) * chunk:t + 1].mean(0) for t in range(n)])
+        x = x + y @ w[f"layers.{layer}.mixer.w"].T
+    return (cap * torch.tanh(norm(x, w["final_norm.weight"]) @ w["head.weight"].T / cap)).numpy()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_one_tensor_cache_with_its_own_retention_norm_block_and_head(dtype):
+    """A mixer with a one-tensor cache and a third retention rule, a layer without feed-forward, a
+    norm that is no RMS norm and a head that caps its logits: all defined in this file, built and
+    stepped through the engine without a change to it; two requests beside each other in portions
+    and token by token, on a pool that holds them only because pages behind a chunk come back."""
+    from minivllm_amd.config import EngineConfig
+    from minivllm_amd.engine.executor import Executor
+    from minivllm_amd.engine.step import SeqStep
+    from minivllm_amd.models import expected_tensors
+    from minivllm_amd.weights import DictSource
+
+    arch, cfg = define_chunk_toy()
+    g = torch.Generator().manual_seed(8)
+    weights = {}
+    for name, decl in expected_tensors(arch, cfg).items():
+        t = torch.randn(decl.shape, generator=g) * 0.3
+        weights[name] = (t + 1.0) if decl.init == "ones_normal" else t
+    assert sorted(weights) == ["embedding.weight", "final_norm.weight", "head.weight", "layers.0.mixer.w",
+                               "layers.0.norm.mixer.weight", "layers.1.mixer.w", "layers.1.norm.mixer.weight"]
+    ex = Executor(EngineConfig(model="", dtype=dtype, max_model_len=128, kv_cache_block_size=8,
+                               kv_cache_num_blocks=8, max_num_batched_seqs=2),
+                  model=(arch, cfg, DictSource(weights)))
+    assert len(ex.groups) == 1 and ex.groups[0].retention.key() == ("KeepChunk", ("chunk", 12))
+    assert {n: tuple(t.shape) for n, t in ex.kv_pages[0].items()} == {"x": (8, 8, 64)}
+    mgr = ex.new_cache_manager(enable_prefix_caching=True)
+    assert not mgr.prefix_caching                      # the rule does not keep everything
+    rng = np.random.default_rng(2)
+    reqs = {r: [int(t) for t in rng.integers(0, 70, size=n)] for r, n in (("a", 61), ("b", 47))}
+    want = {r: chunk_plain(weights, t) for r, t in reqs.items()}
+    tol = 3e-5 if dtype == "float32" else 4e-2
+
+    def run(entries):
+        seqs = []
+        for rid, toks in entries:
+            if rid not in mgr:
+                mgr.admit(rid)
+            mgr.reserve(rid, len(toks))
+            s = mgr.sequence(rid)
+            seqs.append(SeqStep(toks, s.num_computed, [mgr.block_table(rid, 0)], s.state_slot, list(range(len(toks)))))
+        out = ex.step(seqs).cpu().numpy()
+        for rid, toks in entries:
+            mgr.commit(rid, len(toks))
+        mgr.check_invariants()
+        return out
+
+    assert rel_err(run([("a", reqs["a"])]), want["a"]) <= tol           # whole: all 8 pages for one request
+    mgr.release("a")
+    done = {r: 0 for r in reqs}
+    sizes = [5, 2, 9, 3, 1, 1, 7, 2]
+    k = most_used = 0
+    while any(done[r] < len(reqs[r]) for r in reqs):
+        entries = []
+        for r in reqs:
+            if done[r] < len(reqs[r]):
+                n = min(sizes[k % len(sizes)], len(reqs[r]) - done[r]); k += 1
+                entries.append((r, reqs[r][done[r]:done[r] + n]))
+        out = run(entries)
+        most_used = max(most_used, mgr.pools[0].num_used)
+        row = 0
+        for r, toks in entries:
+            assert rel_err(out[row:row + len(toks)], want[r][done[r]:done[r] + len(toks)]) <= tol, (r, done[r])
+            row += len(toks); done[r] += len(toks)
+    # 108 tokens went through a pool of 64 slots: pages behind the chunks were given back and used again
+    assert most_used <= 8 and sum(len(t) for t in reqs.values()) > 8 * 8
+    for r in reqs:
+        mgr.release(r)
+    assert mgr.pools[0].num_free == 8

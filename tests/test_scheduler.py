@@ -8,6 +8,7 @@ import zlib
 import pytest
 
 from minivllm_amd.cache import CacheManager, GroupSpec
+from minivllm_amd.parts import KeepAll, KeepWindow
 from minivllm_amd.config import SamplingParams
 from minivllm_amd.engine.request import Request, RequestState
 from minivllm_amd.engine.scheduler import Scheduler
@@ -34,7 +35,7 @@ def expected_output(prompt, max_tokens, ignore_eos=True):
 class FakeEngine:
     def __init__(self, num_pages, page_size, groups=None, max_tokens=64, max_seqs=8, chunk=None, prefix=False,
                  max_model_len=4096, repeat=1):
-        self.groups = groups or [GroupSpec("full", None, (0,))]
+        self.groups = groups or [GroupSpec(KeepAll(), (0,))]
         self.manager = CacheManager(self.groups, num_pages, page_size, max_seqs, enable_prefix_caching=prefix)
         self.sched = Scheduler(self.manager, max_tokens, max_seqs, max_model_len, eos_token_ids=(EOS,),
                                prefill_chunk=chunk, max_decode_repeat=repeat)
@@ -75,7 +76,7 @@ class FakeEngine:
                 assert end == len(r.tokens)
                 contexts = []
                 for g, spec in enumerate(self.groups):
-                    lo = 0 if spec.retention == "full" else max(0, end - 1 - spec.window)
+                    lo = spec.retention.first_kept_page(end - 1, 1)          # (page size 1: the first kept position)
                     table = seq.pages[g]
                     ctx = [self.mem[g][(table[p // self.ps], p % self.ps)] for p in range(lo, end)]
                     assert ctx == r.tokens[lo:end], "the cache does not hold the request's tokens"
@@ -107,7 +108,7 @@ class FakeEngine:
                     table = seq.pages[g]
                     assert table[pos // self.ps] >= 0
                     self.mem[g][(table[pos // self.ps], pos % self.ps)] = toks[pos]
-                    lo = 0 if spec.retention == "full" else max(0, pos - spec.window)
+                    lo = spec.retention.first_kept_page(pos, 1)
                     ctx = [self.mem[g][(table[p // self.ps], p % self.ps)] for p in range(lo, pos + 1)]
                     assert ctx == toks[lo:pos + 1], "the cache does not hold the request's tokens"
                     contexts.append(ctx)
@@ -245,7 +246,7 @@ def test_preempted_request_returns_to_the_front_and_the_newest_gives_way():
 
 
 def test_windowed_group_and_recycled_pages():
-    groups = [GroupSpec("full", None, (0,)), GroupSpec("window", 6, (1,))]
+    groups = [GroupSpec(KeepAll(), (0,)), GroupSpec(KeepWindow(6), (1,))]
     e = FakeEngine(num_pages=40, page_size=4, groups=groups, max_tokens=24, max_seqs=4)
     rng = random.Random(5)
     reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=20, ignore_eos=True) for n in (30, 3, 18, 9, 25)]
@@ -336,7 +337,7 @@ def test_repeat_shrinks_to_the_free_pages():
 
 
 def test_repeat_with_a_window_group():
-    groups = [GroupSpec("full", None, (0,)), GroupSpec("window", 6, (1,))]
+    groups = [GroupSpec(KeepAll(), (0,)), GroupSpec(KeepWindow(6), (1,))]
     e = FakeEngine(num_pages=48, page_size=4, groups=groups, max_tokens=32, max_seqs=4, repeat=4)
     rng = random.Random(13)
     reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=19, ignore_eos=True) for n in (11, 3)]
