@@ -7,8 +7,9 @@ The default run has the layer sizes of the Qwen3-0.6B shape (28 layers, hidden 1
 heads, 8 key/value heads, head_dim 128, intermediate 3072, vocabulary 151936, tied head), a
 batch of 8 requests with 1,024-token prompts inside a 4,096-token context limit, bfloat16. A
 "step" is one decode step of the whole engine (schedule, run the batch from a HIP graph,
-sample, update). W warm-up steps, then exactly K timed steps between synchronisations. One
-JSON line is printed:
+sample, update). W warm-up steps, then exactly K timed steps between synchronisations; such
+regions of K steps follow each other until half a second has been timed, and the median region
+is the one reported (``timed_regions`` says how many there were). One JSON line is printed:
 
   value        decoded tokens per second at the default batch
   prefill      one 2,048-token prompt run whole: tokens/s, ms, and its share of the bf16 MFMA peak
@@ -37,17 +38,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-SHAPES = {
-    "0.6b": dict(num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
-                 intermediate_size=3072, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
-                 tie_word_embeddings=True),
-    "8b": dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-               intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
-               tie_word_embeddings=False),
-    "32b": dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
-                intermediate_size=25600, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
-                tie_word_embeddings=False),
-}
+from minivllm_amd.config.shapes import QWEN3_SHAPES
+
+SHAPES = {k: v for k, v in QWEN3_SHAPES.items() if k != "tiny"}
+MIN_TIMED_SECONDS = 0.5
+MAX_REGIONS = 101
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
@@ -118,21 +113,34 @@ def measure_decode(llm, vocab, batch, prompt_len, steps, warmup, seed):
         finally:
             llm.config.launch_ahead = ahead
     run(warmup)
-    torch.cuda.synchronize()
-    before = sum(r.num_completion_tokens for r in reqs)
-    t0 = time.perf_counter()
-    run(steps)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    tokens = sum(r.num_completion_tokens for r in reqs) - before
+    # Regions of exactly ``steps`` steps, each between synchronisations, one after the other until
+    # MIN_TIMED_SECONDS have been timed (or the context limit is near): the median region is reported,
+    # so that a short region (20 steps are 30 ms) does not stand on one sample.
+    regions = []
+    margin = steps + 2 * llm.config.num_scheduler_steps + 2
+    while True:
+        torch.cuda.synchronize()
+        before = sum(r.num_completion_tokens for r in reqs)
+        ctx_before = prompt_len + min(r.num_completion_tokens for r in reqs)
+        t0 = time.perf_counter()
+        run(steps)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        tokens = sum(r.num_completion_tokens for r in reqs) - before
+        regions.append((dt / (tokens / batch), tokens, dt, ctx_before + tokens / batch / 2.0))
+        longest = prompt_len + max(r.num_completion_tokens for r in reqs)
+        if sum(r[2] for r in regions) >= MIN_TIMED_SECONDS or longest + margin >= llm.config.max_model_len \
+                or len(regions) >= MAX_REGIONS:
+            break
+    regions.sort()
+    per_step, tokens, dt, mean_ctx = regions[len(regions) // 2]
     done_steps = tokens / batch
-    mean_ctx = prompt_len + 1 + warmup + done_steps / 2.0
     # finish and free
     for r in reqs:
         r.sampling_params.max_tokens = r.num_completion_tokens
     while llm.has_unfinished():
         llm.step()
-    return tokens / dt, dt / done_steps * 1e3, mean_ctx, int(round(done_steps))
+    return tokens / dt, per_step * 1e3, mean_ctx, int(round(done_steps)), len(regions)
 
 
 def measure_prefill(llm, vocab, tokens, repeats, seed):
@@ -256,10 +264,10 @@ def main() -> int:
                    "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
 
     tok_s = ms_step = roofline = None
-    ran = 0
+    ran = regions = 0
     if args.only in ("all", "decode"):
-        tok_s, ms_step, mean_ctx, ran = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len, args.steps,
-                                                       args.warmup, args.seed)
+        tok_s, ms_step, mean_ctx, ran, regions = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len,
+                                                                args.steps, args.warmup, args.seed)
         step_bytes = nums["step_params"] * item + args.batch * mean_ctx * nums["kv_bytes_per_token"] * item
         achieved = step_bytes / (ms_step * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -269,7 +277,7 @@ def main() -> int:
     if not args.no_points and args.only == "all":
         for b, key in ((1, "decode_b1"), (64, "decode_b64")):
             n = min(args.steps, 128)
-            v, _, _, _ = measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8), args.seed + b)
+            v = measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8), args.seed + b)[0]
             points[key] = round(v, 1)
 
     config = {"model": f"qwen3-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
@@ -283,7 +291,7 @@ def main() -> int:
             "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1, "steps": ran if ran else args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms_step, 4) if ms_step is not None else None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic", "config": config,
-            "prefill": prefill, "roofline": roofline, "points": points}
+            "timed_regions": regions, "prefill": prefill, "roofline": roofline, "points": points}
     print(json.dumps(line))
     return 0
 

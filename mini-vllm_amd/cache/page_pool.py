@@ -42,7 +42,11 @@ class OutOfPages(RuntimeError):
 
 
 class PagePool:
-    def __init__(self, num_pages: int):
+    def __init__(self, num_pages: int, on_recycle=None):
+        """``on_recycle(page, why)`` is told when a page is handed out for new content ("allocate")
+        and when its last holder lets go of it ("release"): a debugging hook, see
+        ``EngineConfig.debug_poison_pages``."""
+        self.on_recycle = on_recycle
         if num_pages < 1:
             raise ValueError(f"a page pool needs at least one page, got {num_pages}")
         self.num_pages = num_pages
@@ -74,6 +78,8 @@ class PagePool:
         self._forget(page)
         assert self.refcount[page] == 0
         self.refcount[page] = 1
+        if self.on_recycle is not None:
+            self.on_recycle(page, "allocate")
         return page
 
     def share(self, page: int) -> None:
@@ -91,6 +97,8 @@ class PagePool:
         self.refcount[page] -= 1
         if self.refcount[page] == 0:
             self._free[page] = None
+            if self.on_recycle is not None:
+                self.on_recycle(page, "release")
 
     # ---- content ----------------------------------------------------------------------------
     def _forget(self, page: int) -> None:

@@ -2,6 +2,7 @@ from .model_config import (ConfigError, ModelConfig, Qwen3Config, read_config_js
                            architecture_name)
 from .engine_config import EngineConfig, compute_dtype_name
 from .sampling_params import SamplingParams
+from .shapes import QWEN3_SHAPES, qwen3_shape
 
 __all__ = ["ConfigError", "ModelConfig", "Qwen3Config", "read_config_json", "architecture_name",
-           "EngineConfig", "SamplingParams", "compute_dtype_name"]
+           "EngineConfig", "SamplingParams", "compute_dtype_name", "QWEN3_SHAPES", "qwen3_shape"]

@@ -74,6 +74,11 @@ class EngineConfig:
     # reference does, minivllm/executor/graph.py:24-58) instead of at a graph's first use, which
     # makes that step wait for the recording
     capture_graphs_at_start: bool = False
+    # debugging: fill a cache page with NaN when it is handed out for new content and (without
+    # prefix reuse, which revives given-back pages) when its last holder gives it back, so that a
+    # kernel that reads a slot nobody has written since, or a page that is no longer the request's,
+    # shows in the logits
+    debug_poison_pages: bool = False
     seed: int = 0
 
     def __post_init__(self) -> None:

@@ -152,6 +152,7 @@ class Executor:
         self._token_buffers: List[Optional[torch.Tensor]] = [None] * 4
         self._next_token_buffer = 0
         self.kv_pages: Dict[int, Dict[str, torch.Tensor]] = {}     # per call with a cache need: its page tensors by name
+        self._poison: Dict[int, List[int]] = {}                    # debug_poison_pages: pages to fill, per group
         self.state_tensors: Dict[int, torch.Tensor] = {}
         self.num_pages = 0
         self._allocate_memory()
@@ -229,8 +230,28 @@ class Executor:
         """A manager for this executor's pages and state slots."""
         if enable_prefix_caching is None:
             enable_prefix_caching = self.config.enable_prefix_caching
-        return CacheManager(self.groups, self.num_pages, self.page_size, self.num_state_slots,
-                            enable_prefix_caching=enable_prefix_caching, has_state=self.has_state)
+        manager = CacheManager(self.groups, self.num_pages, self.page_size, self.num_state_slots,
+                               enable_prefix_caching=enable_prefix_caching, has_state=self.has_state)
+        if self.config.debug_poison_pages:
+            self._poison = {g: [] for g in range(len(self.groups))}
+            for g, pool in enumerate(manager.pools):
+                # a page that prefix reuse may revive keeps its content until it is handed out anew
+                pool.on_recycle = (lambda page, why, g=g, keep=manager.prefix_caching:
+                                   None if (keep and why == "release") else self._poison[g].append(page))
+        return manager
+
+    def _flush_poison(self) -> None:
+        """debug_poison_pages: NaN into every page that changed hands since the last step, enqueued
+        before this step's kernels and behind those of every earlier step."""
+        for g, pages in self._poison.items():
+            if not pages:
+                continue
+            index = torch.tensor(sorted(set(pages)), dtype=torch.int64, device=self.device)
+            pages.clear()
+            for call in self.groups[g].calls:
+                for t in self.kv_pages.get(call, {}).values():
+                    if t.is_floating_point():
+                        t.index_fill_(0, index, float("nan"))
 
     # ------------------------------------------------------------------------------------
     # building a step
@@ -404,6 +425,8 @@ class Executor:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         self._validate(seqs)
         self._zero_new_states(seqs)
+        if self._poison:
+            self._flush_poison()
         S = len(seqs)
         decode_only = all(len(s.tokens) == 1 for s in seqs)
         if (self.config.use_cuda_graph and self.model.graph_safe and decode_only and S <= GRAPH_BUCKETS[-1]
@@ -495,6 +518,8 @@ class Executor:
             raise ValueError("a repeated step takes graph-sized batches of single tokens, each wanted")
         self._validate(seqs, lookahead=repeat - 1)
         self._zero_new_states(seqs)
+        if self._poison:
+            self._flush_poison()
         bucket = next(b for b in GRAPH_BUCKETS if b >= S)
         cap = self._repeat_cap(seqs, repeat)
         if after is not None and (after.bucket != bucket or after.count != S):

@@ -38,7 +38,7 @@ class TraceError(RuntimeError):
 
 class TraceRunner:
     def __init__(self, model: str, dtype: str, max_tokens: int, page_size: int = 16, use_graph: bool = True,
-                 max_live: int = 16, enable_prefix_caching: bool = False):
+                 max_live: int = 16, enable_prefix_caching: bool = False, poison_pages: bool = False):
         if TOKEN_ROUNDING % page_size:
             raise ValueError(f"the page size {page_size} must divide {TOKEN_ROUNDING}")
         max_tokens = max(TOKEN_ROUNDING, -(-max_tokens // TOKEN_ROUNDING) * TOKEN_ROUNDING)
@@ -48,7 +48,8 @@ class TraceRunner:
             model=model, dtype=dtype, max_model_len=min(max_pos, max_tokens),
             max_num_batched_tokens=max_tokens, max_num_batched_seqs=max_live,
             kv_cache_block_size=page_size, kv_cache_num_blocks=max_tokens // page_size,
-            use_cuda_graph=use_graph, enable_prefix_caching=enable_prefix_caching)
+            use_cuda_graph=use_graph, enable_prefix_caching=enable_prefix_caching,
+            debug_poison_pages=poison_pages)
         self.executor = Executor(config)
         self.manager = self.executor.new_cache_manager()
         # with prefix caching: every token a live request has brought so far (full pages are

@@ -45,6 +45,10 @@ def add_engine_options(ap: argparse.ArgumentParser) -> None:
                     help="decode-only steps run this many times in a row on the device (1: one token per step)")
     ap.add_argument("--no-launch-ahead", action="store_true",
                     help="read the tokens of a row of decode steps before the next row is launched")
+    ap.add_argument("--capture-graphs-at-start", action="store_true",
+                    help="record every decode graph before the first request instead of at its first use")
+    ap.add_argument("--debug-poison-pages", action="store_true",
+                    help="debugging: fill cache pages with NaN whenever they change hands")
     ap.add_argument("--seed", type=int, default=0)
 
 
@@ -66,7 +70,8 @@ def engine_config_from(args):
                         gpu_memory_utilization=args.gpu_memory_utilization,
                         enable_prefix_caching=args.enable_prefix_caching, use_cuda_graph=not args.no_cuda_graph,
                         num_scheduler_steps=args.num_scheduler_steps, launch_ahead=not args.no_launch_ahead,
-                        seed=args.seed)
+                        capture_graphs_at_start=args.capture_graphs_at_start,
+                        debug_poison_pages=args.debug_poison_pages, seed=args.seed)
 
 
 def sampling_params_from(args):
@@ -90,13 +95,9 @@ def main() -> int:
     from minivllm_amd import LLM
     tmp = None
     if args.random_model:
-        from bench import SHAPES
-        from minivllm_amd.config import Qwen3Config
+        from minivllm_amd.config import Qwen3Config, qwen3_shape
         from minivllm_amd.weights import write_model_folder
-        shape = SHAPES["0.6b"] if args.random_model == "0.6b" else dict(
-            num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
-            intermediate_size=128, vocab_size=256, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True)
-        cfg = Qwen3Config.from_dict(dict(shape, architectures=["Qwen3ForCausalLM"], max_position_embeddings=40960))
+        cfg = Qwen3Config.from_dict(qwen3_shape(args.random_model))
         tmp = tempfile.TemporaryDirectory()
         args.model = write_model_folder(os.path.join(tmp.name, "model"), cfg, seed=args.seed)
         logging.info("wrote a random %s model to %s", args.random_model, args.model)

@@ -127,6 +127,26 @@ def test_mixed(cases, name, dtype):
                 assert pool.num_free == pool.num_pages
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D128"])
+def test_mixed_with_poisoned_pages(cases, name, dtype):
+    """The mixed cutting with the debugging switch that fills every page with NaN when it changes
+    hands: a kernel that reads a slot nobody has written since (masked or not: 0 x NaN is NaN), or a
+    page a window has given back, would put NaN into the logits."""
+    from minivllm_amd.engine.trace import TraceRunner
+    case = cases[(name, "sharp")]
+    prompt_lens = {rid: max(2, len(t) - 12) if len(t) > 3 else len(t) for rid, t in case.reqs.items()}
+    steps = trace_tools.mixed(case.reqs, prompt_lens, max_live=4, seed=2)
+    runner = TraceRunner(case.dir, dtype, trace_tools.max_live_tokens(steps), page_size=case.page, poison_pages=True)
+    filled = []
+    real_flush = runner.executor._flush_poison
+    runner.executor._flush_poison = lambda: (filled.append(sum(len(v) for v in runner.executor._poison.values())),
+                                             real_flush())
+    got = trace_tools.collect(steps, runner.run_step)
+    assert len(got) == case.check(got, dtype, f"tiny {name} mixed on poisoned pages")     # (checks for finite values)
+    assert sum(filled) > runner.manager.pools[0].num_pages, "pages were not used again under the poison"
+
+
 def test_first_tokens_and_single_token_requests(cases):
     """The first positions of a sequence, and requests of one and two tokens."""
     case = cases[("A", "sharp")]
