@@ -10,6 +10,8 @@
 //                      i), so a row's draw does not depend on the rest of the batch.
 // Thresholds are found by radix descent over the order-preserving integer image of z.
 #include "common.h"
+#include "mv_noalloc.h"
+#include <mutex>
 
 #define SP_THREADS 1024
 
@@ -315,4 +317,48 @@ extern "C" int mv_sample_advance(const float* logits, long ld, int M, int V, con
                "sample_advance: the next step's token ids, positions and context lengths are needed");
     return sample_launch(logits, ld, M, V, temperature, top_k, top_p, rng, out, work, chunks,
                          Advance{next_ids, positions, context_lens, rng}, stream);
+}
+
+
+// ---------------------------------------------------------------------------------------
+// The variant that allocates nothing (see mv_noalloc.h): the first pass's partial results go
+// through this array instead of a workspace of the caller's.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[MV_NOALLOC_SCRATCH_BYTES];
+
+#define MV_NOALLOC_MAX_DEVICES 64
+static std::mutex g_scratch_lock;
+static void* g_scratch_ptr[MV_NOALLOC_MAX_DEVICES] = {nullptr};
+
+// The array's address on the current device, looked up once per device (every GPU holds a copy of
+// its own at an address of its own; the name `scratch` itself means nothing to host code).
+static int scratch_on_current_device(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return mv_fail("sample_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    MV_REQUIRE(dev >= 0 && dev < MV_NOALLOC_MAX_DEVICES, "sample_noalloc: device %d is beyond the %d this build knows",
+               dev, MV_NOALLOC_MAX_DEVICES);
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr)
+            return mv_fail("sample_noalloc: hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" int mv_sample_noalloc(const float* logits, long ld, int M, int V, const float* temperature,
+                                 const int* top_k, const float* top_p, const unsigned long long* rng, int* out,
+                                 hipStream_t stream) {
+    static_assert(sizeof(Best) == 8, "a partial result is 8 bytes");
+    MV_REQUIRE(M <= MV_NOALLOC_MAX_ROWS, "sample_noalloc: %d rows exceed the %d rows the library's own scratch "
+               "array holds; split the call, or use mv_sample with a workspace", M, MV_NOALLOC_MAX_ROWS);
+    MV_REQUIRE(logits != nullptr && out != nullptr, "sample_noalloc: logits and output are needed");
+    void* ptr = nullptr;
+    if (int rc = scratch_on_current_device(&ptr)) return rc;
+    return sample_launch(logits, ld, M, V, temperature, top_k, top_p, rng, out, ptr, MV_NOALLOC_CHUNKS,
+                         Advance{nullptr, nullptr, nullptr, nullptr}, stream);
 }

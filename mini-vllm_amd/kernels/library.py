@@ -25,6 +25,9 @@ _SIGNATURES = {
     "mv_built_dtypes": (c_int, []),
     "mv_abi_version": (c_int, []),
     "mv_graph_census": (c_int, [c_void_p, c_void_p]),
+    # logits, ld, M, V, temperature, top_k, top_p, rng, out, stream (no workspace: see csrc/mv_noalloc.h)
+    "mv_sample_noalloc": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p]),
     "mv_embedding": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "mv_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
                                c_int, c_int, c_int, c_void_p]),
