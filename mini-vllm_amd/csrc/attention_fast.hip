@@ -475,8 +475,8 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
                 if (nsplit == 1) {
                     const float inv = 1.f / l_fin;
                     uint2 packed;
-                    packed.x = (uint32_t)f32_to_bf16_bits(o[0] * inv) | ((uint32_t)f32_to_bf16_bits(o[1] * inv) << 16);
-                    packed.y = (uint32_t)f32_to_bf16_bits(o[2] * inv) | ((uint32_t)f32_to_bf16_bits(o[3] * inv) << 16);
+                    packed.x = f32x2_to_bf16x2_bits(o[0] * inv, o[1] * inv);
+                    packed.y = f32x2_to_bf16x2_bits(o[2] * inv, o[3] * inv);
                     *reinterpret_cast<uint2*>(orow + d0) = packed;
                 } else {
 #pragma unroll
@@ -491,12 +491,371 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// The one-wave variant, for steps whose grid is small (few sequences): a workgroup is a single
+// wave that takes a fixed chunk of 32 * BPW keys of one (sequence, kv head) pair, asks for all of
+// its keys and values at once and never meets a barrier or another wave. Which keys a chunk holds
+// does not depend on the sequence's length, so the page ids are asked for together with the
+// position, not after it: the chain of dependent memory accesses is page ids -> keys and values.
+// Chunks above the newest key (or below the window) end at once. The last chunk also takes
+// whatever lies above it (contexts longer than the launch was planned for). Each chunk leaves
+// (o, m, l) in partials[token][head][chunk]; attention_merge_range_kernel adds up the chunks a
+// sequence really has. A sequence that has one chunk only gets its finished output row here.
+// ---------------------------------------------------------------------------------------
+template <int D, bool FUSED, int BPW>
+__global__ void __launch_bounds__(64)
+attention_decode_wave_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
+                             const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+                             const int* __restrict__ block_table, int bt_width, int page_size,
+                             const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
+                             int H, int Hkv, float scale, int window, float* __restrict__ partials,
+                             int nchunks, FusedInput fz) {
+    constexpr int DS = D / 32;
+    constexpr int DT = D / 16;
+    const int G = H / Hkv;
+    const int kvh = blockIdx.y;
+    const int z = blockIdx.z;
+    const int lane = threadIdx.x;
+    const int i = lane % 16;
+    const int g = lane / 16;
+    const int tpu = 16 / G;
+
+    int seq = blockIdx.x, t0, nt;
+    if (FUSED) {
+        t0 = seq;
+        nt = fz.token_seq[t0] >= 0 ? 1 : 0;
+    } else {
+        const int first = cu_seqlens[seq];
+        int count = cu_seqlens[seq + 1] - first;
+        if (count > tpu) count = tpu;
+        t0 = first;
+        nt = count;
+    }
+    if (nt <= 0) return;
+    const int ncols = nt * G;
+    const int* bt = block_table + (size_t)seq * bt_width;
+
+    // the page ids of this chunk's 16-key tiles: asked for before anything is known about the length
+    const int b_first = z * BPW;
+    int pg[2 * BPW];
+#pragma unroll
+    for (int t = 0; t < 2 * BPW; ++t) {
+        const int pidx = (32 * b_first + 16 * t) / page_size;
+        pg[t] = pidx < bt_width ? bt[pidx] : -1;
+    }
+
+    // this lane's column
+    const bool col_ok = i < ncols;
+    const int col_tok = t0 + (col_ok ? i / G : 0);
+    const int col_head = kvh * G + (col_ok ? i % G : 0);
+    Frag qop[DS];
+    {
+        const bf16* qrow = FUSED ? fz.qkv + (size_t)col_tok * fz.stride + fz.q_off + (size_t)col_head * D + 8 * g
+                                 : q + (size_t)col_tok * q_stride + (size_t)col_head * D + 8 * g;
+#pragma unroll
+        for (int s = 0; s < DS; ++s) qop[s].u = col_ok ? *reinterpret_cast<const uint4*>(qrow + 32 * s) : uint4{0u, 0u, 0u, 0u};
+    }
+    const int col_pos = col_ok ? positions[FUSED ? t0 : col_tok] : -1;
+    const int col_lo = (window >= 0 && col_pos - window > 0) ? col_pos - window : 0;
+    int hi_w, lo_w;
+    if (FUSED) {
+        hi_w = positions[t0];
+        lo_w = (window >= 0 && hi_w - window > 0) ? hi_w - window : 0;
+    } else {
+        hi_w = wave_max_i(col_ok ? col_pos : -1);
+        lo_w = wave_min_i(col_ok ? col_lo : 0x7fffffff);
+    }
+    if (hi_w < 0) return;
+    const int b_lo = lo_w / 32, b_hi = hi_w / 32;            // the blocks the sequence has
+    const bool last_chunk = z == nchunks - 1;
+    int b_end = last_chunk ? b_hi + 1 : b_first + BPW;       // the last chunk takes what lies above it too
+    if (b_end > b_hi + 1) b_end = b_hi + 1;
+    const int b_begin = b_first > b_lo ? b_first : b_lo;
+    if (b_begin >= b_end) return;                            // no key of the sequence in this chunk
+    int z_lo = b_lo / BPW, z_hi = b_hi / BPW;
+    if (z_lo > nchunks - 1) z_lo = nchunks - 1;
+    if (z_hi > nchunks - 1) z_hi = nchunks - 1;
+    const bool alone = z_lo == z_hi;                         // the sequence's only chunk: finish the row here
+    const float sc_mul = scale * LOG2E;
+
+    __shared__ __attribute__((aligned(16))) float sh_const[FUSED ? 3 : 1][FUSED ? D : 1];
+    const int b_new = b_hi;
+    const bool owns_new = FUSED && fz.store && b_new >= b_begin && b_new < b_end;
+    Frag knew[DS], kraw[DS];
+    uint16_t vnew[DT];
+    if (FUSED) {
+        for (int d = lane; d < D; d += 64) {
+            if (fz.has_norm) {
+                sh_const[0][d] = fz.qw.at(d) + (fz.unit_offset ? 1.f : 0.f);
+                if (fz.kw.p != nullptr) sh_const[1][d] = fz.kw.at(d) + (fz.unit_offset ? 1.f : 0.f);
+            }
+            if (fz.table != nullptr) sh_const[2][d] = fz.table[(size_t)hi_w * D + d];
+        }
+#pragma unroll
+        for (int s = 0; s < DS; ++s) knew[s].u = kraw[s].u = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vnew[dt] = 0;
+        if (owns_new) {
+            const bf16* row = fz.qkv + (size_t)t0 * fz.stride;
+            const bf16* krow = row + fz.k_off + (size_t)kvh * D + 8 * g;
+#pragma unroll
+            for (int s = 0; s < DS; ++s) kraw[s].u = *reinterpret_cast<const uint4*>(krow + 32 * s);
+            const uint16_t* vrow = reinterpret_cast<const uint16_t*>(row + fz.v_off + (size_t)kvh * D);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vnew[dt] = vrow[16 * dt + i];
+        }
+    }
+
+    struct Operands {
+        int page[2];
+        Frag k[2][DS];
+        Frag v[DT];
+    };
+    auto fetch = [&](int b, int page0, int page1, Operands& op) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int key0 = 32 * b + 16 * t;
+            const int pidx = key0 / page_size;
+            const int slot0 = key0 - pidx * page_size;
+            const int page = (b >= b_begin && b < b_end && key0 <= hi_w) ? (t == 0 ? page0 : page1) : -1;
+            op.page[t] = page;
+            if (page >= 0) {
+                const size_t head = (size_t)page * Hkv + kvh;
+                const bf16* kptr = k_pages + ((head * page_size + slot0 + i) * D + 8 * g);
+#pragma unroll
+                for (int s = 0; s < DS; ++s) op.k[t][s].u = *reinterpret_cast<const uint4*>(kptr + 32 * s);
+                const bf16* vptr = v_pages + (head * D + i) * page_size + slot0 + 4 * g;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    op.v[dt].h[t] = *reinterpret_cast<const uint2*>(vptr + (size_t)16 * dt * page_size);
+            } else {
+#pragma unroll
+                for (int s = 0; s < DS; ++s) op.k[t][s].u = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) op.v[dt].h[t] = uint2{0u, 0u};
+            }
+        }
+    };
+
+    float m_run = -INFINITY, l_run = 0.f;
+    floatx4_t acc_o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](int b, Operands& op) {
+        const int base = 32 * b;
+        if (FUSED && owns_new && b == b_new) {   // the newest key and value come from the registers
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (base + 16 * t + i == hi_w) {
+#pragma unroll
+                    for (int s = 0; s < DS; ++s) op.k[t][s] = knew[s];
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (base + 16 * t + 4 * g + r == hi_w) {
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) op.v[dt].s[t * 4 + r] = vnew[dt];
+                    }
+            }
+        }
+        float p[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+            if (op.page[t] >= 0) {
+#pragma unroll
+                for (int s = 0; s < DS; ++s)
+                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.k[t][s].v, qop[s].v, sacc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = base + 16 * t + 4 * g + r;
+                const bool ok = op.page[t] >= 0 && col_ok && key <= col_pos && key >= col_lo;
+                p[t][r] = ok ? sacc[r] * sc_mul : -INFINITY;
+            }
+        }
+        Frag pop;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mx = fmaxf(mx, p[t][r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
+        float psum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = __builtin_amdgcn_exp2f(p[t][r] - m_safe);
+                psum += e;
+                pop.v[t * 4 + r] = (__bf16)e;
+            }
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc_o[dt] *= corr;
+        if (base + 31 > hi_w) {  // slots above the newest key were never written
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (base + 16 * t + 4 * g + r > hi_w) op.v[dt].s[t * 4 + r] = 0;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.v[dt].v, pop.v, acc_o[dt], 0, 0, 0);
+    };
+
+    // all keys and values of the chunk are asked for at once
+    Operands ops[BPW];
+#pragma unroll
+    for (int j = 0; j < BPW; ++j) fetch(b_first + j, pg[2 * j], pg[2 * j + 1], ops[j]);
+    if (FUSED) {   // while those loads are in flight
+        __syncthreads();                          // (one wave: the constants are in LDS)
+        const float* cs = fz.table != nullptr ? sh_const[2] : nullptr;
+        norm_rotate<DS>(qop, g, fz.has_norm ? sh_const[0] : nullptr, fz.eps, cs, D, qop);
+        if (owns_new) {
+            norm_rotate<DS>(kraw, g, fz.has_norm ? sh_const[1] : nullptr, fz.eps, cs, D, knew);
+            const int pidx = hi_w / page_size;
+            const int page = pidx < bt_width ? bt[pidx] : -1;
+            if (page >= 0) {
+                const int slot = hi_w % page_size;
+                const size_t head = (size_t)page * Hkv + kvh;
+                if (i == 0) {
+                    bf16* kdst = const_cast<bf16*>(k_pages) + ((head * page_size + slot) * D + 8 * g);
+#pragma unroll
+                    for (int s = 0; s < DS; ++s) *reinterpret_cast<uint4*>(kdst + 32 * s) = knew[s].u;
+                }
+                if (g == 0) {
+                    uint16_t* vdst = reinterpret_cast<uint16_t*>(const_cast<bf16*>(v_pages)) + (head * D + i) * page_size + slot;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) vdst[(size_t)16 * dt * page_size] = vnew[dt];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < BPW; ++j) compute(b_first + j, ops[j]);
+    // (the last chunk of a launch planned for shorter contexts: the blocks above it, one after the other)
+    for (int b = b_first + BPW; b < b_end; ++b) {
+        const int p0 = (32 * b) / page_size, p1 = (32 * b + 16) / page_size;
+        fetch(b, p0 < bt_width ? bt[p0] : -1, p1 < bt_width ? bt[p1] : -1, ops[0]);
+        compute(b, ops[0]);
+    }
+
+    l_run += __shfl_xor(l_run, 16, MV_WAVE);
+    l_run += __shfl_xor(l_run, 32, MV_WAVE);
+    if (!col_ok) return;
+    if (alone) {
+        bf16* orow = out + (size_t)col_tok * out_stride + (size_t)col_head * D;
+        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            uint2 packed;
+            packed.x = f32x2_to_bf16x2_bits(acc_o[dt][0] * inv, acc_o[dt][1] * inv);
+            packed.y = f32x2_to_bf16x2_bits(acc_o[dt][2] * inv, acc_o[dt][3] * inv);
+            *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = packed;
+        }
+        return;
+    }
+    float* prow = partials + (((size_t)col_tok * H + col_head) * nchunks + z) * (D + 2);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+        *reinterpret_cast<float4*>(prow + 16 * dt + 4 * g) = float4{acc_o[dt][0], acc_o[dt][1], acc_o[dt][2], acc_o[dt][3]};
+    if (g == 0) {
+        prow[D] = m_run;
+        prow[D + 1] = l_run;
+    }
+}
+
+// Adds up the chunks that attention_decode_wave_kernel left for a token: those between the chunk
+// of the first key its query sees and the chunk of its own position. A token with a single chunk
+// has its row already. One workgroup of D threads per (token, head).
+template <int BPW>
+__global__ void attention_merge_range_kernel(const float* __restrict__ partials, bf16* __restrict__ out, long out_stride,
+                                             const int* __restrict__ token_seq, const int* __restrict__ positions,
+                                             const int* __restrict__ cu_seqlens, int fused,
+                                             int window, int H, int D, int nchunks) {
+    __shared__ float sh_m[64], sh_l[64];
+    const int head = blockIdx.y;
+    const int d = threadIdx.x;            // blockDim.x == D
+    // the sequence's token: row blockIdx.x of a step of one token a sequence (fused: padding rows
+    // are rows too and get zeros), else the first token of sequence blockIdx.x, if it has one
+    int tok = blockIdx.x;
+    if (!fused) {
+        tok = cu_seqlens[blockIdx.x];
+        if (cu_seqlens[blockIdx.x + 1] - tok <= 0) return;
+    }
+    bf16* orow = out + (size_t)tok * out_stride + (size_t)head * D;
+    if (token_seq[tok] < 0) {
+        orow[d] = from_f<bf16>(0.f);
+        return;
+    }
+    const int hi = positions[tok];
+    const int lo = (window >= 0 && hi - window > 0) ? hi - window : 0;
+    int z_lo = (lo / 32) / BPW, z_hi = (hi / 32) / BPW;
+    if (z_lo > nchunks - 1) z_lo = nchunks - 1;
+    if (z_hi > nchunks - 1) z_hi = nchunks - 1;
+    if (z_lo == z_hi) return;             // the attention kernel finished this row itself
+    const int nz = z_hi - z_lo + 1;
+    const float* base = partials + (((size_t)tok * H + head) * nchunks + z_lo) * (D + 2);
+    float m_run = -INFINITY, l_run = 0.f, a = 0.f;
+    for (int z0 = 0; z0 < nz; z0 += 64) {             // batches of 64 chunks, merged as they come
+        const int n = nz - z0 < 64 ? nz - z0 : 64;
+        const float* bz = base + (size_t)z0 * (D + 2);
+        float pre[8];                                  // asked for before the weights are known
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pre[j] = j < n ? bz[(size_t)j * (D + 2) + d] : 0.f;
+        __syncthreads();
+        if (d < n) {
+            sh_m[d] = bz[(size_t)d * (D + 2) + D];
+            sh_l[d] = bz[(size_t)d * (D + 2) + D + 1];
+        }
+        __syncthreads();
+        float mb = -INFINITY;
+        for (int j = 0; j < n; ++j) mb = fmaxf(mb, sh_m[j]);
+        const float m_new = fmaxf(m_run, mb);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = exp2f(m_run - m_safe);     // exp2(-inf) = 0
+        a *= corr;
+        l_run *= corr;
+        m_run = m_new;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (j < n) {
+                const float w = exp2f(sh_m[j] - m_safe);
+                l_run += w * sh_l[j];
+                a += w * pre[j];
+            }
+#pragma unroll 4
+        for (int j = 8; j < n; ++j) {
+            const float w = exp2f(sh_m[j] - m_safe);
+            l_run += w * sh_l[j];
+            a += w * bz[(size_t)j * (D + 2) + d];
+        }
+    }
+    orow[d] = from_f<bf16>(l_run > 0.f ? a / l_run : 0.f);
+}
+
 // Merges the partial results of the key splits: out[token][head] = sum_z o_z 2^(m_z - m) / l.
 #define AF_MAX_SPLITS 64
 __global__ void attention_merge_kernel(const float* __restrict__ partials, bf16* __restrict__ out, long out_stride,
-                                       const int* __restrict__ token_seq, int H, int D, int nsplit) {
+                                       const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens, int fused,
+                                       int H, int D, int nsplit) {
     __shared__ float sh_m[AF_MAX_SPLITS], sh_w[AF_MAX_SPLITS];
-    const int tok = blockIdx.x, head = blockIdx.y;
+    const int head = blockIdx.y;
+    int tok = blockIdx.x;        // fused: row blockIdx.x of a step of one token a sequence; else the sequence's token
+    if (!fused) {
+        tok = cu_seqlens[blockIdx.x];
+        if (cu_seqlens[blockIdx.x + 1] - tok <= 0) return;
+    }
     bf16* orow = out + (size_t)tok * out_stride + (size_t)head * D;
     if (token_seq[tok] < 0) {
         for (int d = threadIdx.x; d < D; d += blockDim.x) orow[d] = from_f<bf16>(0.f);
@@ -550,9 +909,41 @@ static int check_common(const char* what, long q_stride, long out_stride, int pa
 static int decode_common(bool fused, const FusedInput& fz, const void* q, long q_stride, void* out, long out_stride,
                          const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                          int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
-                         float scale, int window, float* partials, int nsplit, int waves, const int* token_seq,
-                         hipStream_t stream) {
+                         float scale, int window, float* partials, int nsplit, int waves, int chunk_keys,
+                         const int* token_seq, hipStream_t stream) {
     MV_REQUIRE(H / Hkv <= 16, "attention_decode: %d query heads per kv head exceed 16", H / Hkv);
+    if (chunk_keys != 0) {
+        // one wave per chunk of chunk_keys keys; nsplit chunks are planned for every sequence
+        MV_REQUIRE(chunk_keys == 64 || chunk_keys == 128, "attention_decode: chunks of %d keys (64 or 128)", chunk_keys);
+        MV_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || partials != nullptr),
+                   "attention_decode: bad chunk count %d or missing work area", nsplit);
+        if (n_seqs <= 0) return 0;
+        dim3 grid(n_seqs, Hkv, nsplit);
+#define AF_WAVE(DD, FF, BB)                                                                                          \
+        hipLaunchKernelGGL((attention_decode_wave_kernel<DD, FF, BB>), grid, dim3(64), 0, stream, (const bf16*)q, q_stride, \
+                           (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,  \
+                           page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit, fz)
+        if (D == 128 && fused && chunk_keys == 64) AF_WAVE(128, true, 2);
+        else if (D == 128 && fused) AF_WAVE(128, true, 4);
+        else if (D == 128 && chunk_keys == 64) AF_WAVE(128, false, 2);
+        else if (D == 128) AF_WAVE(128, false, 4);
+        else if (fused && chunk_keys == 64) AF_WAVE(64, true, 2);
+        else if (fused) AF_WAVE(64, true, 4);
+        else if (chunk_keys == 64) AF_WAVE(64, false, 2);
+        else AF_WAVE(64, false, 4);
+#undef AF_WAVE
+        if (int rc = mv_check_launch("attention_decode (one wave a chunk)")) return rc;
+        if (nsplit > 1) {
+            if (chunk_keys == 64)
+                hipLaunchKernelGGL(attention_merge_range_kernel<2>, dim3(n_seqs, H), dim3(D), 0, stream, partials, (bf16*)out,
+                                   out_stride, token_seq, positions, cu_seqlens, fused ? 1 : 0, window, H, D, nsplit);
+            else
+                hipLaunchKernelGGL(attention_merge_range_kernel<4>, dim3(n_seqs, H), dim3(D), 0, stream, partials, (bf16*)out,
+                                   out_stride, token_seq, positions, cu_seqlens, fused ? 1 : 0, window, H, D, nsplit);
+            return mv_check_launch("attention_merge (chunks)");
+        }
+        return 0;
+    }
     MV_REQUIRE(nsplit >= 1 && nsplit <= AF_MAX_SPLITS && (nsplit == 1 || partials != nullptr),
                "attention_decode: bad split count %d or missing work area", nsplit);
     MV_REQUIRE(waves == 4 || waves == 8, "attention_decode: %d waves per workgroup (4 or 8)", waves);
@@ -592,7 +983,7 @@ static int decode_common(bool fused, const FusedInput& fz, const void* q, long q
     if (int rc = mv_check_launch("attention_decode")) return rc;
     if (nsplit > 1) {
         hipLaunchKernelGGL(attention_merge_kernel, dim3(n_seqs, H), dim3(D >= 128 ? 128 : 64), 0, stream, partials,
-                           (bf16*)out, out_stride, token_seq, H, D, nsplit);
+                           (bf16*)out, out_stride, token_seq, cu_seqlens, fused ? 1 : 0, H, D, nsplit);
         return mv_check_launch("attention_merge");
     }
     return 0;
@@ -600,15 +991,19 @@ static int decode_common(bool fused, const FusedInput& fz, const void* q, long q
 
 // Decode steps: every sequence brings one token. grid = (sequences, kv heads, nsplit); `waves` (4
 // or 8) per workgroup. partials: float [n_seqs * H * nsplit * (D + 2)], needed when nsplit > 1.
+// chunk_keys != 0 (64 or 128) selects the one-wave variant for small grids instead: a wave per
+// chunk of that many keys, nsplit chunks planned per sequence (nsplit * chunk_keys should cover the
+// longest context; the last chunk takes what lies above), `waves` is ignored; `positions` must then
+// hold, for a step of one token a sequence, token t's position at index t.
 extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
                                    const void* v_pages, const int* block_table, int bt_width, int page_size,
                                    const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
-                                   float scale, int window, float* partials, int nsplit, int waves,
+                                   float scale, int window, float* partials, int nsplit, int waves, int chunk_keys,
                                    const int* token_seq, hipStream_t stream) {
     if (int rc = check_common("attention_decode", q_stride, out_stride, page_size, bt_width, H, Hkv, D)) return rc;
     return decode_common(false, FusedInput{}, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,
                          page_size, positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, partials, nsplit, waves,
-                         token_seq, stream);
+                         chunk_keys, token_seq, stream);
 }
 
 // The same for a decode step whose queries, keys and values are still the raw rows of the
@@ -622,7 +1017,8 @@ extern "C" int mv_attention_decode_fused(const void* qkv, long qkv_stride, int q
                                          int n_seqs, int H, int Hkv, int D, float scale, int window,
                                          const void* q_weight, const void* k_weight, int weight_dtype, float eps,
                                          int unit_offset, const float* table, int store_kv, float* partials,
-                                         int nsplit, int waves, const int* token_seq, hipStream_t stream) {
+                                         int nsplit, int waves, int chunk_keys, const int* token_seq,
+                                         hipStream_t stream) {
     if (int rc = check_common("attention_decode_fused", qkv_stride, out_stride, page_size, bt_width, H, Hkv, D))
         return rc;
     MV_REQUIRE(qkv != nullptr && ((uintptr_t)qkv % 16) == 0 && q_off % 8 == 0 && k_off % 8 == 0 && v_off >= 0,
@@ -639,6 +1035,6 @@ extern "C" int mv_attention_decode_fused(const void* qkv, long qkv_stride, int q
     FusedInput fz{(const bf16*)qkv, qkv_stride, q_off, k_off, v_off, WeightPtr{q_weight, weight_dtype},
                   WeightPtr{k_weight, weight_dtype}, has_norm, eps, unit_offset, table, store_kv ? 1 : 0, token_seq};
     return decode_common(true, fz, nullptr, 0, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size,
-                         positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, partials, nsplit, waves, token_seq,
-                         stream);
+                         positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, partials, nsplit, waves, chunk_keys,
+                         token_seq, stream);
 }

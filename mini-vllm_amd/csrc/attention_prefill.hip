@@ -525,10 +525,8 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             uint2 packed;
-            packed.x = (uint32_t)f32_to_bf16_bits(acc_o[ct][dt][0] * inv) |
-                       ((uint32_t)f32_to_bf16_bits(acc_o[ct][dt][1] * inv) << 16);
-            packed.y = (uint32_t)f32_to_bf16_bits(acc_o[ct][dt][2] * inv) |
-                       ((uint32_t)f32_to_bf16_bits(acc_o[ct][dt][3] * inv) << 16);
+            packed.x = f32x2_to_bf16x2_bits(acc_o[ct][dt][0] * inv, acc_o[ct][dt][1] * inv);
+            packed.y = f32x2_to_bf16x2_bits(acc_o[ct][dt][2] * inv, acc_o[ct][dt][3] * inv);
             *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = packed;
         }
     }

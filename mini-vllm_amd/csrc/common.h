@@ -21,11 +21,22 @@ enum MvDtype { MV_F32 = 0, MV_BF16 = 1 };
 __device__ __forceinline__ float to_f(float v) { return v; }
 __device__ __forceinline__ float to_f(bf16 v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
 
+// float -> bf16, round to nearest even: gfx950 has the conversion in hardware (v_cvt_pk_bf16_f32,
+// two values an instruction), which is what these casts compile to. A wave issues about one
+// instruction every four cycles, so a rounding written out in integer instructions (five or six
+// per value) is what small kernels spend their time on.
+typedef __bf16 mv_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float mv_floatx2_t __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);                                               // nearest even
-    return (uint16_t)(u >> 16);
+    const __bf16 h = (__bf16)f;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+// two values in one 32-bit word: a in the low half, b in the high half
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float a, float b) {
+    const mv_bf16x2_t h = __builtin_convertvector(mv_floatx2_t{a, b}, mv_bf16x2_t);
+    return __builtin_bit_cast(uint32_t, h);
 }
 
 template <typename T> __device__ __forceinline__ T from_f(float f);

@@ -43,7 +43,7 @@ template <> struct Vec8<bf16> {
         uint32_t w[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            w[e] = (uint32_t)f32_to_bf16_bits(x[2 * e]) | ((uint32_t)f32_to_bf16_bits(x[2 * e + 1]) << 16);
+            w[e] = f32x2_to_bf16x2_bits(x[2 * e], x[2 * e + 1]);
         *reinterpret_cast<uint4*>(p) = uint4{w[0], w[1], w[2], w[3]};
     }
 };

@@ -30,6 +30,12 @@ union Frag {
 #define SK_STAGE_FRAGS 8    // 16-byte operand loads per lane in one register stage of the main loop
 #endif
 #define SK_NORM_CHUNKS 4   // chunks of 512 columns a wave holds in the fused norm's prologue
+#ifndef SK_MIN_ROWS
+#define SK_MIN_ROWS 8      // fewest output columns of a workgroup
+#endif
+#ifndef SK_WAVE_K
+#define SK_WAVE_K 128      // fewest K elements of a wave
+#endif
 
 template <typename TC> __device__ __forceinline__ void store_c(TC* p, float v);
 template <> __device__ __forceinline__ void store_c<float>(float* p, float v) { *p = v; }
@@ -355,7 +361,7 @@ static int skinny_blocks(int N, int rows) { return (N + rows - 1) / rows; }
 static int pick_rows(int N, int most) {
     int rows = most;
     long best = -1;
-    for (int p = most; p >= 8; p -= 4) {
+    for (int p = most; p >= SK_MIN_ROWS; p -= 4) {
         const long wgs = (N + p - 1) / p;
         const long cost = ((wgs + SK_COMPUTE_UNITS - 1) / SK_COMPUTE_UNITS) * p;
         if (best < 0 || cost < best) {
@@ -390,7 +396,7 @@ static void launch_skinny_norm(const NormInput& norm, const void* W, const void*
 }
 
 static int pick_waves(int K) {
-    int s = K / 128;  // at least four MFMA steps per wave
+    int s = K / SK_WAVE_K;  // at least four MFMA steps per wave
     if (s < 1) s = 1;
     if (s > SK_MAX_WAVES) s = SK_MAX_WAVES;
     return s;

@@ -61,6 +61,9 @@ class AttentionPlan:
     q_lens: Sequence[int] = ()     # tokens per sequence, on the host
     cu_seqlens: Optional[torch.Tensor] = None   # int32 [n_seqs + 1] on the device
     workspace: Optional[object] = None          # where kernels take scratch memory from
+    # decode steps: None lets the launch heuristic choose between the one-wave kernel (chunks of 64 or
+    # 128 keys) and the workgroup kernel (0); a test may force one
+    decode_chunk_keys: Optional[int] = None
 
 
 class StepContext:

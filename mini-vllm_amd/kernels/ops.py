@@ -52,6 +52,9 @@ COMPUTE_UNITS = 256
 PREFILL_TWO_GROUPS_FROM = 1024
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
+# most waves in the grid of the one-wave decode attention (a wave per chunk of keys); above that the
+# workgroup kernel with its pipeline over the keys serves the step
+DECODE_WAVE_GRID = 4096
 # from this many tokens on, value rows are written to their pages 16 tokens of a kv head at a time
 STORE_V_SPLIT_TOKENS = 64
 
@@ -580,19 +583,31 @@ class Ops:
                       float(scale), w, self.code, self._stream())
 
     def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int):
-        """How many workgroups share a sequence's keys in a decode step, and their work area.
+        """How a decode step's keys are dealt out: (nsplit, partials, chunk_keys).
 
-        The keys are split until about 256 workgroups are in flight, but never below 128 keys per
-        split (measured on MI355X with 8 kv heads: batch 1 is fastest at 8 to 16 splits, batch 8 at
-        4, batch 64 without a split). The count is a property of the plan (a captured graph keeps
-        it); each split takes its share of the keys a sequence actually has."""
+        Small grids (few sequences) take the one-wave kernel: a wave per chunk of 64 or 128 keys of a
+        (sequence, kv head) pair, as many chunks as the planned context length has, all of a chunk's
+        keys in flight at once; chunk_keys is 64 or 128 then and nsplit the number of chunks. The grid
+        may hold up to DECODE_WAVE_GRID waves (chunks above a sequence's newest key end at once).
+
+        Larger grids take the workgroup kernel (chunk_keys 0): the keys are split until about 256
+        workgroups are in flight, but never below 128 keys per split (measured on MI355X with 8 kv
+        heads: batch 64 is fastest without a split). The count is a property of the plan (a captured
+        graph keeps it); each split takes its share of the keys a sequence actually has."""
         ctx = max(1, plan.max_context_len)
+        forced = getattr(plan, "decode_chunk_keys", None)
+        for chunk in (64, 128):
+            nchunks = -(-ctx // chunk)
+            if forced == chunk or (forced is None and n_seqs * Hkv * nchunks <= DECODE_WAVE_GRID):
+                rows = max(n_seqs * nchunks, DECODE_WAVE_GRID // max(1, Hkv))      # one size serves every graph
+                partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
+                return nchunks, partials, chunk
         nsplit = max(1, min(256 // max(1, n_seqs * Hkv), max(1, ctx // 128), 64))
         partials = None
         if nsplit > 1:
             rows = max(n_seqs * nsplit, 2048 // Hkv, 256)      # one size serves every batch of a graph set
             partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
-        return nsplit, partials
+        return nsplit, partials, 0
 
     def attention_decode_fused(self, qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor,
                                v_pages: torch.Tensor, block_table: torch.Tensor, page_size: int,
@@ -641,13 +656,13 @@ class Ops:
         _dev(block_table, "block table")
         if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
             raise KernelLibraryError("attention: the block table must be a contiguous int32 matrix")
-        nsplit, partials = self._decode_split(plan, n, H, Hkv, D)
+        nsplit, partials, chunk_keys = self._decode_split(plan, n, H, Hkv, D)
         self.lib.call("mv_attention_decode_fused", qkv.data_ptr(), stride, 0, H * D, (H + Hkv) * D, out.data_ptr(), os_,
                       k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n, H, Hkv, D, float(scale),
                       -1 if window is None else int(window), _ptr(q_weight), _ptr(k_weight), wcode, float(eps),
                       int(unit_offset), _ptr(rope_table), int(store_kv), _ptr(partials), nsplit,
-                      DECODE_ATTENTION_WAVES, token_seq.data_ptr(), self._stream())
+                      DECODE_ATTENTION_WAVES, chunk_keys, token_seq.data_ptr(), self._stream())
         return True
 
     def _attention_fast(self, q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
@@ -660,11 +675,12 @@ class Ops:
         group = H // Hkv
         n_seqs = plan.n_seqs
         if plan.decode_only and group <= 16:
-            nsplit, partials = self._decode_split(plan, n_seqs, H, Hkv, D)
+            nsplit, partials, chunk_keys = self._decode_split(plan, n_seqs, H, Hkv, D)
             self.lib.call("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
-                          _ptr(partials), nsplit, DECODE_ATTENTION_WAVES, token_seq.data_ptr(), self._stream())
+                          _ptr(partials), nsplit, DECODE_ATTENTION_WAVES, chunk_keys, token_seq.data_ptr(),
+                          self._stream())
             return True
         if page_size & (page_size - 1):
             return False

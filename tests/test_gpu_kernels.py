@@ -400,9 +400,13 @@ def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window, ctx_lens, q
 @pytest.mark.parametrize("H,Hkv,D,ps,window", [(16, 8, 128, 16, None), (8, 1, 128, 32, None), (6, 2, 64, 16, 50),
                                                 (16, 1, 64, 16, None)])
 @pytest.mark.parametrize("max_context", [None, 4096, 40000])
-def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
-    """Decode steps on the MFMA kernel: one token per sequence at very different context
-    lengths, a padding sequence in the middle, keys split over 1, a few and many workgroups."""
+@pytest.mark.parametrize("chunk_keys", [0, 64, 128])
+def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context, chunk_keys):
+    """Decode steps on the MFMA kernels: one token per sequence at very different context
+    lengths, a padding sequence in the middle; the workgroup kernel (chunk_keys 0) with its keys
+    split over 1, a few and many workgroups, and the one-wave kernel with chunks of 64 and 128 keys,
+    planned for the longest context, for a longer one, and (None) for a shorter one than the
+    sequences really have: the last chunk then takes what lies above it."""
     ops = ops_for(torch.bfloat16)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(16)
@@ -436,7 +440,9 @@ def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context):
     q = q.to(dtype)
     scale = 1.0 / math.sqrt(D)
     out = torch.empty(n, H * D, dtype=dtype, device="cuda")
-    plan = make_plan(q_lens, ctx_lens, max_context_len=max_context)
+    plan = make_plan(q_lens, ctx_lens, max_context_len=max_context if max_context else (200 if chunk_keys else None),
+                     decode_only=True)
+    plan.decode_chunk_keys = chunk_keys
     ops.attention(dev(q.view(n, H * D)), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale,
                   window, plan=plan)
     want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
@@ -521,7 +527,7 @@ def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
     cu = dev(torch.tensor([0, 1], dtype=torch.int32))
     seq0 = dev(torch.zeros(1, dtype=torch.int32))
     ops.lib.call("mv_attention_decode", qd.data_ptr(), H * D, out.data_ptr(), H * D, kp.data_ptr(), vp.data_ptr(),
-                 bt.data_ptr(), pages, ps, pos.data_ptr(), cu.data_ptr(), 1, H, Hkv, D, D ** -0.5, -1, 0, 1, 4,
+                 bt.data_ptr(), pages, ps, pos.data_ptr(), cu.data_ptr(), 1, H, Hkv, D, D ** -0.5, -1, 0, 1, 4, 0,
                  seq0.data_ptr(), ops._stream())
     torch.cuda.synchronize()
     want = reference_attention(q.double(), k_all, v_all, torch.tensor([ctx - 1]), torch.tensor([0]), H, Hkv, D ** -0.5, None)
@@ -533,7 +539,8 @@ def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
 @pytest.mark.parametrize("with_norm,with_rope,store", [(True, True, True), (False, True, True), (True, False, True),
                                                        (True, True, False)])
 @pytest.mark.parametrize("max_context", [None, 40000])
-def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_rope, store, max_context):
+@pytest.mark.parametrize("chunk_keys", [0, 64, 128])
+def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_rope, store, max_context, chunk_keys):
     """A decode step from the raw [q | k | v] rows: per-head norm, rotation, cache write and attention
     in one kernel. The slot of the new position holds NaN before (unless the cache is another
     layer's and already complete), the finished key and value afterwards."""
@@ -599,7 +606,9 @@ def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_ro
     # as in the engine's padded decode steps: one row per sequence of the plan, padding at the end
     # (a sequence without a token, a row that belongs to no sequence)
     out = torch.full((n + 1, H * D), float("nan"), dtype=dtype, device="cuda")
-    plan = make_plan([1] * n + [0], [ctx_lens[s] for s in live], max_context_len=max_context, decode_only=True)
+    plan = make_plan([1] * n + [0], [ctx_lens[s] for s in live],
+                     max_context_len=max_context if max_context else (200 if chunk_keys == 64 else None), decode_only=True)
+    plan.decode_chunk_keys = chunk_keys
     rows = raw if store else raw[:, :H * D].contiguous()
     qkv = dev(torch.cat([rows, torch.full((1, rows.shape[1]), float("nan"), dtype=dtype)]))
     bt_rows = torch.cat([bt[live], torch.full((1, bt.shape[1]), -1, dtype=torch.int32)]).contiguous()
