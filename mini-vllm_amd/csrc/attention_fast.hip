@@ -494,278 +494,446 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
 // ---------------------------------------------------------------------------------------
 // The one-wave variant, for steps whose grid is small (few sequences): a workgroup is a single
 // wave that takes a fixed chunk of 32 * BPW keys of one (sequence, kv head) pair, asks for all of
-// its keys and values at once and never meets a barrier or another wave. Which keys a chunk holds
-// does not depend on the sequence's length, so the page ids are asked for together with the
-// position, not after it: the chain of dependent memory accesses is page ids -> keys and values.
+// its keys and values at once and never meets a barrier or another wave. It is written for few
+// instructions on the wave's path (a wave issues one instruction in about four cycles, so a
+// thousand instructions are two microseconds whatever the memory does):
+//   * which keys a chunk holds does not depend on the sequence's length, so the page ids are
+//     asked for together with the position, not after it;
+//   * the scores of the whole chunk are made first, one maximum is taken over them, and the
+//     values are added up under that maximum: no rescaling between blocks;
+//   * tiles wholly inside the visible range skip the masks; the tile of the newest key takes the
+//     mask, the clearing of slots that were never written and (fused) the new key and value;
+//   * the query is scaled by scale * log2(e) once, where it is normalised (fused);
+//   * lanes whose column is no head of the group work on a copy of the last head and store nothing.
 // Chunks above the newest key (or below the window) end at once. The last chunk also takes
-// whatever lies above it (contexts longer than the launch was planned for). Each chunk leaves
-// (o, m, l) in partials[token][head][chunk]; attention_merge_range_kernel adds up the chunks a
-// sequence really has. A sequence that has one chunk only gets its finished output row here.
+// whatever lies above it (contexts longer than the launch was planned for), chunk after chunk with
+// the usual rescaling. Each chunk leaves (o, m, l) in partials[token][head][chunk];
+// attention_merge_range_kernel adds up the chunks a sequence really has. A sequence that has one
+// chunk only gets its finished output row here. One token a sequence; the page size is a power of two.
 // ---------------------------------------------------------------------------------------
-template <int D, bool FUSED, int BPW>
+template <int DS>
+__device__ __forceinline__ void prepare_head(const Frag (&raw)[DS], int g, const WeightPtr& w, int has_norm, int unit_offset,
+                                             float eps, const float* cs, float post_scale, int D, Frag (&dst)[DS]) {
+    // the lane's 8 * DS elements of a head (d = 32 s + 8 g + e): RMSNorm over the head (the four lane
+    // groups hold it between them), rotation by the table row cs = cat(cos, sin) (pairs d, d + D/2: the
+    // same lane, DS/2 groups further), a scale, and rounding to the operand type. `w` and
+    // `post_scale` may differ from lane to lane (a column that holds a key beside the query heads).
+    // The norm's factor and the scale are one number per lane; it goes into the cosines and sines
+    // where there is a rotation (which is linear), else into the weights.
+    float x[DS][8];
+#pragma unroll
+    for (int s = 0; s < DS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[s][e] = (float)raw[s].v[e];
+    float factor = post_scale;
+    if (has_norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < DS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += x[s][e] * x[s][e];
+        ss += __shfl_xor(ss, 16, MV_WAVE);
+        ss += __shfl_xor(ss, 32, MV_WAVE);
+        factor *= rsqrtf(ss / (float)D + eps);
+        const float uo = unit_offset ? 1.f : 0.f;
+#pragma unroll
+        for (int s = 0; s < DS; ++s) {
+            float wt[8];
+            w.at8(32 * s + 8 * g, wt);
+            if (cs != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[s][e] *= wt[e] + uo;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[s][e] *= (wt[e] + uo) * factor;
+            }
+        }
+    }
+    if (cs != nullptr) {
+        constexpr int HS = DS / 2;
+#pragma unroll
+        for (int s = 0; s < HS; ++s) {
+            const float4 c0 = *reinterpret_cast<const float4*>(cs + 32 * s + 8 * g);
+            const float4 c1 = *reinterpret_cast<const float4*>(cs + 32 * s + 8 * g + 4);
+            const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2 + 32 * s + 8 * g);
+            const float4 s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 32 * s + 8 * g + 4);
+            const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float cc = c[e] * factor, sc = sn[e] * factor;
+                const float a = x[s][e], b = x[s + HS][e];
+                x[s][e] = a * cc - b * sc;
+                x[s + HS][e] = b * cc + a * sc;
+            }
+        }
+    } else if (!has_norm && post_scale != 1.f) {
+#pragma unroll
+        for (int s = 0; s < DS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[s][e] *= post_scale;
+    }
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+        dst[s].u.x = f32x2_to_bf16x2_bits(x[s][0], x[s][1]);
+        dst[s].u.y = f32x2_to_bf16x2_bits(x[s][2], x[s][3]);
+        dst[s].u.z = f32x2_to_bf16x2_bits(x[s][4], x[s][5]);
+        dst[s].u.w = f32x2_to_bf16x2_bits(x[s][6], x[s][7]);
+    }
+}
+
+// Rows of the two 16-key score tiles of a 32-key block are bound to keys so that a lane ends up
+// with eight neighbouring keys: tile tt, row rho  <->  key 8 * (rho / 4) + 4 * tt + rho % 4 of the
+// block. After the first product lane (column, g) holds the scores of keys 8g .. 8g+7 (tile 0:
+// 8g .. 8g+3, tile 1: 8g+4 .. 8g+7), which are the eight k-slots of its operand in the second
+// product, and the value operand of a lane is one 16-byte load from the transposed page.
+//
+// What a wave does with its chunk. EDGE: the chunk touches an end of the visible range (it holds the
+// newest key, or keys below a window's lower end, or it is the last chunk of a plan that is shorter
+// than the sequence); only then are there masks, slots to clear, the new key and value, and more
+// rounds than one. Chunks wholly inside the range take the other instantiation, which has none of
+// that code. The order of the phases is pinned (keys asked for, query finished, values asked for,
+// scores, sum): it keeps the registers in use below what a lane has, and the query's arithmetic
+// runs while the keys are on their way.
+struct WaveChunk {
+    const bf16* k_pages;
+    const bf16* v_pages;
+    const int* bt;
+    int bt_width, page_size, page_shift, Hkv, kvh, z, nchunks, pos, lo, b_hi;
+    int i, g;
+    float sc_mul;
+    bool owns_new;
+    int kcol;          // the query operand's column in which the new key rides (16: none)
+    int t0;
+    const float* cs;
+};
+
+template <int D, bool FUSED, int BPW, bool PS16, bool EDGE>
+__device__ __forceinline__ void wave_chunk(const WaveChunk& c, const FusedInput& fz, Frag (&qop)[D / 32], int (&pga)[BPW],
+                                           int (&pgb)[BPW], float& m_run, float& l_run,
+                                           floatx4_t (&acc_o)[D / 16]) {
+    constexpr int DS = D / 32;
+    constexpr int DT = D / 16;
+    const int page_size = PS16 ? 16 : c.page_size;
+    const int page_shift = PS16 ? 4 : c.page_shift;
+    const int slot_mask = page_size - 1;
+    const int i = c.i, g = c.g, pos = c.pos, lo = c.lo;
+    const size_t page_elems = (size_t)c.Hkv * page_size * D;      // elements of one page of keys (or values)
+    // this lane's key rows of a block: tile tt, row i is key 8 * (i / 4) + 4 * tt + i % 4 of the block
+    const int krow0 = 8 * (i >> 2) + (i & 3);
+    const bf16* kbase = c.k_pages + (size_t)c.kvh * page_size * D + 8 * g;
+    const bf16* vbase = c.v_pages + ((size_t)c.kvh * D + i) * page_size;
+    const bool last_chunk = c.z == c.nchunks - 1;
+    // with the new key and value coming from the registers, their slot in the page counts as unwritten
+    const int pos_read = (EDGE && c.owns_new) ? pos - 1 : pos;
+
+    // The new key (EDGE, fused, the wave that meets the new position among its keys): its raw row has
+    // been loaded into the query operand's column `kcol`, a column that holds no query head, and is
+    // normalised and rotated there together with the queries, with the key's weights and no scale.
+    // (With sixteen query heads to a kv head there is no such column: the key is prepared by itself.)
+    const bool rides = EDGE && FUSED && c.owns_new && c.kcol < 16 && (!fz.has_norm || fz.kw.p != nullptr);
+    Frag knew[DS];
+    uint16_t vnew[DT];
+    if (EDGE && FUSED && c.owns_new) {   // the raw value of the new position (and the key, where it does not ride)
+        const bf16* row = fz.qkv + (size_t)c.t0 * fz.stride;
+        if (!rides) {
+            const bf16* krow = row + fz.k_off + (size_t)c.kvh * D + 8 * g;
+#pragma unroll
+            for (int s = 0; s < DS; ++s) knew[s].u = *reinterpret_cast<const uint4*>(krow + 32 * s);
+        }
+        const uint16_t* vrow = reinterpret_cast<const uint16_t*>(row + fz.v_off + (size_t)c.kvh * D);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vnew[dt] = vrow[16 * dt + i];
+    }
+
+    bool first = true;
+    for (int blk0 = BPW * c.z;; blk0 += BPW) {                 // one round, but for the last chunk of a short plan
+        if (EDGE && !first) {
+#pragma unroll
+            for (int j = 0; j < BPW; ++j) {
+                const int ia = (32 * (blk0 + j)) >> page_shift, ib = (32 * (blk0 + j) + 16) >> page_shift;
+                pga[j] = ia < c.bt_width ? c.bt[ia] : -1;
+                pgb[j] = ib < c.bt_width ? c.bt[ib] : -1;
+            }
+        }
+        // ---- the keys of the chunk are asked for at once
+        bool valid[BPW];
+        int pa[BPW], pb[BPW];
+        Frag kop[BPW][2][DS];
+#pragma unroll
+        for (int j = 0; j < BPW; ++j) {
+            const int key0 = 32 * (blk0 + j);
+            // a page that is not there (above the newest key, or given back by a window) holds only keys
+            // that are masked below: the lanes that would read it read the block's other page instead
+            pa[j] = (!EDGE || pga[j] >= 0) ? pga[j] : pgb[j];
+            pb[j] = (!EDGE || pgb[j] >= 0) ? pgb[j] : pga[j];
+            valid[j] = !EDGE || (pa[j] >= 0 && key0 <= pos && key0 + 31 >= lo);
+            if (valid[j]) {
+                const int pk = (PS16 && (i & 8)) ? pb[j] : pa[j];      // rows 8..15 of a tile are keys 16..31 of the block
+                const bf16* kptr = kbase + (size_t)pk * page_elems + (size_t)((key0 + krow0) & slot_mask) * D;
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int s = 0; s < DS; ++s)
+                        kop[j][tt][s].u = *reinterpret_cast<const uint4*>(kptr + (size_t)4 * tt * D + 32 * s);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (first && FUSED) {   // while the keys are on their way: the query (and the new key) are finished
+            if (rides) {
+                WeightPtr wl = fz.qw;
+                if (i == c.kcol && fz.kw.p != nullptr) wl.p = fz.kw.p;
+                prepare_head<DS>(qop, g, wl, fz.has_norm, fz.unit_offset, fz.eps, c.cs, i == c.kcol ? 1.f : c.sc_mul, D, qop);
+#pragma unroll
+                for (int s = 0; s < DS; ++s) {       // every lane of a group takes the key from the group's lane of column kcol
+                    knew[s].u.x = __shfl(qop[s].u.x, 16 * g + c.kcol, MV_WAVE);
+                    knew[s].u.y = __shfl(qop[s].u.y, 16 * g + c.kcol, MV_WAVE);
+                    knew[s].u.z = __shfl(qop[s].u.z, 16 * g + c.kcol, MV_WAVE);
+                    knew[s].u.w = __shfl(qop[s].u.w, 16 * g + c.kcol, MV_WAVE);
+                }
+            } else {
+                prepare_head<DS>(qop, g, fz.qw, fz.has_norm, fz.unit_offset, fz.eps, c.cs, c.sc_mul, D, qop);
+            }
+            if (EDGE && c.owns_new) {
+                if (!rides)
+                    prepare_head<DS>(knew, g, fz.kw, fz.has_norm && fz.kw.p != nullptr, fz.unit_offset, fz.eps, c.cs, 1.f, D, knew);
+                const int pidx = pos >> page_shift;
+                const int page = pidx < c.bt_width ? c.bt[pidx] : -1;
+                if (page >= 0) {
+                    const int slot = pos & slot_mask;
+                    if (i == 0) {
+                        bf16* kdst = const_cast<bf16*>(c.k_pages) + (size_t)page * page_elems +
+                                     ((size_t)c.kvh * page_size + slot) * D + 8 * g;
+#pragma unroll
+                        for (int s = 0; s < DS; ++s) *reinterpret_cast<uint4*>(kdst + 32 * s) = knew[s].u;
+                    }
+                    if (g == 0) {
+                        uint16_t* vdst = reinterpret_cast<uint16_t*>(const_cast<bf16*>(c.v_pages)) + (size_t)page * page_elems +
+                                         ((size_t)c.kvh * D + i) * page_size + slot;
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) vdst[(size_t)16 * dt * page_size] = vnew[dt];
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- the values of the chunk
+        Frag vop[BPW][DT];
+#pragma unroll
+        for (int j = 0; j < BPW; ++j) {
+            if (valid[j]) {
+                const int pv = (PS16 && (g & 2)) ? pb[j] : pa[j];      // keys 8g .. 8g+7 of the block
+                const bf16* vptr = vbase + (size_t)pv * page_elems + ((32 * (blk0 + j) + 8 * g) & slot_mask);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    vop[j][dt].u = *reinterpret_cast<const uint4*>(vptr + (size_t)16 * dt * page_size);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- scores^T of every block (in units of log2: the query carries scale * log2 e when fused)
+        float sc[BPW][8];                                  // this lane's keys 8g .. 8g+7 of each block
+#pragma unroll
+        for (int j = 0; j < BPW; ++j) {
+            if (valid[j]) {
+                const int key0 = 32 * (blk0 + j);
+                const bool new_here = EDGE && FUSED && c.owns_new && blk0 + j == c.b_hi;
+                if (new_here) {                            // the newest key comes from the registers
+                    const int rel = pos & 31;
+                    const bool mine = i == (((rel >> 3) << 2) | (rel & 3));
+                    const bool second = (rel >> 2) & 1;
+#pragma unroll
+                    for (int s = 0; s < DS; ++s) {
+                        if (mine && !second) kop[j][0][s] = knew[s];
+                        if (mine && second) kop[j][1][s] = knew[s];
+                    }
+                }
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < DS; ++s)
+                        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[j][tt][s].v, qop[s].v, sacc, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) sc[j][4 * tt + r] = FUSED ? sacc[r] : sacc[r] * c.sc_mul;
+                }
+                if (EDGE && (key0 + 31 > pos_read || key0 < lo)) {   // a block at an edge of the visible range
+                    const int k0 = key0 + 8 * g;           // this lane's first key
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (k0 + e > pos || k0 + e < lo) sc[j][e] = -INFINITY;
+                    // value slots above the newest key were never written, the newest key's own slot is not
+                    // written yet where its value comes from the registers, and a page below a window may be
+                    // another page's copy: everything outside [lo, pos_read] is cleared
+                    uint32_t keep[4];
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const bool a0 = k0 + 2 * w >= lo && k0 + 2 * w <= pos_read;
+                        const bool a1 = k0 + 2 * w + 1 >= lo && k0 + 2 * w + 1 <= pos_read;
+                        keep[w] = (a0 ? 0x0000ffffu : 0u) | (a1 ? 0xffff0000u : 0u);
+                    }
+                    if (new_here && g == ((pos & 31) >> 3)) {
+                        // (the cleared slot of the new position takes the value from the registers)
+                        const int e = pos & 7;
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) {
+                            const uint32_t v = (uint32_t)vnew[dt] << (16 * (e & 1));
+                            vop[j][dt].u.x = (vop[j][dt].u.x & keep[0]) | ((e >> 1) == 0 ? v : 0u);
+                            vop[j][dt].u.y = (vop[j][dt].u.y & keep[1]) | ((e >> 1) == 1 ? v : 0u);
+                            vop[j][dt].u.z = (vop[j][dt].u.z & keep[2]) | ((e >> 1) == 2 ? v : 0u);
+                            vop[j][dt].u.w = (vop[j][dt].u.w & keep[3]) | ((e >> 1) == 3 ? v : 0u);
+                        }
+                    } else {
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) {
+                            vop[j][dt].u.x &= keep[0];
+                            vop[j][dt].u.y &= keep[1];
+                            vop[j][dt].u.z &= keep[2];
+                            vop[j][dt].u.w &= keep[3];
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sc[j][e] = -INFINITY;
+            }
+        }
+        // ---- one maximum over the chunk, per column
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < BPW; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) mx = fmaxf(mx, sc[j][e]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
+        const float m_new = (!EDGE || first) ? mx : fmaxf(m_run, mx);
+        const float m_safe = (EDGE && m_new == -INFINITY) ? 0.f : m_new;
+        if (EDGE && !first) {
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
+            l_run *= corr;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) acc_o[dt] *= corr;
+        }
+        m_run = m_new;
+        // ---- out^T += V^T P^T, block by block
+        float psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < BPW; ++j) {
+            if (!valid[j]) continue;
+            float e[8];
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+                e[x] = __builtin_amdgcn_exp2f(sc[j][x] - m_safe);
+                psum += e[x];
+            }
+            Frag pop;
+            pop.u.x = f32x2_to_bf16x2_bits(e[0], e[1]);
+            pop.u.y = f32x2_to_bf16x2_bits(e[2], e[3]);
+            pop.u.z = f32x2_to_bf16x2_bits(e[4], e[5]);
+            pop.u.w = f32x2_to_bf16x2_bits(e[6], e[7]);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[j][dt].v, pop.v, acc_o[dt], 0, 0, 0);
+        }
+        l_run += psum;
+        first = false;
+        if (!EDGE || !last_chunk || 32 * (blk0 + BPW) > pos) break;
+    }
+}
+
+template <int D, bool FUSED, int BPW, bool PS16>
 __global__ void __launch_bounds__(64)
 attention_decode_wave_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                              const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
-                             const int* __restrict__ block_table, int bt_width, int page_size,
+                             const int* __restrict__ block_table, int bt_width, int page_size_rt, int page_shift_rt,
                              const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
                              int H, int Hkv, float scale, int window, float* __restrict__ partials,
                              int nchunks, FusedInput fz) {
     constexpr int DS = D / 32;
     constexpr int DT = D / 16;
+    const int page_shift = PS16 ? 4 : page_shift_rt;
     const int G = H / Hkv;
-    const int kvh = blockIdx.y;
-    const int z = blockIdx.z;
+    const int seq = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
     const int lane = threadIdx.x;
-    const int i = lane % 16;
-    const int g = lane / 16;
-    const int tpu = 16 / G;
+    const int i = lane & 15;
+    const int g = lane >> 4;
 
-    int seq = blockIdx.x, t0, nt;
+    int t0;                                  // the sequence's one token
     if (FUSED) {
         t0 = seq;
-        nt = fz.token_seq[t0] >= 0 ? 1 : 0;
+        if (fz.token_seq[t0] < 0) return;
     } else {
-        const int first = cu_seqlens[seq];
-        int count = cu_seqlens[seq + 1] - first;
-        if (count > tpu) count = tpu;
-        t0 = first;
-        nt = count;
+        t0 = cu_seqlens[seq];
+        if (cu_seqlens[seq + 1] - t0 <= 0) return;
     }
-    if (nt <= 0) return;
-    const int ncols = nt * G;
     const int* bt = block_table + (size_t)seq * bt_width;
-
-    // the page ids of this chunk's 16-key tiles: asked for before anything is known about the length
-    const int b_first = z * BPW;
-    int pg[2 * BPW];
+    // the page ids of this chunk's blocks (two a block: keys 0..15 and 16..31 of it, the same page
+    // where pages are larger): asked for before anything is known about the length
+    int pga[BPW], pgb[BPW];
 #pragma unroll
-    for (int t = 0; t < 2 * BPW; ++t) {
-        const int pidx = (32 * b_first + 16 * t) / page_size;
-        pg[t] = pidx < bt_width ? bt[pidx] : -1;
+    for (int j = 0; j < BPW; ++j) {
+        const int ia = (32 * (BPW * z + j)) >> page_shift, ib = (32 * (BPW * z + j) + 16) >> page_shift;
+        pga[j] = ia < bt_width ? bt[ia] : -1;
+        pgb[j] = ib < bt_width ? bt[ib] : -1;
     }
-
-    // this lane's column
-    const bool col_ok = i < ncols;
-    const int col_tok = t0 + (col_ok ? i / G : 0);
-    const int col_head = kvh * G + (col_ok ? i % G : 0);
+    const int pos = positions[t0];
+    // the query head of this lane's column (lanes beyond the group copy its last head and store nothing;
+    // fused with a cache write, the first column beyond the group holds the raw key of the new position,
+    // which only the wave that meets the new position makes use of)
+    const int head = kvh * G + (i < G ? i : G - 1);
+    const int kcol = (FUSED && fz.store && G < 16) ? G : 16;
     Frag qop[DS];
     {
-        const bf16* qrow = FUSED ? fz.qkv + (size_t)col_tok * fz.stride + fz.q_off + (size_t)col_head * D + 8 * g
-                                 : q + (size_t)col_tok * q_stride + (size_t)col_head * D + 8 * g;
+        const bf16* qrow = FUSED ? fz.qkv + (size_t)t0 * fz.stride + (i == kcol ? fz.k_off + (size_t)kvh * D
+                                                                                  : fz.q_off + (size_t)head * D) + 8 * g
+                                 : q + (size_t)t0 * q_stride + (size_t)head * D + 8 * g;
 #pragma unroll
-        for (int s = 0; s < DS; ++s) qop[s].u = col_ok ? *reinterpret_cast<const uint4*>(qrow + 32 * s) : uint4{0u, 0u, 0u, 0u};
+        for (int s = 0; s < DS; ++s) qop[s].u = *reinterpret_cast<const uint4*>(qrow + 32 * s);
     }
-    const int col_pos = col_ok ? positions[FUSED ? t0 : col_tok] : -1;
-    const int col_lo = (window >= 0 && col_pos - window > 0) ? col_pos - window : 0;
-    int hi_w, lo_w;
-    if (FUSED) {
-        hi_w = positions[t0];
-        lo_w = (window >= 0 && hi_w - window > 0) ? hi_w - window : 0;
-    } else {
-        hi_w = wave_max_i(col_ok ? col_pos : -1);
-        lo_w = wave_min_i(col_ok ? col_lo : 0x7fffffff);
-    }
-    if (hi_w < 0) return;
-    const int b_lo = lo_w / 32, b_hi = hi_w / 32;            // the blocks the sequence has
+    if (pos < 0) return;
+    const int lo = (window >= 0 && pos - window > 0) ? pos - window : 0;
+    const int b_lo = lo >> 5, b_hi = pos >> 5;            // the 32-key blocks the sequence has
     const bool last_chunk = z == nchunks - 1;
-    int b_end = last_chunk ? b_hi + 1 : b_first + BPW;       // the last chunk takes what lies above it too
-    if (b_end > b_hi + 1) b_end = b_hi + 1;
-    const int b_begin = b_first > b_lo ? b_first : b_lo;
-    if (b_begin >= b_end) return;                            // no key of the sequence in this chunk
+    int b_stop = last_chunk ? b_hi + 1 : BPW * z + BPW;    // the last chunk takes what lies above it too
+    if (b_stop > b_hi + 1) b_stop = b_hi + 1;
+    if ((BPW * z > b_lo ? BPW * z : b_lo) >= b_stop) return;   // no key of the sequence in this chunk
     int z_lo = b_lo / BPW, z_hi = b_hi / BPW;
     if (z_lo > nchunks - 1) z_lo = nchunks - 1;
     if (z_hi > nchunks - 1) z_hi = nchunks - 1;
-    const bool alone = z_lo == z_hi;                         // the sequence's only chunk: finish the row here
-    const float sc_mul = scale * LOG2E;
+    const bool alone = z_lo == z_hi;                       // the sequence's only chunk: finish the row here
 
-    __shared__ __attribute__((aligned(16))) float sh_const[FUSED ? 3 : 1][FUSED ? D : 1];
-    const int b_new = b_hi;
-    const bool owns_new = FUSED && fz.store && b_new >= b_begin && b_new < b_end;
-    Frag knew[DS], kraw[DS];
-    uint16_t vnew[DT];
-    if (FUSED) {
-        for (int d = lane; d < D; d += 64) {
-            if (fz.has_norm) {
-                sh_const[0][d] = fz.qw.at(d) + (fz.unit_offset ? 1.f : 0.f);
-                if (fz.kw.p != nullptr) sh_const[1][d] = fz.kw.at(d) + (fz.unit_offset ? 1.f : 0.f);
-            }
-            if (fz.table != nullptr) sh_const[2][d] = fz.table[(size_t)hi_w * D + d];
-        }
-#pragma unroll
-        for (int s = 0; s < DS; ++s) knew[s].u = kraw[s].u = uint4{0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vnew[dt] = 0;
-        if (owns_new) {
-            const bf16* row = fz.qkv + (size_t)t0 * fz.stride;
-            const bf16* krow = row + fz.k_off + (size_t)kvh * D + 8 * g;
-#pragma unroll
-            for (int s = 0; s < DS; ++s) kraw[s].u = *reinterpret_cast<const uint4*>(krow + 32 * s);
-            const uint16_t* vrow = reinterpret_cast<const uint16_t*>(row + fz.v_off + (size_t)kvh * D);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vnew[dt] = vrow[16 * dt + i];
-        }
-    }
-
-    struct Operands {
-        int page[2];
-        Frag k[2][DS];
-        Frag v[DT];
-    };
-    auto fetch = [&](int b, int page0, int page1, Operands& op) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int key0 = 32 * b + 16 * t;
-            const int pidx = key0 / page_size;
-            const int slot0 = key0 - pidx * page_size;
-            const int page = (b >= b_begin && b < b_end && key0 <= hi_w) ? (t == 0 ? page0 : page1) : -1;
-            op.page[t] = page;
-            if (page >= 0) {
-                const size_t head = (size_t)page * Hkv + kvh;
-                const bf16* kptr = k_pages + ((head * page_size + slot0 + i) * D + 8 * g);
-#pragma unroll
-                for (int s = 0; s < DS; ++s) op.k[t][s].u = *reinterpret_cast<const uint4*>(kptr + 32 * s);
-                const bf16* vptr = v_pages + (head * D + i) * page_size + slot0 + 4 * g;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-                    op.v[dt].h[t] = *reinterpret_cast<const uint2*>(vptr + (size_t)16 * dt * page_size);
-            } else {
-#pragma unroll
-                for (int s = 0; s < DS; ++s) op.k[t][s].u = uint4{0u, 0u, 0u, 0u};
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) op.v[dt].h[t] = uint2{0u, 0u};
-            }
-        }
-    };
+    WaveChunk c;
+    c.k_pages = k_pages; c.v_pages = v_pages; c.bt = bt; c.bt_width = bt_width;
+    c.page_size = page_size_rt; c.page_shift = page_shift_rt; c.Hkv = Hkv; c.kvh = kvh; c.z = z; c.nchunks = nchunks;
+    c.pos = pos; c.lo = lo; c.b_hi = b_hi; c.i = i; c.g = g; c.sc_mul = scale * LOG2E; c.t0 = t0;
+    c.owns_new = FUSED && fz.store && b_hi >= BPW * z && (last_chunk || b_hi < BPW * z + BPW);
+    c.cs = (FUSED && fz.table != nullptr) ? fz.table + (size_t)pos * D : nullptr;
+    c.kcol = kcol;
 
     float m_run = -INFINITY, l_run = 0.f;
     floatx4_t acc_o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-
-    auto compute = [&](int b, Operands& op) {
-        const int base = 32 * b;
-        if (FUSED && owns_new && b == b_new) {   // the newest key and value come from the registers
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (base + 16 * t + i == hi_w) {
-#pragma unroll
-                    for (int s = 0; s < DS; ++s) op.k[t][s] = knew[s];
-                }
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (base + 16 * t + 4 * g + r == hi_w) {
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) op.v[dt].s[t * 4 + r] = vnew[dt];
-                    }
-            }
-        }
-        float p[2][4];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
-            if (op.page[t] >= 0) {
-#pragma unroll
-                for (int s = 0; s < DS; ++s)
-                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.k[t][s].v, qop[s].v, sacc, 0, 0, 0);
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = base + 16 * t + 4 * g + r;
-                const bool ok = op.page[t] >= 0 && col_ok && key <= col_pos && key >= col_lo;
-                p[t][r] = ok ? sacc[r] * sc_mul : -INFINITY;
-            }
-        }
-        Frag pop;
-        float mx = -INFINITY;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) mx = fmaxf(mx, p[t][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16, MV_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, MV_WAVE));
-        const float m_new = fmaxf(m_run, mx);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
-        float psum = 0.f;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float e = __builtin_amdgcn_exp2f(p[t][r] - m_safe);
-                psum += e;
-                pop.v[t * 4 + r] = (__bf16)e;
-            }
-        l_run = l_run * corr + psum;
-        m_run = m_new;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) acc_o[dt] *= corr;
-        if (base + 31 > hi_w) {  // slots above the newest key were never written
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (base + 16 * t + 4 * g + r > hi_w) op.v[dt].s[t * 4 + r] = 0;
-        }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-            acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.v[dt].v, pop.v, acc_o[dt], 0, 0, 0);
-    };
-
-    // all keys and values of the chunk are asked for at once
-    Operands ops[BPW];
-#pragma unroll
-    for (int j = 0; j < BPW; ++j) fetch(b_first + j, pg[2 * j], pg[2 * j + 1], ops[j]);
-    if (FUSED) {   // while those loads are in flight
-        __syncthreads();                          // (one wave: the constants are in LDS)
-        const float* cs = fz.table != nullptr ? sh_const[2] : nullptr;
-        norm_rotate<DS>(qop, g, fz.has_norm ? sh_const[0] : nullptr, fz.eps, cs, D, qop);
-        if (owns_new) {
-            norm_rotate<DS>(kraw, g, fz.has_norm ? sh_const[1] : nullptr, fz.eps, cs, D, knew);
-            const int pidx = hi_w / page_size;
-            const int page = pidx < bt_width ? bt[pidx] : -1;
-            if (page >= 0) {
-                const int slot = hi_w % page_size;
-                const size_t head = (size_t)page * Hkv + kvh;
-                if (i == 0) {
-                    bf16* kdst = const_cast<bf16*>(k_pages) + ((head * page_size + slot) * D + 8 * g);
-#pragma unroll
-                    for (int s = 0; s < DS; ++s) *reinterpret_cast<uint4*>(kdst + 32 * s) = knew[s].u;
-                }
-                if (g == 0) {
-                    uint16_t* vdst = reinterpret_cast<uint16_t*>(const_cast<bf16*>(v_pages)) + (head * D + i) * page_size + slot;
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) vdst[(size_t)16 * dt * page_size] = vnew[dt];
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < BPW; ++j) compute(b_first + j, ops[j]);
-    // (the last chunk of a launch planned for shorter contexts: the blocks above it, one after the other)
-    for (int b = b_first + BPW; b < b_end; ++b) {
-        const int p0 = (32 * b) / page_size, p1 = (32 * b + 16) / page_size;
-        fetch(b, p0 < bt_width ? bt[p0] : -1, p1 < bt_width ? bt[p1] : -1, ops[0]);
-        compute(b, ops[0]);
-    }
+    // a chunk wholly inside the visible range (and not the one that may have to go on above itself)
+    const bool inside = 32 * BPW * z >= lo && 32 * BPW * (z + 1) - 1 < pos && !last_chunk;
+    if (inside) wave_chunk<D, FUSED, BPW, PS16, false>(c, fz, qop, pga, pgb, m_run, l_run, acc_o);
+    else wave_chunk<D, FUSED, BPW, PS16, true>(c, fz, qop, pga, pgb, m_run, l_run, acc_o);
 
     l_run += __shfl_xor(l_run, 16, MV_WAVE);
     l_run += __shfl_xor(l_run, 32, MV_WAVE);
-    if (!col_ok) return;
+    if (i >= G) return;
     if (alone) {
-        bf16* orow = out + (size_t)col_tok * out_stride + (size_t)col_head * D;
+        bf16* orow = out + (size_t)t0 * out_stride + (size_t)head * D + 4 * g;
         const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             uint2 packed;
             packed.x = f32x2_to_bf16x2_bits(acc_o[dt][0] * inv, acc_o[dt][1] * inv);
             packed.y = f32x2_to_bf16x2_bits(acc_o[dt][2] * inv, acc_o[dt][3] * inv);
-            *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = packed;
+            *reinterpret_cast<uint2*>(orow + 16 * dt) = packed;
         }
         return;
     }
-    float* prow = partials + (((size_t)col_tok * H + col_head) * nchunks + z) * (D + 2);
+    float* prow = partials + (((size_t)t0 * H + head) * nchunks + z) * (D + 2);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
         *reinterpret_cast<float4*>(prow + 16 * dt + 4 * g) = float4{acc_o[dt][0], acc_o[dt][1], acc_o[dt][2], acc_o[dt][3]};
@@ -917,12 +1085,25 @@ static int decode_common(bool fused, const FusedInput& fz, const void* q, long q
         MV_REQUIRE(chunk_keys == 64 || chunk_keys == 128, "attention_decode: chunks of %d keys (64 or 128)", chunk_keys);
         MV_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || partials != nullptr),
                    "attention_decode: bad chunk count %d or missing work area", nsplit);
+        MV_REQUIRE((page_size & (page_size - 1)) == 0, "attention_decode: the one-wave kernel takes pages of a power of "
+                   "two slots, got %d", page_size);
         if (n_seqs <= 0) return 0;
+        int page_shift = 0;
+        while ((1 << page_shift) < page_size) ++page_shift;
         dim3 grid(n_seqs, Hkv, nsplit);
 #define AF_WAVE(DD, FF, BB)                                                                                          \
-        hipLaunchKernelGGL((attention_decode_wave_kernel<DD, FF, BB>), grid, dim3(64), 0, stream, (const bf16*)q, q_stride, \
-                           (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,  \
-                           page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit, fz)
+        do {                                                                                                          \
+            if (page_size == 16)                                                                                      \
+                hipLaunchKernelGGL((attention_decode_wave_kernel<DD, FF, BB, true>), grid, dim3(64), 0, stream,        \
+                                   (const bf16*)q, q_stride, (bf16*)out, out_stride, (const bf16*)k_pages,            \
+                                   (const bf16*)v_pages, block_table, bt_width, page_size, page_shift, positions,     \
+                                   cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit, fz);                  \
+            else                                                                                                      \
+                hipLaunchKernelGGL((attention_decode_wave_kernel<DD, FF, BB, false>), grid, dim3(64), 0, stream,       \
+                                   (const bf16*)q, q_stride, (bf16*)out, out_stride, (const bf16*)k_pages,            \
+                                   (const bf16*)v_pages, block_table, bt_width, page_size, page_shift, positions,     \
+                                   cu_seqlens, n_seqs, H, Hkv, scale, window, partials, nsplit, fz);                  \
+        } while (0)
         if (D == 128 && fused && chunk_keys == 64) AF_WAVE(128, true, 2);
         else if (D == 128 && fused) AF_WAVE(128, true, 4);
         else if (D == 128 && chunk_keys == 64) AF_WAVE(128, false, 2);

@@ -52,9 +52,11 @@ COMPUTE_UNITS = 256
 PREFILL_TWO_GROUPS_FROM = 1024
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
-# most waves in the grid of the one-wave decode attention (a wave per chunk of keys); above that the
-# workgroup kernel with its pipeline over the keys serves the step
-DECODE_WAVE_GRID = 4096
+# most waves in the grid of the one-wave decode attention (a wave per chunk of keys): about one wave
+# for each of the chip's 1024 SIMDs. Above that the workgroup kernel with its pipeline over the keys
+# serves the step (measured on MI355X at 0.6B sizes and contexts of 1100: one sequence 13 against 16 us
+# with the merge kernel, eight sequences 25 against 21)
+DECODE_WAVE_GRID = 1024
 # from this many tokens on, value rows are written to their pages 16 tokens of a kv head at a time
 STORE_V_SPLIT_TOKENS = 64
 
@@ -582,7 +584,7 @@ class Ops:
                       positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim,
                       float(scale), w, self.code, self._stream())
 
-    def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int):
+    def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int, page_size: int = 16):
         """How a decode step's keys are dealt out: (nsplit, partials, chunk_keys).
 
         Small grids (few sequences) take the one-wave kernel: a wave per chunk of 64 or 128 keys of a
@@ -598,6 +600,8 @@ class Ops:
         forced = getattr(plan, "decode_chunk_keys", None)
         for chunk in (64, 128):
             nchunks = -(-ctx // chunk)
+            if page_size & (page_size - 1):
+                break                              # the one-wave kernel takes pages of a power of two slots
             if forced == chunk or (forced is None and n_seqs * Hkv * nchunks <= DECODE_WAVE_GRID):
                 rows = max(n_seqs * nchunks, DECODE_WAVE_GRID // max(1, Hkv))      # one size serves every graph
                 partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
@@ -656,7 +660,7 @@ class Ops:
         _dev(block_table, "block table")
         if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
             raise KernelLibraryError("attention: the block table must be a contiguous int32 matrix")
-        nsplit, partials, chunk_keys = self._decode_split(plan, n, H, Hkv, D)
+        nsplit, partials, chunk_keys = self._decode_split(plan, n, H, Hkv, D, page_size)
         self.lib.call("mv_attention_decode_fused", qkv.data_ptr(), stride, 0, H * D, (H + Hkv) * D, out.data_ptr(), os_,
                       k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n, H, Hkv, D, float(scale),
@@ -675,7 +679,7 @@ class Ops:
         group = H // Hkv
         n_seqs = plan.n_seqs
         if plan.decode_only and group <= 16:
-            nsplit, partials, chunk_keys = self._decode_split(plan, n_seqs, H, Hkv, D)
+            nsplit, partials, chunk_keys = self._decode_split(plan, n_seqs, H, Hkv, D, page_size)
             self.lib.call("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
