@@ -17,6 +17,10 @@ is the one reported (``timed_regions`` says how many there were). One JSON line 
                divided by its time, against 8 TB/s of HBM
   points       decode tokens/s at batch 1 and batch 64
 
+``--emit-kernels CSV`` measures nothing: it takes the kernel trace that rocprofv3 wrote for a run
+with the same options and prints one row per kernel of the step with its time, the bytes it has to
+move, its operations and the share of the HBM and MFMA peaks these amount to.
+
 ``--only serve`` runs a continuous-batching workload instead (``--requests`` requests, 256 by
 default, with prompt lengths uniform in 128..2048 and ``--gen-len`` generated tokens each, all
 submitted at once under a budget of ``--token-budget`` tokens a step) and prints its own line:
@@ -184,6 +188,49 @@ def measure_serve(llm, vocab, requests, gen_len, seed, prompt_min=128, prompt_ma
             llm.scheduler.num_preemptions - before)
 
 
+def emit_kernels(llm, cfg, args) -> int:
+    """Prints, for the step kinds of this run, a table of their kernels: time from the rocprofv3
+    kernel trace ``args.emit_kernels``, bytes and operations from what the engine launches."""
+    from minivllm_amd import SamplingParams
+    from minivllm_amd.engine import roofline
+    vocab = cfg.vocab_size
+    ex = llm.executor
+    if args.only in ("all", "decode"):
+        k = llm.config.num_scheduler_steps
+        sp = SamplingParams(temperature=0.0, max_tokens=3 * k + 2, ignore_eos=True)
+        reqs = [llm.submit(random_prompt(vocab, args.prompt_len, args.seed + i), sp) for i in range(args.batch)]
+        while llm.has_unfinished():
+            llm.step()
+        rows = [key for key in ex.graph_ledger if len(key) == 3 and key[0] >= args.batch]
+        single = [key for key in ex.graph_ledger if len(key) == 2 and key[0] >= args.batch]
+        if not rows and not single:
+            print("bench.py: no decode graph was recorded for this batch (graphs off?); nothing to price")
+            return 2
+        key = max(rows, key=lambda t: (-t[0], t[2])) if rows else min(single)
+        ledger = roofline.one_step(roofline.launches(ex.graph_ledger[key]))
+        ctx = args.prompt_len + (args.warmup + args.steps) // 2
+        title = (f"decode step, qwen3-{args.shape} shape, batch {args.batch}, priced at a context of {ctx} tokens "
+                 f"(graph for {key[0]} sequences, contexts up to {key[1]})")
+        print(roofline.kernel_table(args.emit_kernels, ledger, args.dtype, keys=args.batch * ctx, pairs=args.batch * ctx,
+                                    title=title, wall_ms=args.step_ms))
+    if args.only in ("all", "prefill"):
+        if args.only == "all":
+            print()
+        sp = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
+        llm.submit(random_prompt(vocab, args.prefill_tokens, args.seed + 100), sp)
+        ex.ops.ledger = []
+        try:
+            while llm.has_unfinished():
+                llm.step()
+            ledger = roofline.launches(ex.ops.ledger)
+        finally:
+            ex.ops.ledger = None
+        title = f"prefill of one {args.prefill_tokens}-token prompt, qwen3-{args.shape} shape"
+        print(roofline.kernel_table(args.emit_kernels, ledger, args.dtype, title=title,
+                                    wall_ms=args.step_ms if args.only == "prefill" else None))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -213,6 +260,13 @@ def main() -> int:
     ap.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the serve workload")
     ap.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the serve workload")
     ap.add_argument("--max-seqs", type=int, default=256, help="most requests in one step of the serve workload")
+    ap.add_argument("--emit-kernels", metavar="CSV", default=None,
+                    help="measure nothing; read the *_kernel_trace.csv that `rocprofv3 --kernel-trace --output-format csv` "
+                         "wrote for a run with the same options and print a table of the step's kernels: time, bytes, "
+                         "operations, share of the HBM and MFMA peaks")
+    ap.add_argument("--step-ms", type=float, default=None,
+                    help="with --emit-kernels: the step's time on the clock (ms_per_step of the measured line), to "
+                         "show the time between kernels")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -251,6 +305,8 @@ def main() -> int:
             "total_tok_s": round((gen + prompt) / dt, 1), "preemptions": preempted}))
         return 0
     llm, cfg = build_llm(args, shape, layers)
+    if args.emit_kernels:
+        return emit_kernels(llm, cfg, args)
     nums = model_numbers(shape, layers)
     item = 2 if args.dtype == "bfloat16" else 4
 

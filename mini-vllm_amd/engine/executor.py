@@ -148,6 +148,8 @@ class Executor:
         self._graph_workspace: Optional[Workspace] = None
         # what each recorded graph holds, by kind of node (see _record)
         self.graph_census: Dict[Tuple, Dict[str, int]] = {}
+        # what each recorded graph launches, in order: (entry point, bytes, operations, ...) per launch
+        self.graph_ledger: Dict[tuple, list] = {}
         # pinned buffers for the tokens of launches in flight, used in turn (two launches at most are)
         self._token_buffers: List[Optional[torch.Tensor]] = [None] * 4
         self._next_token_buffer = 0
@@ -389,7 +391,9 @@ class Executor:
             max_q_len=max(facts["q_lens"]) if facts["q_lens"] else 0,
             max_context_len=max((s.start + len(s.tokens) for s in seqs), default=0),
             n_seqs=facts["Sp"], q_lens=list(facts["q_lens"]) + [0] * (facts["Sp"] - facts["S"]),
-            cu_seqlens=ctx.cu_seqlens, workspace=self.rt.workspace)
+            cu_seqlens=ctx.cu_seqlens, workspace=self.rt.workspace,
+            kv_tokens=sum(s.start + len(s.tokens) for s in seqs),
+            attention_pairs=sum(len(s.tokens) * s.start + len(s.tokens) * (len(s.tokens) + 1) // 2 for s in seqs))
         for call in range(len(self.plan.calls)):
             g = self.group_of_call.get(call)
             if g is not None:
@@ -645,12 +649,14 @@ class Executor:
         only, and must be clean then."""
         for library in (True, False):
             self.ops.library_in_graphs = library
+            self.ops.ledger = []
             try:
                 graph = torch.cuda.CUDAGraph(keep_graph=True)
                 with torch.cuda.graph(graph, pool=self._graph_pool):
                     body()
             finally:
                 self.ops.library_in_graphs = True
+                self.graph_ledger[key], self.ops.ledger = self.ops.ledger, None
             census = self.ops.graph_census(graph.raw_cuda_graph())
             self.graph_census[key] = census
             if census["memset"] == 0:

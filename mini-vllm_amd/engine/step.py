@@ -61,9 +61,13 @@ class AttentionPlan:
     q_lens: Sequence[int] = ()     # tokens per sequence, on the host
     cu_seqlens: Optional[torch.Tensor] = None   # int32 [n_seqs + 1] on the device
     workspace: Optional[object] = None          # where kernels take scratch memory from
-    # decode steps: None lets the launch heuristic choose between the one-wave kernel (chunks of 64 or
-    # 128 keys) and the workgroup kernel (0); a test may force one
-    decode_chunk_keys: Optional[int] = None
+    # decode steps: over how many workgroups a sequence's keys are dealt out; None lets the launch
+    # rule choose (tests force counts)
+    decode_splits: Optional[int] = None
+    # for measurement: keys in the cache of the step's sequences after the step (summed), and the
+    # number of (query, visible key) pairs without windows
+    kv_tokens: int = 0
+    attention_pairs: int = 0
 
 
 class StepContext:

@@ -52,11 +52,10 @@ COMPUTE_UNITS = 256
 PREFILL_TWO_GROUPS_FROM = 1024
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
-# most waves in the grid of the one-wave decode attention (a wave per chunk of keys): about one wave
-# for each of the chip's 1024 SIMDs. Above that the workgroup kernel with its pipeline over the keys
-# serves the step (measured on MI355X at 0.6B sizes and contexts of 1100: one sequence 13 against 16 us
-# with the merge kernel, eight sequences 25 against 21)
-DECODE_WAVE_GRID = 1024
+# the workgroup kernel splits a sequence's keys until about this many workgroups are in flight
+DECODE_SPLIT_WORKGROUPS = 256
+# (sequence, kv head) pairs of one decode step whose keys may be split over workgroups
+SPLIT_COUNTERS = 1 << 16
 # from this many tokens on, value rows are written to their pages 16 tokens of a kv head at a time
 STORE_V_SPLIT_TOKENS = 64
 
@@ -133,6 +132,19 @@ class Ops:
         self._split_pending: Optional[SplitSum] = None     # partial sums in the work area nobody has used yet
         self._mid_retired: list = []
         self._sample_work: Optional[torch.Tensor] = None
+        self._attn_counters: Optional[torch.Tensor] = None
+        # measurement: with a list here, every launch leaves (entry point, bytes it has to move,
+        # floating-point operations) in it; the benchmark sets it for one eager step and prices the
+        # kernels of a profile with the totals (engine/roofline.py)
+        self.ledger: Optional[list] = None
+
+    def _note(self, entry: str, nbytes, flops=0) -> None:
+        if self.ledger is not None:
+            self.ledger.append((entry, int(nbytes), int(flops)))
+
+    @staticmethod
+    def _size(*tensors) -> int:
+        return sum(t.numel() * t.element_size() for t in tensors if t is not None)
 
     # ------------------------------------------------------------------------------------
     def bind_stream(self) -> None:
@@ -161,6 +173,7 @@ class Ops:
             raise KernelLibraryError("embedding: ids must be int32 [>= n] and the residual float32 [n, h]")
         if table.dim() != 2 or table.shape[1] != h or not table.is_contiguous() or not resid.is_contiguous():
             raise KernelLibraryError(f"embedding: table {tuple(table.shape)} does not fit residual {tuple(resid.shape)}")
+        self._note("mv_embedding", n * h * (table.element_size() + 4) + n * 4)
         self.lib.call("mv_embedding", ids.data_ptr(), table.data_ptr(), _weight_code(table, "embedding table"),
                       resid.data_ptr(), n, h, table.shape[0], float(scale), self._stream())
 
@@ -200,6 +213,9 @@ class Ops:
                 raise KernelLibraryError(f"add_rmsnorm: weight of {weight.numel()} elements for rows of {h}")
             if out.dim() != 2 or out.shape[0] < n_out or out.shape[1] != h or not out.is_contiguous():
                 raise KernelLibraryError(f"add_rmsnorm: output {tuple(out.shape)} does not fit [{n_out}, {h}]")
+        self._note("mv_add_rmsnorm", (n * h * (8 if rows is None and delta is not None else 4) if rows is None else n_out * h * 4)
+                   + (0 if delta is None else (n if rows is None else n_out) * h * delta.element_size())
+                   + (0 if out is None else n_out * h * out.element_size()), 4 * n_out * h)
         self.lib.call("mv_add_rmsnorm", resid.data_ptr(), _ptr(delta), _ptr(weight), wcode, float(eps),
                       int(unit_offset), _ptr(out), _ptr(rows), n_out, h, self.code, self._stream())
 
@@ -215,6 +231,8 @@ class Ops:
                 or (rows is None and out.shape[0] < n)):
             return False
         n_out = n if rows is None else rows.numel()
+        self._note("mv_add_rmsnorm_split", n_out * h * (4 * delta.splits + (8 if rows is None else 4) + out.element_size()),
+                   (4 + delta.splits) * n_out * h)
         self.lib.call("mv_add_rmsnorm_split", resid.data_ptr(), delta.work.data_ptr(), delta.splits, n * h,
                       _ptr(delta.bias), weight.data_ptr(), _weight_code(weight, "norm weight"), float(eps),
                       int(unit_offset), out.data_ptr(), _ptr(rows), n_out, h, self.code, self._stream())
@@ -231,6 +249,7 @@ class Ops:
         n, h = x.shape
         if weight.numel() != h or not weight.is_contiguous():
             raise KernelLibraryError(f"rmsnorm: weight of {weight.numel()} elements for rows of {h}")
+        self._note("mv_rmsnorm", self._size(x, out), 4 * n * h)
         self.lib.call("mv_rmsnorm", x.data_ptr(), x.stride(0) if n > 1 else h, weight.data_ptr(),
                       _weight_code(weight, "norm weight"), float(eps), int(unit_offset), out.data_ptr(),
                       out.stride(0) if n > 1 else h, n, h, self.code, self._stream())
@@ -296,6 +315,8 @@ class Ops:
         # with many tokens the values go to their transposed pages tile by tile, so that
         # neighbouring tokens write neighbouring slots (mode 3); with few, a store per token and head
         mode = 0 if not store else (3 if n >= STORE_V_SPLIT_TOKENS else 1)
+        self._note("mv_qk_norm_rope_store", n * (width + q_dim + (2 * kv_dim if store else 0)) * qkv.element_size()
+                   + (n * rot * 4 if rope_table is not None else 0), 10 * n * (q_dim + (kv_dim if store else 0)))
         self.lib.call("mv_qk_norm_rope_store", qkv.data_ptr(), stride, 0, q_dim,
                       q_dim + kv_dim, positions.data_ptr(), token_seq.data_ptr(), _ptr(block_table), bt_width,
                       page_size, _ptr(k_pages), _ptr(v_pages), n, num_heads, num_kv_heads, head_dim,
@@ -308,6 +329,7 @@ class Ops:
         n, two_i = gate_up.shape
         if two_i % 2 or out.shape != (n, two_i // 2) or not gate_up.is_contiguous() or not out.is_contiguous():
             raise KernelLibraryError(f"swiglu: {tuple(gate_up.shape)} -> {tuple(out.shape)} is not [n, 2I] -> [n, I]")
+        self._note("mv_swiglu", self._size(gate_up, out), 6 * out.numel())
         self.lib.call("mv_swiglu", gate_up.data_ptr(), out.data_ptr(), n, two_i // 2, self.code, self._stream())
 
     # ------------------------------------------------------------------------------------
@@ -367,6 +389,7 @@ class Ops:
             # more rows than one workgroup takes are dealt out to groups of workgroups by the kernel
             for m0 in range(0, M, SKINNY_LAUNCH_ROWS):
                 m = min(SKINNY_LAUNCH_ROWS, M - m0)
+                self._note("mv_gemm_skinny", m * K * 2 + (N * K * 2 if m0 == 0 else 0) + m * N * out.element_size(), 2 * m * N * K)
                 self.lib.call("mv_gemm_skinny", a.data_ptr() + m0 * lda * 2, lda, w.data_ptr(), K, _ptr(bias),
                               out.data_ptr() + m0 * ldc * out.element_size(), ldc, _CODES[out.dtype], m, N, K,
                               self._stream())
@@ -374,6 +397,7 @@ class Ops:
         if fast and M > SKINNY_MAX_M and self._library_serves(out) and \
                 self._library_allowed(M, N, K, bias is not None, out.dtype) and self._library_product(a, w, bias, out):
             return
+        self._note("mv_gemm_ref", self._size(a, w, out), 2 * M * N * K)
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
 
@@ -404,6 +428,7 @@ class Ops:
                 if torch.cuda.is_current_stream_capturing():
                     raise KernelLibraryError("the library's workspace must be made before a capture")
                 self._lt_work = torch.empty(int(self.lib.dll.mv_gemm_lt_workspace()), dtype=torch.uint8, device=a.device)
+            self._note("mv_gemm_lt", self._size(a, w, out), 2 * M * N * K)
             return self.lib.offer("mv_gemm_lt", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias),
                                   out.data_ptr(), out.stride(0) if M > 1 else N, _CODES[out.dtype], M, N, K,
                                   self._lt_work.data_ptr(), self._lt_work.numel(), self._stream())
@@ -453,11 +478,13 @@ class Ops:
         if self._split_pending is not None:
             self._split_pending.materialize()                  # its sums are about to be overwritten
         if defer_sum and not swiglu and self.lib.has("mv_add_rmsnorm_split"):
+            self._note("mv_gemm_mid", self._size(a, w) + 4 * M * N * int(self.lib.dll.mv_gemm_mid_splits(N, K)), 2 * M * N * K)
             self.lib.call("mv_gemm_mid_sums", a.data_ptr(), lda, w.data_ptr(), M, N, K, self._mid_work.data_ptr(),
                           self._mid_work.numel(), self._stream())
             pending = SplitSum(self, out, self._mid_work, int(self.lib.dll.mv_gemm_mid_splits(N, K)), bias)
             self._split_pending = pending
             return pending
+        self._note("mv_gemm_mid", self._size(a, w, out) + 8 * M * N * int(self.lib.dll.mv_gemm_mid_splits(N, K)), 2 * M * N * K)
         self.lib.call("mv_gemm_mid", a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(), ldc,
                       _CODES[out.dtype], M, N, K, int(swiglu), self._mid_work.data_ptr(), self._mid_work.numel(),
                       self._stream())
@@ -502,6 +529,8 @@ class Ops:
         resid_in, delta, resid_out = pending.fused()
         if isinstance(delta, SplitSum):
             delta = delta.materialize()
+        self._note("mv_gemm_skinny_norm", M * K * (4 + (2 + 4 if delta is not None else 0)) + self._size(w, out),
+                   2 * M * w.shape[0] * K + 4 * M * K)
         self.lib.call("mv_gemm_skinny_norm", resid_in.data_ptr(), _ptr(delta), _ptr(resid_out), weight.data_ptr(),
                       _weight_code(weight, "norm weight"), float(eps), int(unit_offset), w.data_ptr(),
                       _ptr(bias), out.data_ptr(), out.stride(0) if M > 1 else N, _CODES[out.dtype], M, N, K,
@@ -535,6 +564,7 @@ class Ops:
         if self._gemm_mid(a, a.stride(0) if M > 1 else K, w_gate_up, None, out, out.stride(0) if M > 1 else two_i // 2,
                           M, two_i, K, swiglu=True):
             return True
+        self._note("mv_gemm_skinny_swiglu", self._size(a, w_gate_up, out), 2 * M * two_i * K)
         self.lib.call("mv_gemm_skinny_swiglu", a.data_ptr(), a.stride(0) if M > 1 else K, w_gate_up.data_ptr(),
                       out.data_ptr(), out.stride(0) if M > 1 else two_i // 2, M, two_i // 2, K, self._stream())
         return True
@@ -579,39 +609,54 @@ class Ops:
         if self._attention_fast(q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
                                 num_heads, num_kv_heads, head_dim, scale, w, plan):
             return
+        self._note_attention("mv_attention_ref", plan, n, num_heads, num_kv_heads, head_dim, q.element_size())
         self.lib.call("mv_attention_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim,
                       float(scale), w, self.code, self._stream())
 
-    def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int, page_size: int = 16):
-        """How a decode step's keys are dealt out: (nsplit, partials, chunk_keys).
+    def _note_attention(self, entry: str, plan, n_tokens: int, H: int, Hkv: int, D: int, item: int, splits: int = 1) -> None:
+        """Bytes: the keys and values of every sequence once (per key, so that the line can be priced
+        at another context length), queries and outputs, the partial results of split keys written and
+        read back. Operations: two products over every (query, visible key) pair."""
+        if self.ledger is None:
+            return
+        keys = getattr(plan, "kv_tokens", 0) if plan is not None else 0
+        pairs = getattr(plan, "attention_pairs", 0) if plan is not None else 0
+        fixed = 2 * n_tokens * H * D * item
+        if splits > 1:
+            fixed += 2 * n_tokens * H * splits * (D + 2) * 4
+        self.ledger.append((entry, fixed, 0, keys, pairs, 2 * Hkv * D * item, 4 * H * D))
 
-        Small grids (few sequences) take the one-wave kernel: a wave per chunk of 64 or 128 keys of a
-        (sequence, kv head) pair, as many chunks as the planned context length has, all of a chunk's
-        keys in flight at once; chunk_keys is 64 or 128 then and nsplit the number of chunks. The grid
-        may hold up to DECODE_WAVE_GRID waves (chunks above a sequence's newest key end at once).
+    def _split_counters(self, n: int, partials) -> Optional[int]:
+        """One counter for every (sequence, kv head) of a decode step whose keys are split over
+        workgroups: the workgroups count themselves in and the last one adds the partial results up.
+        The counters are zero between launches (the last workgroup puts its counter back), so they are
+        cleared once, here; launches that share them must follow each other on one stream."""
+        if partials is None:
+            return None
+        if self._attn_counters is None:
+            self._attn_counters = torch.zeros(SPLIT_COUNTERS, dtype=torch.int32, device=partials.device)
+        if n > SPLIT_COUNTERS:
+            raise ValueError(f"a decode step of {n} (sequence, kv head) pairs exceeds the {SPLIT_COUNTERS} split counters")
+        return self._attn_counters.data_ptr()
 
-        Larger grids take the workgroup kernel (chunk_keys 0): the keys are split until about 256
-        workgroups are in flight, but never below 128 keys per split (measured on MI355X with 8 kv
-        heads: batch 64 is fastest without a split). The count is a property of the plan (a captured
-        graph keeps it); each split takes its share of the keys a sequence actually has."""
+    def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int):
+        """Over how many workgroups a decode step deals a sequence's keys out, and the work area for
+        their partial results: (nsplit, partials). The keys go round in groups of 128 (a block of 32
+        to each of a workgroup's four waves), so a split beyond the number of such groups in the
+        planned context would only add workgroups that end at once. The count is a property of the
+        plan (a captured graph keeps it): about DECODE_SPLIT_WORKGROUPS workgroups in flight, one for
+        every compute unit (measured on MI355X with 8 kv heads at contexts of 1,100: 512 and 1,024
+        workgroups are 5 and 18 % slower at batch 8; batch 64 is fastest without a split)."""
         ctx = max(1, plan.max_context_len)
-        forced = getattr(plan, "decode_chunk_keys", None)
-        for chunk in (64, 128):
-            nchunks = -(-ctx // chunk)
-            if page_size & (page_size - 1):
-                break                              # the one-wave kernel takes pages of a power of two slots
-            if forced == chunk or (forced is None and n_seqs * Hkv * nchunks <= DECODE_WAVE_GRID):
-                rows = max(n_seqs * nchunks, DECODE_WAVE_GRID // max(1, Hkv))      # one size serves every graph
-                partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
-                return nchunks, partials, chunk
-        nsplit = max(1, min(256 // max(1, n_seqs * Hkv), max(1, ctx // 128), 64))
+        forced = getattr(plan, "decode_splits", None)
+        nsplit = forced if forced else max(1, min(DECODE_SPLIT_WORKGROUPS // max(1, n_seqs * Hkv), -(-ctx // 128), 64))
         partials = None
         if nsplit > 1:
             rows = max(n_seqs * nsplit, 2048 // Hkv, 256)      # one size serves every batch of a graph set
             partials = plan.workspace.get("attn.partials", (rows * H * (D + 2),), torch.float32)
-        return nsplit, partials, 0
+        return nsplit, partials
 
     def attention_decode_fused(self, qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor,
                                v_pages: torch.Tensor, block_table: torch.Tensor, page_size: int,
@@ -660,13 +705,15 @@ class Ops:
         _dev(block_table, "block table")
         if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
             raise KernelLibraryError("attention: the block table must be a contiguous int32 matrix")
-        nsplit, partials, chunk_keys = self._decode_split(plan, n, H, Hkv, D, page_size)
+        nsplit, partials = self._decode_split(plan, n, H, Hkv, D)
+        self._note_attention("mv_attention_decode_fused", plan, n, H, Hkv, D, 2, splits=nsplit)
         self.lib.call("mv_attention_decode_fused", qkv.data_ptr(), stride, 0, H * D, (H + Hkv) * D, out.data_ptr(), os_,
                       k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n, H, Hkv, D, float(scale),
                       -1 if window is None else int(window), _ptr(q_weight), _ptr(k_weight), wcode, float(eps),
-                      int(unit_offset), _ptr(rope_table), int(store_kv), _ptr(partials), nsplit,
-                      DECODE_ATTENTION_WAVES, chunk_keys, token_seq.data_ptr(), self._stream())
+                      int(unit_offset), _ptr(rope_table), int(store_kv), _ptr(partials),
+                      self._split_counters(n * Hkv, partials), nsplit, -(-max(1, plan.max_context_len) // page_size),
+                      DECODE_ATTENTION_WAVES, token_seq.data_ptr(), self._stream())
         return True
 
     def _attention_fast(self, q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
@@ -679,11 +726,13 @@ class Ops:
         group = H // Hkv
         n_seqs = plan.n_seqs
         if plan.decode_only and group <= 16:
-            nsplit, partials, chunk_keys = self._decode_split(plan, n_seqs, H, Hkv, D, page_size)
+            nsplit, partials = self._decode_split(plan, n_seqs, H, Hkv, D)
+            self._note_attention("mv_attention_decode", plan, q.shape[0], H, Hkv, D, 2, splits=nsplit)
             self.lib.call("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
-                          _ptr(partials), nsplit, DECODE_ATTENTION_WAVES, chunk_keys, token_seq.data_ptr(),
+                          _ptr(partials), self._split_counters(n_seqs * Hkv, partials), nsplit,
+                          -(-max(1, plan.max_context_len) // page_size), DECODE_ATTENTION_WAVES, token_seq.data_ptr(),
                           self._stream())
             return True
         if page_size & (page_size - 1):
@@ -707,6 +756,7 @@ class Ops:
         # the grid leaves compute units waiting for the longest walk (measured on MI355X: faster up
         # to two workgroups per compute unit, slower beyond)
         kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_units * Hkv <= 2 * COMPUTE_UNITS else 1
+        self._note_attention("mv_attention_prefill", plan, q.shape[0], H, Hkv, D, 2)
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, nt, kw, H, Hkv, D,
@@ -751,6 +801,7 @@ class Ops:
                 self._sample_work = torch.empty(SAMPLE_WORK_ROWS * SAMPLE_CHUNKS * 2, dtype=torch.int32,
                                                 device=logits.device)
             work = self._sample_work
+        self._note("mv_sample", M * V * 4, 2 * M * V)
         if advance is not None:
             for t, what in zip(advance, ("next token ids", "positions", "context lengths")):
                 _dev(t, what)

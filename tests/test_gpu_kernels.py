@@ -400,13 +400,14 @@ def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window, ctx_lens, q
 @pytest.mark.parametrize("H,Hkv,D,ps,window", [(16, 8, 128, 16, None), (8, 1, 128, 32, None), (6, 2, 64, 16, 50),
                                                 (16, 1, 64, 16, None)])
 @pytest.mark.parametrize("max_context", [None, 4096, 40000])
-@pytest.mark.parametrize("chunk_keys", [0, 64, 128])
-def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context, chunk_keys):
-    """Decode steps on the MFMA kernels: one token per sequence at very different context
-    lengths, a padding sequence in the middle; the workgroup kernel (chunk_keys 0) with its keys
-    split over 1, a few and many workgroups, and the one-wave kernel with chunks of 64 and 128 keys,
-    planned for the longest context, for a longer one, and (None) for a shorter one than the
-    sequences really have: the last chunk then takes what lies above it."""
+@pytest.mark.parametrize("splits", [None, 1, 3, 16, 64])
+def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context, splits):
+    """Decode steps on the MFMA kernel: one token per sequence at very different context lengths, a
+    padding sequence in the middle; the keys split over as many workgroups as the launch rule
+    chooses (None), over one, a few and many (more than some sequences have blocks of keys: those
+    splits end at once and the others add the partial results up among themselves), planned for the
+    longest context, for a longer one, and (forced splits, no max_context) for a shorter one than
+    the sequences really have: the page ids beyond the plan are then looked up as the keys go."""
     ops = ops_for(torch.bfloat16)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(16)
@@ -440,9 +441,9 @@ def test_attention_decode_kernel(H, Hkv, D, ps, window, max_context, chunk_keys)
     q = q.to(dtype)
     scale = 1.0 / math.sqrt(D)
     out = torch.empty(n, H * D, dtype=dtype, device="cuda")
-    plan = make_plan(q_lens, ctx_lens, max_context_len=max_context if max_context else (200 if chunk_keys else None),
+    plan = make_plan(q_lens, ctx_lens, max_context_len=max_context if max_context else (200 if splits else None),
                      decode_only=True)
-    plan.decode_chunk_keys = chunk_keys
+    plan.decode_splits = splits
     ops.attention(dev(q.view(n, H * D)), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale,
                   window, plan=plan)
     want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
@@ -505,6 +506,53 @@ def test_attention_decode_with_more_workgroups_than_compute_units(H, Hkv, D, fus
             assert torch.equal(vp[page, :, :, slot].float().cpu().double(), v_all[s_][c - 1])
 
 
+@pytest.mark.parametrize("splits", [4, 10, 37])
+def test_attention_decode_splits_agree_over_many_launches(splits):
+    """The workgroups that share a sequence's keys hand their partial results to whichever of them
+    finishes last, through memory and a counter, with no second launch in between. Three hundred
+    launches in a row (other launches in between, so that the caches hold other data) give the very
+    same bits each time and agree with the reference, and every counter is back at zero: a workgroup
+    that read a row before it had arrived, or a counter left standing, would show here."""
+    ops = ops_for(torch.bfloat16)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(77)
+    H, Hkv, D, ps = 16, 8, 128, 16
+    ctx_lens = [1160, 900, 1200, 77, 1024, 1153, 640, 1199]
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    pages_per = [-(-c // ps) for c in ctx_lens]
+    num_pages = sum(pages_per) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, cur = [], 0
+    for n_p in pages_per:
+        tables.append(perm[cur:cur + n_p]); cur += n_p
+    kp, vp = fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype)
+    bt = torch.full((len(tables), max(pages_per)), -1, dtype=torch.int32)
+    for s_, t in enumerate(tables):
+        bt[s_, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    n = len(ctx_lens)
+    positions = torch.tensor([c - 1 for c in ctx_lens], dtype=torch.int32)
+    token_seq = torch.arange(n, dtype=torch.int32)
+    q = torch.randn(n, H, D, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    plan = make_plan([1] * n, ctx_lens, max_context_len=2048, decode_only=True)
+    plan.decode_splits = splits
+    qd, btd, posd, seqd = dev(q.view(n, H * D)), dev(bt), dev(positions), dev(token_seq)
+    outs = [torch.full((n, H * D), float("nan"), dtype=dtype, device="cuda") for _ in range(300)]
+    churn = torch.randn(1 << 22, device="cuda")
+    for it, out in enumerate(outs):
+        ops.attention(qd, out, kp, vp, btd, ps, posd, seqd, H, Hkv, D, scale, None, plan=plan)
+        if it % 7 == 0:
+            churn.mul_(1.0001)
+    torch.cuda.synchronize()
+    want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, None)
+    assert rel_err(outs[0].float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+    first = outs[0].view(torch.int16)
+    differing = [i for i, o in enumerate(outs) if not torch.equal(o.view(torch.int16), first)]
+    assert differing == []
+    assert int(ops._attn_counters.abs().sum()) == 0
+
+
 def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
     """One workgroup walks 18,000 keys (1,125 pages of 16): more page ids than it keeps in LDS, the
     rest are read from the block table as it goes."""
@@ -527,7 +575,7 @@ def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
     cu = dev(torch.tensor([0, 1], dtype=torch.int32))
     seq0 = dev(torch.zeros(1, dtype=torch.int32))
     ops.lib.call("mv_attention_decode", qd.data_ptr(), H * D, out.data_ptr(), H * D, kp.data_ptr(), vp.data_ptr(),
-                 bt.data_ptr(), pages, ps, pos.data_ptr(), cu.data_ptr(), 1, H, Hkv, D, D ** -0.5, -1, 0, 1, 4, 0,
+                 bt.data_ptr(), pages, ps, pos.data_ptr(), cu.data_ptr(), 1, H, Hkv, D, D ** -0.5, -1, 0, 0, 1, 0, 4,
                  seq0.data_ptr(), ops._stream())
     torch.cuda.synchronize()
     want = reference_attention(q.double(), k_all, v_all, torch.tensor([ctx - 1]), torch.tensor([0]), H, Hkv, D ** -0.5, None)
@@ -539,8 +587,8 @@ def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
 @pytest.mark.parametrize("with_norm,with_rope,store", [(True, True, True), (False, True, True), (True, False, True),
                                                        (True, True, False)])
 @pytest.mark.parametrize("max_context", [None, 40000])
-@pytest.mark.parametrize("chunk_keys", [0, 64, 128])
-def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_rope, store, max_context, chunk_keys):
+@pytest.mark.parametrize("splits", [None, 1, 5, 64])
+def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_rope, store, max_context, splits):
     """A decode step from the raw [q | k | v] rows: per-head norm, rotation, cache write and attention
     in one kernel. The slot of the new position holds NaN before (unless the cache is another
     layer's and already complete), the finished key and value afterwards."""
@@ -607,8 +655,8 @@ def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_ro
     # (a sequence without a token, a row that belongs to no sequence)
     out = torch.full((n + 1, H * D), float("nan"), dtype=dtype, device="cuda")
     plan = make_plan([1] * n + [0], [ctx_lens[s] for s in live],
-                     max_context_len=max_context if max_context else (200 if chunk_keys == 64 else None), decode_only=True)
-    plan.decode_chunk_keys = chunk_keys
+                     max_context_len=max_context if max_context else (200 if splits == 5 else None), decode_only=True)
+    plan.decode_splits = splits
     rows = raw if store else raw[:, :H * D].contiguous()
     qkv = dev(torch.cat([rows, torch.full((1, rows.shape[1]), float("nan"), dtype=dtype)]))
     bt_rows = torch.cat([bt[live], torch.full((1, bt.shape[1]), -1, dtype=torch.int32)]).contiguous()
