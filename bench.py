@@ -197,8 +197,14 @@ def emit_kernels(llm, cfg, args) -> int:
     ex = llm.executor
     if args.only in ("all", "decode"):
         k = llm.config.num_scheduler_steps
-        sp = SamplingParams(temperature=0.0, max_tokens=3 * k + 2, ignore_eos=True)
+        sp = SamplingParams(temperature=0.0, max_tokens=llm.config.max_model_len - args.prompt_len - 1, ignore_eos=True)
         reqs = [llm.submit(random_prompt(vocab, args.prompt_len, args.seed + i), sp) for i in range(args.batch)]
+        while any(r.num_completion_tokens == 0 for r in reqs):          # prompts in, first token drawn
+            llm.step()
+        for _ in range(3):                                               # the whole batch decodes: its graphs are recorded
+            llm.step()
+        for r in reqs:
+            r.sampling_params.max_tokens = r.num_completion_tokens
         while llm.has_unfinished():
             llm.step()
         rows = [key for key in ex.graph_ledger if len(key) == 3 and key[0] >= args.batch]

@@ -34,7 +34,7 @@ KERNELS_OF: Dict[str, Tuple[str, int]] = {
     "mv_gemm_skinny_swiglu": (r"\bgemm_skinny_kernel", 1),
     "mv_gemm_ref": (r"\bgemm_nt_kernel", 1),
     "mv_gemm_mid": (r"\bgemm_mid(_reduce)?_kernel", 2),
-    "mv_gemm_lt": (r"^(Cijk_|void hipblaslt|hipblaslt|.*rocblaslt)", 3),
+    "mv_gemm_lt": (r"^((Custom_)?Cijk_|void hipblaslt|hipblaslt|.*rocblaslt)", 3),
     "mv_attention_ref": (r"\battention_ref_kernel", 1),
     "mv_attention_decode": (r"\battention_(decode(_wave)?|merge(_range)?)_kernel", 2),
     "mv_attention_decode_fused": (r"\battention_(decode(_wave)?|merge(_range)?)_kernel", 2),
@@ -102,7 +102,8 @@ def short_name(kernel: str) -> str:
         depth -= ch == ">"
         out.append(ch)
     name = "".join(out).replace("__hip_bfloat16", "bf16").replace(", ", ",")
-    if name.startswith("Cijk_"):
+    if name.startswith(("Cijk_", "Custom_Cijk_")):
+        name = name[name.index("Cijk_"):]
         m = re.search(r"MT(\d+x\d+x\d+)", name)
         kind = name.split("_")[3] if name.count("_") > 3 else ""
         name = f"hipBLASLt {kind} MT{m.group(1)}" if m else name[:40]

@@ -35,6 +35,8 @@ def step_kernels(scale, split=True, rows=8):
 
 def test_steps_are_found_and_priced(tmp_path):
     trace = [("void add_rmsnorm_kernel<float>(float*)", 9.0), ("Cijk_Alik_Bljk_BBS_BH_MT64x64x32_SN", 50.0)]
+    assert roofline.short_name("Custom_Cijk_Alik_Bljk_BBS_BH_Bias_HA_S_SAV_NTD_SK3_UserArgs_MT256x256x64_MI16") == "hipBLASLt BBS MT256x256x64"
+    assert roofline._OURS.search("Custom_Cijk_Alik_Bljk_BBS_BH_Bias") and roofline._OURS.search(trace[1][0])
     for scale in (1.0, 1.2, 0.8, 1.0, 5.0):
         trace += step_kernels(scale)
     trace += step_kernels(1.0, rows=4) * 2             # steps of another batch size: other kernels, left out
