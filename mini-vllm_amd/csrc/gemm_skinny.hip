@@ -31,7 +31,7 @@ union Frag {
 #endif
 #define SK_NORM_CHUNKS 4   // chunks of 512 columns a wave holds in the fused norm's prologue
 #ifndef SK_MIN_ROWS
-#define SK_MIN_ROWS 8      // fewest output columns of a workgroup
+#define SK_MIN_ROWS 4      // fewest output columns of a workgroup
 #endif
 #ifndef SK_WAVE_K
 #define SK_WAVE_K 128      // fewest K elements of a wave
