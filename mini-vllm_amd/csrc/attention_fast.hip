@@ -164,6 +164,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         const bf16* row = fz.qkv + (size_t)t0 * fz.stride;
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
+            if (r * HW > G) break;                 // no head left for any half wave (the same for the whole workgroup)
             const int h = hw + r * HW;
             const bf16* src = h < G ? row + fz.q_off + (size_t)(kvh * G + h) * D + E * hj
                                     : (h == G && fz.store ? row + fz.k_off + (size_t)kvh * D + E * hj : nullptr);
@@ -171,9 +172,12 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
             for (int e = 0; e < E / 2; ++e)
                 raw[r].u[e] = src != nullptr ? reinterpret_cast<const uint32_t*>(src)[e] : 0u;
             if (fz.has_norm && src != nullptr) {
+                if (h < G) fz.qw.at_few<E>(E * hj, head_w[r]);
+                else fz.kw.at_few<E>(E * hj, head_w[r]);
+                if (fz.unit_offset) {
 #pragma unroll
-                for (int e = 0; e < E; ++e)
-                    head_w[r][e] = (h < G ? fz.qw.at(E * hj + e) : fz.kw.at(E * hj + e)) + (fz.unit_offset ? 1.f : 0.f);
+                    for (int e = 0; e < E; ++e) head_w[r][e] += 1.f;
+                }
             }
         }
         if (window < 0) {
@@ -420,6 +424,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         // that will meet it) are prepared by half a wave each and handed round through LDS
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
+            if (r * HW > G) break;
             const int h = hw + r * HW;
             if (h < G || (h == G && wg_owns_new))          // uniform over the half wave, and the exchange stays inside it
                 prepare_head_spread<D>(raw[r].s, hj, fz.has_norm != 0, head_w[r], fz.eps, fz.table != nullptr, rot_c, rot_s,

@@ -56,6 +56,32 @@ struct WeightPtr {
         if (dtype == MV_F32) return ((const float*)p)[i];
         return to_f(((const bf16*)p)[i]);
     }
+    // E (2 or 4) consecutive elements from i (i a multiple of E, the tensor 16-byte aligned): one load
+    template <int E> __device__ __forceinline__ void at_few(size_t i, float (&out)[E]) const {
+        static_assert(E == 2 || E == 4, "at_few: two or four elements");
+        if (dtype == MV_F32) {
+            if constexpr (E == 4) {
+                const float4 a = *reinterpret_cast<const float4*>((const float*)p + i);
+                out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+            } else {
+                const float2 a = *reinterpret_cast<const float2*>((const float*)p + i);
+                out[0] = a.x; out[1] = a.y;
+            }
+        } else {
+            uint32_t w[E / 2];
+            if constexpr (E == 4) {
+                const uint2 u = *reinterpret_cast<const uint2*>((const bf16*)p + i);
+                w[0] = u.x; w[1] = u.y;
+            } else {
+                w[0] = *reinterpret_cast<const uint32_t*>((const bf16*)p + i);
+            }
+#pragma unroll
+            for (int e = 0; e < E / 2; ++e) {
+                out[2 * e] = __uint_as_float(w[e] << 16);
+                out[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+            }
+        }
+    }
     // eight consecutive elements from i (i a multiple of 8, the tensor 16-byte aligned)
     __device__ __forceinline__ void at8(size_t i, float (&out)[8]) const {
         if (dtype == MV_F32) {
