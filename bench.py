@@ -21,6 +21,9 @@ is the one reported (``timed_regions`` says how many there were). One JSON line 
 with the same options and prints one row per kernel of the step with its time, the bytes it has to
 move, its operations and the share of the HBM and MFMA peaks these amount to.
 
+``--only floor`` times a replayed graph of empty kernels: what every dependent launch of a decode step
+costs before it computes anything.
+
 ``--only serve`` runs a continuous-batching workload instead (``--requests`` requests, 256 by
 default, with prompt lengths uniform in 128..2048 and ``--gen-len`` generated tokens each, all
 submitted at once under a budget of ``--token-budget`` tokens a step) and prints its own line:
@@ -188,6 +191,39 @@ def measure_serve(llm, vocab, requests, gen_len, seed, prompt_min=128, prompt_ma
             llm.scheduler.num_preemptions - before)
 
 
+def measure_floor(args) -> int:
+    """What a dependent kernel launch costs inside a replayed graph, whatever the kernel does: a graph of
+    ``--nodes`` empty kernels in a row (170 by default, about the nodes of a decode step of the default
+    shape before fusion), replayed; microseconds per node at several launch sizes."""
+    import torch
+    from minivllm_amd.kernels.ops import dtype_from_name, get_ops
+    ops = get_ops(dtype_from_name(args.dtype))
+    buf = torch.zeros(16, device="cuda:0")
+    points = {}
+    for grid, block in ((1, 64), (256, 64), (256, 256), (256, 512), (1024, 256)):
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            launch = lambda: ops.lib.call("mv_launch_empty", grid, block, buf.data_ptr(), torch.cuda.current_stream().cuda_stream)
+            launch()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for _ in range(args.nodes):
+                    launch()
+            for _ in range(3):
+                g.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(200):
+                g.replay()
+            torch.cuda.synchronize()
+            points[f"{grid}x{block}"] = round((time.perf_counter() - t0) / 200 / args.nodes * 1e6, 3)
+    print(json.dumps({"metric": "microseconds per dependent empty kernel in a replayed graph of %d" % args.nodes,
+                      "value": points["256x256"], "unit": "us", "n_gpus": 1, "higher_is_better": False,
+                      "points": points, "nodes": args.nodes}))
+    return 0
+
+
 def emit_kernels(llm, cfg, args) -> int:
     """Prints, for the step kinds of this run, a table of their kernels: time from the rocprofv3
     kernel trace ``args.emit_kernels``, bytes and operations from what the engine launches."""
@@ -257,9 +293,10 @@ def main() -> int:
                     help="launch the next decode steps before the running ones' tokens are read (default: the engine's)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", "--mode", dest="only", choices=["all", "decode", "prefill", "serve"], default="all",
+    ap.add_argument("--only", "--mode", dest="only", choices=["all", "decode", "prefill", "serve", "floor"], default="all",
                     help="measure one phase alone (for profiling); the line then lacks the other's fields. "
-                         "'serve': the continuous-batching workload")
+                         "'serve': the continuous-batching workload; 'floor': what a dependent launch costs in a graph")
+    ap.add_argument("--nodes", type=int, default=170, help="kernels in the graph of --only floor")
     ap.add_argument("--requests", type=int, default=256, help="requests of the serve workload")
     ap.add_argument("--gen-len", type=int, default=256, help="generated tokens per request of the serve workload")
     ap.add_argument("--token-budget", type=int, default=8192, help="tokens per step of the serve workload")
@@ -282,6 +319,8 @@ def main() -> int:
         return 2
 
     import torch
+    if args.only == "floor":
+        return measure_floor(args)
     shape = SHAPES[args.shape]
     layers_full = shape["num_hidden_layers"]
     layers = args.layers or layers_full

@@ -35,6 +35,17 @@ extern "C" int mv_built_dtypes() {
 
 extern "C" int mv_abi_version() { return 1; }
 
+// A kernel that does nothing: a graph of these, each depending on the one before, shows what a
+// dependent launch costs on the device whatever it computes (the floor of a decode step that is a
+// chain of small kernels).
+__global__ void empty_kernel(const void* unused) {}
+
+extern "C" int mv_launch_empty(int grid, int block, const void* arg, hipStream_t stream) {
+    MV_REQUIRE(grid > 0 && block > 0 && block <= 1024, "launch_empty: bad launch %d x %d", grid, block);
+    hipLaunchKernelGGL(empty_kernel, dim3(grid), dim3(block), 0, stream, arg);
+    return mv_check_launch("launch_empty");
+}
+
 // What a captured graph holds, by kind of node: out[0] kernels, out[1] memsets, out[2] copies,
 // out[3] anything else. The engine admits no memset node in a graph it replays (such nodes have
 // given wrong results on replays after the first); a library call that records one is found here.

@@ -90,6 +90,7 @@ _OPTIONAL_SIGNATURES = {
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                      c_int, c_void_p]),
     "mv_attention_prefill_unit_tokens": (c_int, [c_int, c_int]),
+    "mv_launch_empty": (c_int, [c_int, c_int, c_void_p, c_void_p]),
 }
 
 
