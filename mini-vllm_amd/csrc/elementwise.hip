@@ -318,6 +318,49 @@ extern "C" int mv_rmsnorm(const void* in, long in_stride, const void* weight, in
 }
 
 // ---------------------------------------------------------------------------------------
+// Rows that a product left weighted but not yet normalised (gemm_skinny.hip, the FOLD variant):
+//   out[m][k] = weighted[m][k] / sqrt(sum_p partial[m][p] / width + eps).
+// For whatever comes behind such a norm and does not divide its own output rows. The partial
+// sums are added in the order the SCALED product adds them (it depends on their number alone).
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void scale_rows_kernel(const T* __restrict__ weighted, long ldw, const float* __restrict__ partial, int P,
+                                  float eps, T* __restrict__ out, long ldo, int width) {
+    __shared__ float sh_rinv;
+    const int m = blockIdx.x;
+    if (threadIdx.x < MV_WAVE) {
+        float t = 0.f;
+        if (P <= 64) {
+            if (threadIdx.x < 8)
+                for (int p = threadIdx.x; p < P; p += 8) t += partial[(size_t)m * P + p];
+            t += __shfl_xor(t, 1, MV_WAVE);
+            t += __shfl_xor(t, 2, MV_WAVE);
+            t += __shfl_xor(t, 4, MV_WAVE);
+        } else {
+            for (int p = threadIdx.x; p < P; p += MV_WAVE) t += partial[(size_t)m * P + p];
+            t = wave_sum(t);
+        }
+        if (threadIdx.x == 0) sh_rinv = rsqrtf(t / (float)width + eps);
+    }
+    __syncthreads();
+    const float rinv = sh_rinv;
+    for (int k = threadIdx.x; k < width; k += blockDim.x)
+        out[(size_t)m * ldo + k] = from_f<T>(to_f(weighted[(size_t)m * ldw + k]) * rinv);
+}
+
+extern "C" int mv_scale_rows(const void* weighted, long ldw, const float* partial, int P, float eps, void* out, long ldo,
+                             int dtype, int M, int width, hipStream_t stream) {
+    MV_REQUIRE(M >= 0 && width > 0 && P > 0 && eps > 0.f && ldw >= width && ldo >= width,
+               "scale_rows: bad sizes M=%d width=%d P=%d", M, width, P);
+    MV_REQUIRE(weighted != nullptr && partial != nullptr && out != nullptr, "scale_rows: null argument");
+    if (M == 0) return 0;
+    MV_DISPATCH_T(dtype, "scale_rows",
+                    hipLaunchKernelGGL(scale_rows_kernel<T>, dim3(M), dim3(256), 0, stream, (const T*)weighted, ldw,
+                                       partial, P, eps, (T*)out, ldo, width));
+    return mv_check_launch("scale_rows");
+}
+
+// ---------------------------------------------------------------------------------------
 // Rotary table: table[pos, 0:R/2] = cos(pos * inv_freq), table[pos, R/2:R] = sin(...).
 // The angle is the float product of the float position and the float inverse frequency.
 // ---------------------------------------------------------------------------------------

@@ -12,6 +12,14 @@
 //
 // A fused variant computes the gated activation of a feed-forward in the same pass:
 //     out[M, I] = silu(A Wg^T) * (A Wu^T)  with Wg = W[0:I], Wu = W[I:2I].
+//
+// Two more variants take a residual add and an RMSNorm between two products apart, for steps
+// with too many rows to normalise them in every workgroup of the second product. The product in
+// front of the norm (FOLD) owns each element of its output once, so it adds it to the residual
+// there, leaves x * weight (rounded to bf16, not yet divided by the row's root mean square) and
+// the sum of x^2 over its own columns; the product behind the norm (SCALED) multiplies with
+// those rows and divides each output row by the root mean square, which it gets from the
+// partial sums: (x w / rms) W^T = (x w) W^T / rms.
 #include "dispatch.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -51,6 +59,24 @@ struct NormInput {
     int unit_offset;
 };
 
+// What the FOLD and SCALED variants need beside the product (EPI below).
+struct RowsInput {
+    float* resid;            // FOLD: [M, N] float, updated in place: resid += bf16(product)
+    long ldr;
+    WeightPtr weight;        // FOLD: [N], the weight of the norm that follows
+    int unit_offset;
+    bf16* weighted;          // FOLD: [M, N] out: bf16(resid * weight)
+    long ldw;
+    float* partial;          // FOLD: [M, P] out, P = workgroups along N: sums of resid^2 over a workgroup's columns
+                             // SCALED: the same array, read: row m of the input is to be divided by
+                             //         sqrt(sum_p partial[m][p] / width + eps)
+    int P;
+    float eps;               // SCALED
+    int width;               // SCALED: elements of an input row (the norm's size)
+};
+
+enum { EPI_NONE = 0, EPI_FOLD = 1, EPI_SCALED = 2 };
+
 // R: 16-row weight tiles per workgroup; TM: 16-token tiles (M <= 16 * TM); SWIGLU: R == 2 and
 // the two tiles are the gate rows and the up rows of the same output columns.
 // NORM (TM == 1): the activations are not read from A but made here:
@@ -58,12 +84,12 @@ struct NormInput {
 // Every workgroup normalises the (few) rows for itself into LDS, which costs less than a kernel
 // launch; workgroup 0 also writes x to resid_out (a buffer other than resid_in: the other
 // workgroups still read that one).
-template <int R, int TM, bool SWIGLU, bool NORM, typename TC>
+template <int R, int TM, bool SWIGLU, bool NORM, typename TC, int EPI = EPI_NONE>
 __global__ void __launch_bounds__(64 * SK_MAX_WAVES)
 gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W, const bf16* __restrict__ bias,
                    TC* __restrict__ C, long ldc, int M, int N, int K, int groups, int blocks, int rows,
-                   NormInput norm) {
-    extern __shared__ float red[];  // [S - 1][R * TM][64][4], then (NORM) bf16 [M][K + 8]
+                   NormInput norm, RowsInput fold) {
+    extern __shared__ float red[];  // [S - 1][R * TM][64][4], then (NORM) bf16 [M][K + 8], or (SCALED) float [16 * TM]
     // The tokens may be dealt out to `groups` workgroups per weight tile (16 * TM tokens each): with
     // few weight tiles that fills more compute units, and each unit pulls fewer activation rows.
     // Workgroups go to the chip's eight dies in turn, so the groups of one tile are given ids that
@@ -76,6 +102,11 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
         if (block >= blocks) return;
         A += (size_t)tg * 16 * TM * lda;
         C += (size_t)tg * 16 * TM * ldc;
+        if (EPI == EPI_FOLD) {
+            fold.resid += (size_t)tg * 16 * TM * fold.ldr;
+            fold.weighted += (size_t)tg * 16 * TM * fold.ldw;
+        }
+        if (EPI != EPI_NONE) fold.partial += (size_t)tg * 16 * TM * fold.P;
         M -= tg * 16 * TM;
         if (M <= 0) return;
         if (M > 16 * TM) M = 16 * TM;
@@ -228,6 +259,60 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 #pragma unroll
         for (int t = 0; t < TM; ++t) acc[r][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
+    // SCALED: one over the root mean square of each of the workgroup's rows, from the partial sums
+    // the product in front left; a wave takes every S-th row and adds a row's partial sums in a
+    // fixed order (the same in every workgroup). Read after the barrier behind the main loop.
+    float* sh_rinv = red + (size_t)(S - 1) * R * TM * 256;
+    // The sums of a row are added in an order that depends on nothing but their number P. Up to 64
+    // of them: eight lanes a row, lane j of them adds the sums j, j + 8, ... in order, then the eight
+    // are added pairwise; a thread's first row is asked for here and added up behind the main loop,
+    // so that neither the sums nor the weights wait for each other. More than 64: a wave takes every
+    // S-th row, lane j adds the sums j, j + 64, ..., then the lanes are added pairwise; the first
+    // eight loads of a wave are asked for here.
+    const bool scaled_narrow = EPI == EPI_SCALED && fold.P <= 64;
+    const int scaled_chunks = EPI == EPI_SCALED ? (fold.P + MV_WAVE - 1) / MV_WAVE : 1;
+    float scaled_first[EPI == EPI_SCALED ? 8 : 1];
+    if (EPI == EPI_SCALED) {
+        if (scaled_narrow) {
+            const int m = threadIdx.x / 8;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int p = threadIdx.x % 8 + 8 * u;
+                scaled_first[u] = (m < M && p < fold.P) ? fold.partial[(size_t)m * fold.P + p] : 0.f;
+            }
+        } else {
+            int m = wave, c = 0;                   // (no division: it would stand in front of the first weight load)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int p = lane + MV_WAVE * c;
+                scaled_first[u] = (m < M && p < fold.P) ? fold.partial[(size_t)m * fold.P + p] : 0.f;
+                if (++c == scaled_chunks) {
+                    c = 0;
+                    m += S;
+                }
+            }
+        }
+    }
+    // FOLD: the residual and the norm's weights of the elements this workgroup will own are asked
+    // for now (by the wave that stores them), not after the product
+    float4 fold_resid[EPI == EPI_FOLD ? R : 1][EPI == EPI_FOLD ? TM : 1];
+    float fold_w[EPI == EPI_FOLD ? R : 1][4];
+    if (EPI == EPI_FOLD && wave == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int col0 = n_base + 16 * r + 4 * g;
+            const bool live = col0 < n_end;      // N, the workgroup's columns and col0 are multiples of four
+            if (live) fold.weight.at_few<4>(col0, fold_w[r]);
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                const int tok = 16 * t + i;
+                fold_resid[r][t] = (live && tok < M)
+                                       ? *reinterpret_cast<const float4*>(fold.resid + (size_t)tok * fold.ldr + col0)
+                                       : float4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    }
+
     // Two register stages of U k-steps each: while the MFMAs of one stage run, the loads of the
     // next are in flight, so a wave always has a stage's worth of weight bytes on the way.
     struct Stage {
@@ -289,6 +374,40 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
                 acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[r].v, a[t].v, acc[r][t], 0, 0, 0);
     }
 
+    if (EPI == EPI_SCALED && scaled_narrow) {
+        for (int m = threadIdx.x / 8; m < M; m += blockDim.x / 8) {
+            float t = 0.f;
+            if (m == (int)threadIdx.x / 8) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) t += scaled_first[u];
+            } else {
+                for (int p = threadIdx.x % 8; p < fold.P; p += 8) t += fold.partial[(size_t)m * fold.P + p];
+            }
+            t += __shfl_xor(t, 1, MV_WAVE);
+            t += __shfl_xor(t, 2, MV_WAVE);
+            t += __shfl_xor(t, 4, MV_WAVE);
+            if (threadIdx.x % 8 == 0) sh_rinv[m] = rsqrtf(t / (float)fold.width + fold.eps);
+        }
+    } else if (EPI == EPI_SCALED) {
+        int item = 0;
+        for (int m = wave; m < M; m += S) {
+            float t = 0.f;
+            for (int c = 0; c < scaled_chunks; ++c, ++item) {
+                float v;
+                if (item < 8) {
+                    v = scaled_first[0];
+#pragma unroll
+                    for (int u = 1; u < 8; ++u) v = item == u ? scaled_first[u] : v;
+                } else {
+                    const int p = lane + MV_WAVE * c;
+                    v = p < fold.P ? fold.partial[(size_t)m * fold.P + p] : 0.f;
+                }
+                t += v;
+            }
+            t = wave_sum(t);
+            if (lane == 0) sh_rinv[m] = rsqrtf(t / (float)fold.width + fold.eps);
+        }
+    }
     // partial tiles of waves 1 .. S-1 go through LDS; wave 0 adds them in order
     if (wave > 0) {
         float* dst = red + ((size_t)(wave - 1) * R * TM) * 256;
@@ -311,6 +430,49 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
                 for (int e = 0; e < 4; ++e) acc[r][t][e] += src[(r * TM + t) * 256 + e * 64 + lane];
     }
 
+    if (EPI == EPI_SCALED) {
+#pragma unroll
+        for (int t = 0; t < TM; ++t) {
+            const float rinv = 16 * t + i < M ? sh_rinv[16 * t + i] : 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][t] *= rinv;
+        }
+    }
+    if (EPI == EPI_FOLD) {
+        // x = resid + bf16(product (+ bias)) (the sum the stand-alone add makes from the rounded
+        // product); resid = x; weighted = bf16(x * w); partial[tok][block] = sum of x^2 over this
+        // workgroup's columns (the four lane groups of a token, then its R tiles, in a fixed order)
+#pragma unroll
+        for (int t = 0; t < TM; ++t) {
+            const int tok = 16 * t + i;
+            float ssq = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int col0 = n_base + 16 * r + 4 * g;
+                if (tok < M && col0 < n_end) {
+                    const float old4[4] = {fold_resid[r][t].x, fold_resid[r][t].y, fold_resid[r][t].z, fold_resid[r][t].w};
+                    float x[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float v = acc[r][t][e];
+                        if (bias) v += to_f(bias[col0 + e]);
+                        x[e] = old4[e] + __uint_as_float((uint32_t)f32_to_bf16_bits(v) << 16);
+                        ssq += x[e] * x[e];
+                    }
+                    *reinterpret_cast<float4*>(fold.resid + (size_t)tok * fold.ldr + col0) = float4{x[0], x[1], x[2], x[3]};
+                    const float off = fold.unit_offset ? 1.f : 0.f;
+                    uint2 packed;
+                    packed.x = f32x2_to_bf16x2_bits(x[0] * (fold_w[r][0] + off), x[1] * (fold_w[r][1] + off));
+                    packed.y = f32x2_to_bf16x2_bits(x[2] * (fold_w[r][2] + off), x[3] * (fold_w[r][3] + off));
+                    *reinterpret_cast<uint2*>(fold.weighted + (size_t)tok * fold.ldw + col0) = packed;
+                }
+            }
+            ssq += __shfl_xor(ssq, 16, MV_WAVE);
+            ssq += __shfl_xor(ssq, 32, MV_WAVE);
+            if (g == 0 && tok < M) fold.partial[(size_t)tok * fold.P + block] = ssq;
+        }
+        return;
+    }
     if (SWIGLU) {
 #pragma unroll
         for (int t = 0; t < TM; ++t) {
@@ -343,9 +505,10 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     }
 }
 
-static size_t skinny_lds_bytes(int S, int R, int TM, bool with_norm, int M, int K) {
+static size_t skinny_lds_bytes(int S, int R, int TM, bool with_norm, int M, int K, bool scaled = false) {
     size_t lds = (size_t)(S - 1) * R * TM * 256 * sizeof(float);
     if (with_norm) lds += (size_t)M * (K + 8) * sizeof(uint16_t) + (size_t)M * ((K + 511) / 512) * sizeof(float);
+    if (scaled) lds += (size_t)16 * TM * sizeof(float);
     return lds;
 }
 
@@ -372,16 +535,16 @@ static int pick_rows(int N, int most) {
     return rows;
 }
 
-template <int R, int TM, bool SWIGLU, typename TC>
+template <int R, int TM, bool SWIGLU, typename TC, int EPI = EPI_NONE>
 static void launch_skinny(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N,
-                          int K, int S, int rows, hipStream_t stream) {
+                          int K, int S, int rows, hipStream_t stream, const RowsInput& fold = RowsInput{}) {
     const int blocks = skinny_blocks(N, rows);
     const int groups = (M + 16 * TM - 1) / (16 * TM);
     const int grid = groups > 1 ? (blocks + 7) / 8 * 8 * groups : blocks;
-    const size_t lds = skinny_lds_bytes(S, R, TM, false, M, K);
-    hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC>), dim3(grid), dim3(64 * S), lds, stream,
+    const size_t lds = skinny_lds_bytes(S, R, TM, false, M, K, EPI == EPI_SCALED);
+    hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC, EPI>), dim3(grid), dim3(64 * S), lds, stream,
                        (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, groups, blocks,
-                       rows, NormInput{});
+                       rows, NormInput{}, fold);
 }
 
 template <int R, bool SWIGLU, typename TC>
@@ -392,7 +555,7 @@ static void launch_skinny_norm(const NormInput& norm, const void* W, const void*
     const size_t lds = skinny_lds_bytes(S, R, 1, true, M, K);
     hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC>), dim3(blocks), dim3(64 * S), lds, stream,
                        (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K, 1, blocks,
-                       rows, norm);
+                       rows, norm, RowsInput{});
 }
 
 static int pick_waves(int K) {
@@ -402,9 +565,9 @@ static int pick_waves(int K) {
     return s;
 }
 
-template <int R, bool SWIGLU, typename TC>
+template <int R, bool SWIGLU, typename TC, int EPI = EPI_NONE>
 static int dispatch_tm(const void* A, long lda, const void* W, const void* bias, void* C, long ldc, int M, int N, int K,
-                       int S, int rows, hipStream_t stream) {
+                       int S, int rows, hipStream_t stream, const RowsInput& fold = RowsInput{}) {
     // Token tiles per workgroup: all of them (the weights pass each compute unit once), or fewer
     // with the tokens dealt out to several workgroups per weight tile. A compute unit pulls
     // R + TM operand rows of 16 per workgroup it runs; the choice with the least per unit wins.
@@ -421,10 +584,10 @@ static int dispatch_tm(const void* A, long lda, const void* W, const void* bias,
             best_tm = tm;
         }
     }
-    if (best_tm == 1) launch_skinny<R, 1, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
-    else if (best_tm == 2) launch_skinny<R, 2, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
-    else if (best_tm == 3) launch_skinny<R, 3, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
-    else launch_skinny<R, 4, SWIGLU, TC>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
+    if (best_tm == 1) launch_skinny<R, 1, SWIGLU, TC, EPI>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream, fold);
+    else if (best_tm == 2) launch_skinny<R, 2, SWIGLU, TC, EPI>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream, fold);
+    else if (best_tm == 3) launch_skinny<R, 3, SWIGLU, TC, EPI>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream, fold);
+    else launch_skinny<R, 4, SWIGLU, TC, EPI>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream, fold);
     return 0;
 }
 
@@ -437,6 +600,22 @@ static int check_skinny(const char* what, const void* A, long lda, const void* W
     return 0;
 }
 
+// Waves per workgroup, weight tiles per workgroup and output columns per workgroup of the plain product.
+static void skinny_shape(int M, int N, int K, int& S, int& R, int& rows) {
+    S = pick_waves(K);
+    const int tiles = (N + 15) / 16;
+    const int TM = (M + 15) / 16;
+    // more row tiles per workgroup reuse the activation registers; keep at least ~512 workgroups
+    // and the partial tiles of the waves within 56 KiB of LDS
+    R = tiles >= 2048 ? 4 : (tiles >= 1024 ? 2 : 1);
+    while (R > 1 && (size_t)(S - 1) * R * TM * 1024 > 56 * 1024) R /= 2;
+    rows = 16 * R;
+    if (R == 1 && M <= 16) {
+        rows = pick_rows(N, 32);
+        R = rows > 16 ? 2 : 1;
+    }
+}
+
 // c_dtype: MV_BF16 or MV_F32.
 extern "C" int mv_gemm_skinny(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, long ldc,
                               int c_dtype, int M, int N, int K, hipStream_t stream) {
@@ -444,18 +623,8 @@ extern "C" int mv_gemm_skinny(const void* A, long lda, const void* W, long ldw, 
     MV_REQUIRE(ldw == K, "gemm_skinny: the weight must be contiguous (ldw=%ld, K=%d)", ldw, K);
     MV_REQUIRE(c_dtype == MV_F32 || c_dtype == MV_BF16, "gemm_skinny: bad output dtype %d", c_dtype);
     if (M == 0) return 0;
-    const int S = pick_waves(K);
-    const int tiles = (N + 15) / 16;
-    const int TM = (M + 15) / 16;
-    // more row tiles per workgroup reuse the activation registers; keep at least ~512 workgroups
-    // and the partial tiles of the waves within 56 KiB of LDS
-    int R = tiles >= 2048 ? 4 : (tiles >= 1024 ? 2 : 1);
-    while (R > 1 && (size_t)(S - 1) * R * TM * 1024 > 56 * 1024) R /= 2;
-    int rows = 16 * R;
-    if (R == 1 && M <= 16) {
-        rows = pick_rows(N, 32);
-        R = rows > 16 ? 2 : 1;
-    }
+    int S, R, rows;
+    skinny_shape(M, N, K, S, R, rows);
     int rc = 0;
     if (c_dtype == MV_F32) {
         if (R == 4) rc = dispatch_tm<4, false, float>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream);
@@ -468,6 +637,69 @@ extern "C" int mv_gemm_skinny(const void* A, long lda, const void* W, long ldw, 
     }
     if (rc) return rc;
     return mv_check_launch("gemm_skinny");
+}
+
+// The product in front of a residual add and an RMSNorm, with both folded into it (see the top of
+// the file): resid[M, N] (float) += bf16(A W^T (+ bias)); weighted[M, N] = bf16(resid * norm_weight
+// (+ 1 with unit_offset)); partial[M, P] = sums of resid^2 over the columns of each of the P
+// workgroups along N, P = mv_gemm_skinny_fold_parts(M, N, K). The product behind the norm
+// (mv_gemm_skinny_scaled), or mv_scale_rows, turns `weighted` and `partial` into normalised rows.
+extern "C" int mv_gemm_skinny_fold_parts(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    int S, R, rows;
+    skinny_shape(M, N, K, S, R, rows);
+    return skinny_blocks(N, rows);
+}
+
+extern "C" int mv_gemm_skinny_fold(const void* A, long lda, const void* W, const void* bias, float* resid, long ldr,
+                                   const void* norm_weight, int norm_weight_dtype, int unit_offset, void* weighted,
+                                   long ldw, float* partial, int P, int M, int N, int K, hipStream_t stream) {
+    if (int rc = check_skinny("gemm_skinny_fold", A, lda, W, ldw, M, N, K)) return rc;
+    MV_REQUIRE(resid != nullptr && weighted != nullptr && partial != nullptr && ldr >= N,
+               "gemm_skinny_fold: the residual, the weighted rows or the partial sums are missing (ldr=%ld)", ldr);
+    MV_REQUIRE(mv_valid_dtype(norm_weight_dtype) && norm_weight != nullptr && ((uintptr_t)norm_weight % 16) == 0,
+               "gemm_skinny_fold: the norm weight is missing, of an unknown type or not 16-byte aligned");
+    MV_REQUIRE(N % 4 == 0 && ldr % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weighted % 8) == 0,
+               "gemm_skinny_fold: N=%d and the row pitches %ld / %ld must be multiples of four, the rows aligned", N, ldr, ldw);
+    if (M == 0) return 0;
+    int S, R, rows;
+    skinny_shape(M, N, K, S, R, rows);
+    MV_REQUIRE(P == skinny_blocks(N, rows), "gemm_skinny_fold: %d partial sums a row, the launch makes %d", P,
+               skinny_blocks(N, rows));
+    RowsInput fold{resid, ldr, WeightPtr{norm_weight, norm_weight_dtype}, unit_offset, (bf16*)weighted, ldw, partial,
+                   P, 0.f, 0};
+    int rc = 0;
+    if (R == 4) rc = dispatch_tm<4, false, bf16, EPI_FOLD>(A, lda, W, bias, nullptr, 0, M, N, K, S, rows, stream, fold);
+    else if (R == 2) rc = dispatch_tm<2, false, bf16, EPI_FOLD>(A, lda, W, bias, nullptr, 0, M, N, K, S, rows, stream, fold);
+    else rc = dispatch_tm<1, false, bf16, EPI_FOLD>(A, lda, W, bias, nullptr, 0, M, N, K, S, rows, stream, fold);
+    if (rc) return rc;
+    return mv_check_launch("gemm_skinny_fold");
+}
+
+// The product behind such a norm: C = (A W^T) / rms (+ bias), or the gated pair
+// silu(g / rms) * (u / rms), where A = the weighted rows [M, K] and rms[m] =
+// sqrt(sum_p partial[m][p] / K + eps). bf16 out.
+extern "C" int mv_gemm_skinny_scaled(const void* A, long lda, const void* W, const void* bias, void* C, long ldc,
+                                     const float* partial, int P, float eps, int M, int N, int K, int swiglu,
+                                     hipStream_t stream) {
+    if (int rc = check_skinny("gemm_skinny_scaled", A, lda, W, ldc, M, N, K)) return rc;
+    MV_REQUIRE(partial != nullptr && P > 0 && eps > 0.f, "gemm_skinny_scaled: bad partial sums (P=%d) or eps", P);
+    if (M == 0) return 0;
+    RowsInput fold{nullptr, 0, WeightPtr{nullptr, MV_BF16}, 0, nullptr, 0, const_cast<float*>(partial), P, eps, K};
+    int rc = 0;
+    if (swiglu) {
+        const int S = pick_waves(K);
+        rc = dispatch_tm<2, true, bf16, EPI_SCALED>(A, lda, W, nullptr, C, ldc, M, N, K, S,
+                                                    M <= 16 ? pick_rows(N, 16) : 16, stream, fold);
+    } else {
+        int S, R, rows;
+        skinny_shape(M, N, K, S, R, rows);
+        if (R == 4) rc = dispatch_tm<4, false, bf16, EPI_SCALED>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream, fold);
+        else if (R == 2) rc = dispatch_tm<2, false, bf16, EPI_SCALED>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream, fold);
+        else rc = dispatch_tm<1, false, bf16, EPI_SCALED>(A, lda, W, bias, C, ldc, M, N, K, S, rows, stream, fold);
+    }
+    if (rc) return rc;
+    return mv_check_launch("gemm_skinny_scaled");
 }
 
 // out[M, I] = silu(A Wgu[0:I]^T) * (A Wgu[I:2I]^T), bf16 in and out.

@@ -32,6 +32,9 @@ KERNELS_OF: Dict[str, Tuple[str, int]] = {
     "mv_gemm_skinny": (r"\bgemm_skinny_kernel", 1),
     "mv_gemm_skinny_norm": (r"\bgemm_skinny_kernel", 1),
     "mv_gemm_skinny_swiglu": (r"\bgemm_skinny_kernel", 1),
+    "mv_gemm_skinny_fold": (r"\bgemm_skinny_kernel", 1),
+    "mv_gemm_skinny_scaled": (r"\bgemm_skinny_kernel", 1),
+    "mv_scale_rows": (r"\bscale_rows_kernel", 1),
     "mv_gemm_ref": (r"\bgemm_nt_kernel", 1),
     "mv_gemm_mid": (r"\bgemm_mid(_reduce)?_kernel", 2),
     "mv_gemm_lt": (r"^((Custom_)?Cijk_|void hipblaslt|hipblaslt|.*rocblaslt)", 3),

@@ -58,6 +58,15 @@ _OPTIONAL_SIGNATURES = {
     "mv_gemm_skinny": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int,
                                c_int, c_int, c_int, c_void_p]),
     "mv_gemm_skinny_swiglu": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),
+    "mv_gemm_skinny_fold_parts": (c_int, [c_int, c_int, c_int]),
+    # A, lda, W, bias, resid, ldr, norm_weight, norm_weight_dtype, unit_offset, weighted, ldw, partial, P, M, N, K, stream
+    "mv_gemm_skinny_fold": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_int,
+                                    c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    # A, lda, W, bias, C, ldc, partial, P, eps, M, N, K, swiglu, stream
+    "mv_gemm_skinny_scaled": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_float,
+                                      c_int, c_int, c_int, c_int, c_void_p]),
+    # weighted, ldw, partial, P, eps, out, ldo, dtype, M, width, stream
+    "mv_scale_rows": (c_int, [c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_skinny_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
                                     c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_lt_workspace": (c_long, []),

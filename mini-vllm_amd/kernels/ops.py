@@ -112,6 +112,36 @@ class SplitSum:
             self.ops._split_pending = None
 
 
+class WeightedRows:
+    """What ``Ops.gemm(..., fold=...)`` returns when it took the residual add and the norm into its
+    product: the rows of the new residual times the norm's weight (``weighted``, the activation
+    type) and, per row, ``P`` partial sums of squares. ``Ops.gemm`` / ``Ops.gemm_swiglu`` take it as
+    their input and divide their output rows by the root mean square; ``materialize()`` gives the
+    normalised rows to anything else. Used once."""
+    is_weighted_rows = True
+
+    def __init__(self, ops: "Ops", fold, P: int):
+        self.ops, self.norm = ops, fold.norm
+        self.weighted, self.partial, self.P, self.eps = fold.weighted, fold.partial, P, float(fold.eps)
+        self.normed = fold.normed
+        self.shape = fold.weighted.shape
+        self.used = False
+        self._done = False
+
+    def take(self) -> None:
+        if self.used:
+            raise RuntimeError("half-normalised rows were used twice")
+        self.used = True
+
+    def materialize(self) -> torch.Tensor:
+        """Runs the second half of the norm (once) and returns the normalised rows."""
+        if not self._done:
+            self.take()
+            self.ops.scale_rows(self.weighted, self.partial, self.P, self.eps, self.normed)
+            self._done = True
+        return self.normed
+
+
 class Ops:
     def __init__(self, dtype: torch.dtype):
         if dtype not in _CODES:
@@ -334,7 +364,7 @@ class Ops:
 
     # ------------------------------------------------------------------------------------
     def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
-             exact: bool = False, defer_sum: bool = False) -> Optional["SplitSum"]:
+             exact: bool = False, defer_sum: bool = False, fold=None):
         """out[M, N] = a[M, K] @ w[N, K]^T (+ bias). ``out`` is the activation type or float32.
 
         With ``defer_sum`` the caller can take a ``SplitSum`` instead of the finished ``out``: when
@@ -348,9 +378,18 @@ class Ops:
         ``exact`` is set or when no other kernel takes the shape.
 
         ``a`` may be a pending norm (parts.base.PendingNorm): then the residual add, the norm and
-        the product run as one kernel when the step has at most 16 rows, else the norm runs first."""
+        the product run as one kernel when the step has at most 16 rows, else the norm runs first.
+        ``a`` may also be ``WeightedRows``: the output rows are then divided by the rows' root mean
+        square where the weight-streaming kernel takes the shape, else the rows are normalised first.
+
+        ``fold`` (parts.base.NormFold) offers the residual add and the norm behind this product: when
+        the weight-streaming kernel takes the shape it adds the product to the residual, leaves the
+        rows weighted for the norm, and ``WeightedRows`` is returned; ``out`` is not written then."""
         if not isinstance(a, torch.Tensor):
-            if not exact and self._gemm_fused_norm(a, w, out, bias, swiglu=False):
+            if isinstance(a, WeightedRows):
+                if not exact and self._gemm_scaled(a, w, out, bias, swiglu=False):
+                    return None
+            elif not exact and self._gemm_fused_norm(a, w, out, bias, swiglu=False):
                 return None
             a = a.materialize()
         self._act(a, "gemm input"); _dev(w, "gemm weight"); _dev(out, "gemm output")
@@ -386,6 +425,16 @@ class Ops:
             if M > SKINNY_MAX_M and self._library_serves(out) and \
                     self._library_allowed(M, N, K, bias is not None, out.dtype) and self._library_product(a, w, bias, out):
                 return
+            if fold is not None and self._fold_serves(fold, out, M, N):
+                P = int(self.lib.dll.mv_gemm_skinny_fold_parts(M, N, K))
+                resid = fold.stream.resid
+                self._note("mv_gemm_skinny_fold", M * K * 2 + N * K * 2 + M * N * (8 + 2) + M * P * 4, 2 * M * N * K + 4 * M * N)
+                self.lib.call("mv_gemm_skinny_fold", a.data_ptr(), lda, w.data_ptr(), _ptr(bias), resid.data_ptr(),
+                              resid.stride(0) if M > 1 else N, fold.weight.data_ptr(),
+                              _weight_code(fold.weight, "norm weight"), int(fold.unit_offset), fold.weighted.data_ptr(),
+                              fold.weighted.stride(0) if M > 1 else N, fold.partial.data_ptr(), P, M, N, K,
+                              self._stream())
+                return WeightedRows(self, fold, P)
             # more rows than one workgroup takes are dealt out to groups of workgroups by the kernel
             for m0 in range(0, M, SKINNY_LAUNCH_ROWS):
                 m = min(SKINNY_LAUNCH_ROWS, M - m0)
@@ -497,6 +546,73 @@ class Ops:
             return False
         return (N * K >= MID_ALWAYS_WEIGHT and K >= MID_ALWAYS_K) or (N * K >= MID_MIN_WEIGHT and M >= MID_MIN_M)
 
+    def can_fold_norm(self, rows: int, width: int, consumer=None) -> bool:
+        """Whether a residual add and a norm over ``rows`` x ``width`` may be offered to the product in
+        front of them (``gemm(..., fold=...)``): steps of up to SKINNY_MAX_M rows that are too large
+        for the fused add + norm + product kernel, when the product behind the norm (``consumer`` =
+        (weight rows, weight columns, gated)) is one the weight-streaming kernel takes — behind any
+        other the rows would have to be normalised by a kernel of their own, and nothing is gained
+        (32B sizes, where gate/up goes to the library: 2 % slower)."""
+        if not (self.use_fast_kernels and self.dtype == torch.bfloat16 and self.lib.has("mv_gemm_skinny_fold")
+                and self.lib.has("mv_gemm_skinny_scaled") and 0 < rows <= SKINNY_MAX_M and width % 4 == 0
+                and not self.can_fuse_norm(rows, width)):
+            return False
+        if consumer is None:
+            return True
+        n, k, gated = consumer
+        return (k == width and k % 32 == 0 and not (gated and n % 2)
+                and not (self.wants_mid(rows, n, k) and self.lib.has("mv_gemm_mid"))
+                and not self.prefers_library(rows, n, k, gated=gated))
+
+    def _fold_serves(self, fold, out: torch.Tensor, M: int, N: int) -> bool:
+        resid = fold.stream.resid
+        return (M <= SKINNY_MAX_M and out.dtype == self.dtype and self.lib.has("mv_gemm_skinny_fold")
+                and resid.dtype == torch.float32 and resid.shape == (M, N) and resid.stride(1) == 1
+                and fold.weight.numel() == N and fold.weight.is_contiguous()
+                and fold.weighted.shape == (M, N) and fold.weighted.stride(1) == 1 and fold.weighted.dtype == self.dtype
+                and N % 4 == 0 and (M == 1 or (resid.stride(0) % 4 == 0 and fold.weighted.stride(0) % 4 == 0))
+                and resid.data_ptr() % 16 == 0 and fold.weighted.data_ptr() % 8 == 0 and fold.weight.data_ptr() % 16 == 0
+                and fold.partial.numel() >= M * ((N + 3) // 4) and fold.stream.delta is None
+                and fold.stream.weighted is None)
+
+    def _gemm_scaled(self, rows: "WeightedRows", w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor],
+                     swiglu: bool) -> bool:
+        """The product (or gated pair) behind a folded norm: output rows divided by the input rows' root
+        mean square; False if the shape is not taken (nothing has been done then)."""
+        a = rows.weighted
+        M, K = a.shape
+        if (not self.use_fast_kernels or not self.lib.has("mv_gemm_skinny_scaled") or M == 0 or M > SKINNY_MAX_M
+                or w.dtype != torch.bfloat16 or not w.is_contiguous() or w.shape[1] != K or K % 32
+                or a.stride(1) != 1 or (M > 1 and a.stride(0) % 8) or a.data_ptr() % 16
+                or out.stride(1) != 1 or out.dtype != torch.bfloat16 or (swiglu and w.shape[0] % 2)):
+            return False
+        N = w.shape[0] // 2 if swiglu else w.shape[0]
+        if out.shape != (M, N):
+            return False
+        if self.wants_mid(M, w.shape[0], K) and self.lib.has("mv_gemm_mid"):
+            return False
+        if self.prefers_library(M, w.shape[0], K, gated=swiglu) and self._library_allowed(M, w.shape[0], K, bias is not None):
+            return False
+        if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N):
+            return False
+        rows.take()
+        self._note("mv_gemm_skinny_scaled", self._size(a, w, out) + M * rows.P * 4, 2 * M * w.shape[0] * K)
+        self.lib.call("mv_gemm_skinny_scaled", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias),
+                      out.data_ptr(), out.stride(0) if M > 1 else N, rows.partial.data_ptr(), rows.P, rows.eps, M, N, K,
+                      int(swiglu), self._stream())
+        return True
+
+    def scale_rows(self, weighted: torch.Tensor, partial: torch.Tensor, P: int, eps: float, out: torch.Tensor) -> None:
+        """out[m] = weighted[m] / sqrt(sum_p partial[m][p] / width + eps): the norm of rows that a product
+        left half normalised, for whatever cannot divide its own output rows."""
+        M, width = weighted.shape
+        self._act(weighted, "weighted rows"); self._act(out, "normed rows")
+        if out.shape != (M, width) or out.stride(1) != 1 or weighted.stride(1) != 1 or partial.numel() < M * P:
+            raise KernelLibraryError("scale_rows: shapes do not fit")
+        self._note("mv_scale_rows", self._size(weighted, out) + M * P * 4, 2 * M * width)
+        self.lib.call("mv_scale_rows", weighted.data_ptr(), weighted.stride(0) if M > 1 else width, partial.data_ptr(), P,
+                      float(eps), out.data_ptr(), out.stride(0) if M > 1 else width, self.code, M, width, self._stream())
+
     def can_fuse_norm(self, rows: int, width: int) -> bool:
         """Whether a norm over ``rows`` x ``width`` may be deferred into the next product."""
         return (self.use_fast_kernels and self.lib.has("mv_gemm_skinny_norm") and 0 < rows <= FUSED_NORM_MAX_M
@@ -543,7 +659,10 @@ class Ops:
         otherwise; the caller then runs the product and the activation separately. ``a`` may be a
         pending norm, as in ``gemm``."""
         if not isinstance(a, torch.Tensor):
-            if self._gemm_fused_norm(a, w_gate_up, out, None, swiglu=True):
+            if isinstance(a, WeightedRows):
+                if self._gemm_scaled(a, w_gate_up, out, None, swiglu=True):
+                    return True
+            elif self._gemm_fused_norm(a, w_gate_up, out, None, swiglu=True):
                 return True
             a = a.materialize()
         if not (self.use_fast_kernels and self.lib.has("mv_gemm_skinny_swiglu")):

@@ -161,7 +161,15 @@ class CausalLM:
         self.embedding.forward(ctx, resid)
         stream = HiddenStream(resid, rt.workspace.get("resid.spare", (n, plan.hidden_size), torch.float32))
         for call_index, call in enumerate(plan.calls):
-            self.blocks[call.layer].forward(stream, ctx, call_index)
+            block = self.blocks[call.layer]
+            after = None
+            if getattr(block, "accepts_next_norm", False) and call_index + 1 < len(plan.calls):
+                # the norm the next block starts with may be folded into this block's last product
+                after = self.blocks[plan.calls[call_index + 1].layer]
+            if after is not None and hasattr(after, "entry_norm") and hasattr(after, "entry_part"):
+                block.forward(stream, ctx, call_index, next_norm=after.entry_norm(), next_part=after.entry_part())
+            else:
+                block.forward(stream, ctx, call_index)
         m = ctx.n_logit_rows
         if m == 0:
             discard = getattr(stream.delta, "discard", None)

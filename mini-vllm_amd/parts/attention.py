@@ -48,6 +48,7 @@ class AttentionSpec(PartSpec):
 class Attention(Mixer):
     spec_class = AttentionSpec
     accepts_pending_norm = True      # the input is used by one packed product only
+    accepts_fold = True              # the output comes from one product
 
     @classmethod
     def tensors(cls, spec: AttentionSpec) -> Dict[str, TensorDecl]:
@@ -100,7 +101,10 @@ class Attention(Mixer):
             raise ValueError("a position encoding must offer rotary() or apply()")
         self.width = spec.q_dim + (0 if spec.shares_kv else 2 * spec.kv_dim)
 
-    def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
+    def first_product(self):
+        return self.w_qkv.shape[0], self.w_qkv.shape[1], False
+
+    def forward(self, x: torch.Tensor, ctx, call: int, fold=None) -> torch.Tensor:
         spec, rt, ops = self.spec, self.rt, self.rt.ops
         n = x.shape[0]
         ws = rt.workspace
@@ -125,7 +129,7 @@ class Attention(Mixer):
                                           spec.head_dim, spec.scale, spec.window, plan, self.q_norm, self.k_norm,
                                           spec.qk_norm_eps, table, interleaved, not spec.shares_kv):
                 y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
-                return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True) or y
+                return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True, fold=fold) or y
         ops.qk_norm_rope_store(
             qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, ctx.positions, ctx.token_seq,
             self.q_norm, self.k_norm, spec.qk_norm_eps, table, interleaved,
@@ -136,4 +140,4 @@ class Attention(Mixer):
                       spec.num_kv_heads, spec.head_dim, spec.scale, spec.window, plan=ctx.attention_plan)
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         # (the sums of a product whose K was split may be left to the next norm)
-        return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True) or y
+        return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True, fold=fold) or y

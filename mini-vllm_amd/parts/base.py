@@ -256,11 +256,14 @@ class HiddenStream:
     defer_sum=True)`` returned in its place (an output whose partial sums the norm's kernel adds
     up itself; it has ``shape``, ``materialize()`` and ``discard()``)."""
 
-    __slots__ = ("resid", "delta", "spare")
+    __slots__ = ("resid", "delta", "spare", "weighted")
 
     def __init__(self, resid: torch.Tensor, spare: Optional[torch.Tensor] = None):
         self.resid = resid
         self.delta: Optional[torch.Tensor] = None
+        # rows that the last product already added to ``resid`` and left half normalised for the
+        # norm that comes next (see NormFold); that norm takes them from here
+        self.weighted = None
         # a second buffer of the same shape: a kernel that adds the delta while other workgroups
         # still read the old sum writes the new sum here, and the two change places
         self.spare = spare
@@ -303,6 +306,32 @@ class PendingNorm:
             st.resid, st.spare = resid_out, resid_in
             st.delta = None
         return resid_in, delta, resid_out
+
+
+class NormFold:
+    """A residual add and the norm behind it, offered to the product in front of them. With too many
+    rows to normalise them inside every workgroup of the next product (``PendingNorm``), the add and
+    the norm can still go without a kernel of their own: the product that makes the delta owns each
+    element once, so it adds it to ``stream.resid`` there, writes the sum times the norm's weight to
+    ``weighted`` and the sums of squares of its column slices to ``partial``; the product behind the
+    norm divides its output rows by the root mean square it gets from those sums.
+
+    It is offered only when the part behind the norm says what its first product is
+    (``first_product() -> (weight rows, weight columns, gated)``, beside ``accepts_pending_norm``)
+    and the kernels take that product from such rows.
+
+    A part that declares ``accepts_fold = True`` gets one as ``fold=`` (or None), hands it to
+    ``ops.gemm(..., fold=fold)`` with its last product and returns whatever that returns: the delta
+    as before when the shape was not taken, else the half-normalised rows (``ops.WeightedRows``),
+    which the block leaves in ``stream.weighted`` for the norm."""
+
+    __slots__ = ("norm", "stream", "weight", "eps", "unit_offset", "weighted", "partial", "normed")
+
+    def __init__(self, norm, stream: HiddenStream, weight: torch.Tensor, eps: float, unit_offset: bool,
+                 weighted: torch.Tensor, partial: torch.Tensor, normed: torch.Tensor):
+        self.norm, self.stream = norm, stream
+        self.weight, self.eps, self.unit_offset = weight, eps, unit_offset
+        self.weighted, self.partial, self.normed = weighted, partial, normed
 
 
 # ---------------------------------------------------------------------------------------
@@ -398,10 +427,24 @@ class Head(Part):
 
 
 class Block:
-    """Wires the parts of one layer: forward(stream, ctx, call) updates the stream."""
+    """Wires the parts of one layer: forward(stream, ctx, call) updates the stream.
+
+    A block that declares ``accepts_next_norm = True`` is also given ``next_norm=`` and ``next_part=``:
+    the norm that the block called next applies first to the stream and the part that takes its
+    output (``entry_norm()``, ``entry_part()``), or None. It may offer that norm to its last part
+    (``NormFold``)."""
+    accepts_next_norm: ClassVar[bool] = False
 
     def __init__(self, spec, norms: Dict[str, Norm], mixer: Mixer, ffn: FeedForward):
         raise NotImplementedError
+
+    def entry_norm(self) -> Optional["Norm"]:
+        """The norm this block applies to the stream before anything else, if it starts with one."""
+        return None
+
+    def entry_part(self):
+        """The part that takes the output of ``entry_norm()``."""
+        return None
 
     def forward(self, stream: HiddenStream, ctx, call: int) -> None:
         raise NotImplementedError

@@ -6,7 +6,7 @@ norm before the feed-forward, residual add; nothing after either.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Tuple
+from typing import Dict, Optional, Tuple
 
 from .base import Block, FeedForward, HiddenStream, Mixer, Norm, PartSpec, register_block
 
@@ -28,12 +28,35 @@ class PreNormBlock(Block):
         self.mixer = mixer
         self.ffn = ffn
 
-    def forward(self, stream: HiddenStream, ctx, call: int) -> None:
+    accepts_next_norm = True
+
+    def entry_norm(self) -> Norm:
+        return self.norm_mixer
+
+    def entry_part(self):
+        return self.mixer
+
+    def forward(self, stream: HiddenStream, ctx, call: int, next_norm: Optional[Norm] = None, next_part=None) -> None:
         # a part that starts with one matrix product over its input may get the norm unrun, to
-        # fuse it into that product
-        defer = getattr(self.mixer, "accepts_pending_norm", False)
-        h = self.norm_mixer.pending(stream, ctx) if defer else self.norm_mixer.forward(stream, ctx)
-        stream.delta = self.mixer.forward(h, ctx, call)
-        defer = getattr(self.ffn, "accepts_pending_norm", False)
-        h = self.norm_ffn.pending(stream, ctx) if defer else self.norm_ffn.forward(stream, ctx)
-        stream.delta = self.ffn.forward(h, ctx)
+        # fuse it into that product; a part that ends with one may be offered the add and the norm
+        # that follow it, to fold them into that product, when the part behind that norm can go on
+        # from rows that are not yet divided by their root mean square
+        self._run(stream, ctx, self.norm_mixer, self.mixer, self.norm_ffn, self.ffn, (call,))
+        self._run(stream, ctx, self.norm_ffn, self.ffn, next_norm, next_part, ())
+
+    @staticmethod
+    def _run(stream: HiddenStream, ctx, norm: Norm, part, norm_after: Optional[Norm], part_after, extra: tuple) -> None:
+        defer = getattr(part, "accepts_pending_norm", False)
+        h = norm.pending(stream, ctx) if defer else norm.forward(stream, ctx)
+        fold = None
+        if norm_after is not None and getattr(part, "accepts_fold", False) \
+                and getattr(part_after, "accepts_pending_norm", False):
+            make = getattr(norm_after, "fold", None)
+            first = getattr(part_after, "first_product", None)
+            if make is not None and first is not None:
+                fold = make(stream, ctx, first())
+        out = part.forward(h, ctx, *extra, fold=fold) if fold is not None else part.forward(h, ctx, *extra)
+        if getattr(out, "is_weighted_rows", False):
+            stream.delta, stream.weighted = None, out      # already added to the residual
+        else:
+            stream.delta = out

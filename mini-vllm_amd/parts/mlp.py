@@ -25,6 +25,7 @@ class SwiGLUSpec(PartSpec):
 class SwiGLU(FeedForward):
     spec_class = SwiGLUSpec
     accepts_pending_norm = True      # the input is used by one packed product only
+    accepts_fold = True              # the output comes from one product
 
     @classmethod
     def tensors(cls, spec: SwiGLUSpec) -> Dict[str, TensorDecl]:
@@ -40,7 +41,10 @@ class SwiGLU(FeedForward):
         self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous()
         self.w_down = tensors["down"]
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    def first_product(self):
+        return self.w_gate_up.shape[0], self.w_gate_up.shape[1], True
+
+    def forward(self, x: torch.Tensor, ctx, fold=None) -> torch.Tensor:
         spec, rt, ops = self.spec, self.rt, self.rt.ops
         n = x.shape[0]
         act = rt.workspace.get("ffn.act", (n, spec.intermediate_size), rt.dtype)
@@ -51,5 +55,6 @@ class SwiGLU(FeedForward):
             ops.gemm(x, self.w_gate_up, gu)
             ops.swiglu(gu, act)
         y = rt.workspace.get("ffn.out", (n, spec.hidden_size), rt.dtype)
-        # (the sums of a product whose K was split may be left to the next norm)
-        return ops.gemm(act, self.w_down, y, defer_sum=True) or y
+        # (the sums of a product whose K was split may be left to the next norm, or the residual add and
+        # that norm folded into the product)
+        return ops.gemm(act, self.w_down, y, defer_sum=True, fold=fold) or y

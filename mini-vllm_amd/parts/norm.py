@@ -13,7 +13,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import HiddenStream, Norm, PartSpec, PendingNorm, Runtime, TensorDecl, register_norm
+from .base import HiddenStream, Norm, NormFold, PartSpec, PendingNorm, Runtime, TensorDecl, register_norm
 
 
 @dataclass(frozen=True)
@@ -39,6 +39,11 @@ class RMSNorm(Norm):
 
     def forward(self, stream: HiddenStream, ctx, rows: Optional[torch.Tensor] = None,
                 tag: str = "normed") -> torch.Tensor:
+        taken = self._take_weighted(stream)
+        if taken is not None:
+            if rows is not None:
+                raise RuntimeError("rows left half normalised for a norm that wants only some of them")
+            return taken.materialize()
         n = stream.resid.shape[0] if rows is None else rows.numel()
         out = self.rt.workspace.get(tag, (n, self.spec.size), self.rt.dtype)
         self.rt.ops.add_rmsnorm(stream.resid, stream.delta, self.weight, self.spec.eps, out, rows=rows,
@@ -47,8 +52,36 @@ class RMSNorm(Norm):
             stream.delta = None
         return out
 
+    def _take_weighted(self, stream: HiddenStream):
+        """The rows the product in front left half normalised for this norm (``fold``), if any."""
+        taken = stream.weighted
+        if taken is None:
+            return None
+        stream.weighted = None
+        if taken.norm is not self or stream.delta is not None:
+            raise RuntimeError("the stream holds rows that were prepared for another norm")
+        return taken
+
+    def fold(self, stream: HiddenStream, ctx, consumer=None) -> Optional[NormFold]:
+        """The residual add and this norm, offered to the product in front of them, for steps of more
+        rows than the fused add + norm + product kernel takes. ``consumer``: the product that comes
+        behind the norm, (weight rows, weight columns, gated); without it, or when the kernels would
+        not take that product from half-normalised rows, nothing is offered."""
+        n, size = stream.resid.shape[0], self.spec.size
+        if consumer is None or consumer[1] != size or not self.rt.ops.can_fold_norm(n, size, consumer):
+            return None
+        ws = self.rt.workspace
+        return NormFold(self, stream, self.weight, self.spec.eps, self.spec.unit_offset,
+                        ws.get("fold.weighted", (n, size), self.rt.dtype),
+                        ws.get("fold.partial", (n * ((size + 3) // 4),), torch.float32),
+                        ws.get("normed", (n, size), self.rt.dtype))
+
     def pending(self, stream: HiddenStream, ctx):
-        """Deferred when the step is small enough for the fused add + norm + product kernel."""
+        """Deferred when the step is small enough for the fused add + norm + product kernel; rows that
+        the product in front left half normalised go on as they are."""
+        taken = self._take_weighted(stream)
+        if taken is not None:
+            return taken
         if stream.spare is not None and self.rt.ops.can_fuse_norm(stream.resid.shape[0], self.spec.size):
             return PendingNorm(self, stream, ctx)
         return self.forward(stream, ctx)

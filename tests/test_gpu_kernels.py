@@ -1058,6 +1058,67 @@ def test_gemm_with_fused_add_and_norm(M, N, K, swiglu, with_delta):
         assert stream.resid is first
 
 
+@pytest.mark.parametrize("M,N,K,N2,swiglu", [(64, 1024, 2048, 4096, False), (17, 1024, 3072, 3072, True),
+                                             (40, 224, 96, 333, False), (33, 96, 64, 56, True),
+                                             (8, 4096, 4096, 6144, False), (20, 992, 1024, 100, False)])
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("consumer", ["product", "rows"])
+def test_residual_add_and_norm_folded_into_the_products_around_them(M, N, K, N2, swiglu, with_bias, consumer):
+    """A step of more rows than the fused add + norm + product kernel takes: the product in front of
+    the norm adds its output to the residual and leaves the rows weighted with partial sums of
+    squares (``gemm(..., fold=...)``), the product behind it divides its output rows by the root mean
+    square (``gemm(WeightedRows, ...)``) — or, for a consumer that cannot, the rows are normalised by
+    a kernel of their own. Against the stand-alone add and norm between two plain products."""
+    from minivllm_amd.kernels.ops import WeightedRows
+    from minivllm_amd.parts import NORMS, HiddenStream, RMSNormSpec, Runtime, Workspace
+    ops = ops_for(torch.bfloat16)
+    rt = Runtime(device=torch.device("cuda:0"), dtype=torch.bfloat16, ops=ops,
+                 workspace=Workspace(torch.device("cuda:0")), max_positions=16)
+    g = torch.Generator().manual_seed(45)
+    eps = 1e-5
+    spec = RMSNormSpec(size=N, eps=eps)
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).to(torch.bfloat16)
+    norm = NORMS.get(spec.kind)(spec, {"weight": dev(nw)}, rt)
+    resid = 3.0 * torch.randn(M, N, generator=g)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b1 = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
+    w2 = (torch.randn((2 * N2 if swiglu else N2), N, generator=g) / math.sqrt(N)).to(torch.bfloat16)
+    b2 = torch.randn(N2, generator=g).to(torch.bfloat16) if (with_bias and not swiglu) else None
+    assert not ops.can_fuse_norm(M, N) and ops.can_fold_norm(M, N)
+    stream = HiddenStream(dev(resid).clone(), torch.full((M, N), float("nan"), device="cuda"))
+    assert norm.fold(stream, None) is None                      # nobody said what comes behind the norm
+    assert norm.fold(stream, None, (200 * 1000, N, False)) is None or N * 200 * 1000 < 96 * 1000 * 1000   # the library's
+    fold = norm.fold(stream, None, (w2.shape[0], N, swiglu))
+    assert fold is not None
+    y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rows = ops.gemm(dev(a), dev(w1), y, dev(b1) if b1 is not None else None, defer_sum=True, fold=fold)
+    assert isinstance(rows, WeightedRows) and torch.isnan(y.float()).all()      # the delta was never written
+    stream.weighted = rows
+    # the reference: plain product, rounded; add; norm; plain product
+    delta = (a.double() @ w1.double().T + (b1.double() if b1 is not None else 0)).to(torch.bfloat16).double()
+    x = resid.double() + delta
+    assert rel_err(stream.resid.cpu().numpy(), x.float().numpy()) <= 2e-3       # a delta may round the other way
+    normed = (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * nw.double())
+    out = torch.full((M, N2), float("nan"), dtype=torch.bfloat16, device="cuda")
+    if consumer == "rows":
+        h = norm.forward(stream, None)              # whoever wants a tensor gets the normalised rows
+        assert rel_err(h.float().cpu().numpy(), normed.numpy()) <= OP_TOL[torch.bfloat16]
+        assert stream.weighted is None
+        return
+    h = norm.pending(stream, None)
+    assert h is rows and stream.weighted is None
+    if swiglu:
+        assert ops.gemm_swiglu(h, dev(w2), out)
+        gu = normed.to(torch.bfloat16).double() @ w2.double().T
+        want = torch.nn.functional.silu(gu[:, :N2]) * gu[:, N2:]
+    else:
+        ops.gemm(h, dev(w2), out, dev(b2) if b2 is not None else None)
+        want = normed.to(torch.bfloat16).double() @ w2.double().T + (b2.double() if b2 is not None else 0)
+    assert rows.used
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[torch.bfloat16]
+
+
 def test_norm_is_not_deferred_for_many_rows():
     from minivllm_amd.parts import NORMS, HiddenStream, RMSNormSpec, Runtime, Workspace
     ops = ops_for(torch.bfloat16)

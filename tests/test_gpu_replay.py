@@ -159,6 +159,41 @@ def test_first_tokens_and_single_token_requests(cases):
             assert rel_err(row, case.want[src][pos]) <= case.tol(dtype)
 
 
+def test_which_kernels_take_the_norms(cases):
+    """The residual add and the norm between two products go three ways, by the number of rows of the
+    step (bfloat16, sizes the MFMA products take): up to 16 rows they run inside the product behind
+    them; from 17 to 64 the product in front adds and weights, the product behind divides; above
+    that they are a kernel of their own. Seen in what the kernel front end launches; the logits of
+    every one of these steps agree with the plain model."""
+    case = cases[("D128", "mild")]
+    toks = case.reqs["r2"]
+    assert len(toks) >= 130
+    cuts = [0, 8, 48, 130]                         # portions of 8, 40 and 82 tokens
+    steps = [{"step": i, "entries": [{"id": "x", "tokens": toks[a:b], "want": list(range(b - a))}], "end": []}
+             for i, (a, b) in enumerate(zip(cuts, cuts[1:]))]
+    runner = runner_for(case, "bfloat16", steps)
+    ops = runner.executor.ops
+    seen = []
+
+    def run_step(st):
+        ops.ledger = []
+        try:
+            return runner.run_step(st)
+        finally:
+            seen.append([line[0] for line in ops.ledger])
+            ops.ledger = None
+
+    got = trace_tools.collect(steps, run_step)
+    layers = case.cfg["num_hidden_layers"]
+    assert seen[0].count("mv_gemm_skinny_norm") == 2 * layers and "mv_gemm_skinny_fold" not in seen[0]
+    assert seen[1].count("mv_gemm_skinny_fold") == 2 * layers - 1          # the last product has the final norm behind it
+    assert seen[1].count("mv_gemm_skinny_scaled") == 2 * layers - 1 and seen[1].count("mv_add_rmsnorm") == 2
+    assert "mv_gemm_skinny_fold" not in seen[2] and seen[2].count("mv_add_rmsnorm") == 2 * layers + 1
+    assert len(got) == 130
+    for (rid, pos), row in got.items():
+        assert rel_err(row, case.want["r2"][pos]) <= case.tol("bfloat16")
+
+
 def test_long_decoding(cases):
     """One token after another from the very first, 300 of them, across many pages."""
     case = cases[("B", "sharp")]
