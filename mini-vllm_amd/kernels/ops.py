@@ -548,14 +548,15 @@ class Ops:
 
     def can_fold_norm(self, rows: int, width: int, consumer=None) -> bool:
         """Whether a residual add and a norm over ``rows`` x ``width`` may be offered to the product in
-        front of them (``gemm(..., fold=...)``): steps of up to SKINNY_MAX_M rows that are too large
-        for the fused add + norm + product kernel, when the product behind the norm (``consumer`` =
-        (weight rows, weight columns, gated)) is one the weight-streaming kernel takes — behind any
-        other the rows would have to be normalised by a kernel of their own, and nothing is gained
-        (32B sizes, where gate/up goes to the library: 2 % slower)."""
+        front of them (``gemm(..., fold=...)``): steps of up to SKINNY_MAX_M rows, when the product
+        behind the norm (``consumer`` = (weight rows, weight columns, gated)) is one the
+        weight-streaming kernel takes — behind any other the rows would have to be normalised by a
+        kernel of their own, and nothing is gained (32B sizes, where gate/up goes to the library: 2 %
+        slower). Where both this and the fused add + norm + product kernel could serve (up to 16
+        rows), this is taken: the product behind reads finished bf16 rows instead of normalising
+        them in every workgroup (0.6B sizes: a step of 1, 8, 16 sequences 5, 3, 4 % faster)."""
         if not (self.use_fast_kernels and self.dtype == torch.bfloat16 and self.lib.has("mv_gemm_skinny_fold")
-                and self.lib.has("mv_gemm_skinny_scaled") and 0 < rows <= SKINNY_MAX_M and width % 4 == 0
-                and not self.can_fuse_norm(rows, width)):
+                and self.lib.has("mv_gemm_skinny_scaled") and 0 < rows <= SKINNY_MAX_M and width % 4 == 0):
             return False
         if consumer is None:
             return True

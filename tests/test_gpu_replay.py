@@ -160,10 +160,10 @@ def test_first_tokens_and_single_token_requests(cases):
 
 
 def test_which_kernels_take_the_norms(cases):
-    """The residual add and the norm between two products go three ways, by the number of rows of the
-    step (bfloat16, sizes the MFMA products take): up to 16 rows they run inside the product behind
-    them; from 17 to 64 the product in front adds and weights, the product behind divides; above
-    that they are a kernel of their own. Seen in what the kernel front end launches; the logits of
+    """The residual add and the norm between two products, by the number of rows of the step (bfloat16,
+    sizes the MFMA products take): up to 64 rows the product in front adds and weights and the
+    product behind divides (the first norm of a step of up to 16 rows, which has no product in
+    front, runs inside the product behind it); above that they are a kernel of their own. Seen in what the kernel front end launches; the logits of
     every one of these steps agree with the plain model."""
     case = cases[("D128", "mild")]
     toks = case.reqs["r2"]
@@ -185,8 +185,10 @@ def test_which_kernels_take_the_norms(cases):
 
     got = trace_tools.collect(steps, run_step)
     layers = case.cfg["num_hidden_layers"]
-    assert seen[0].count("mv_gemm_skinny_norm") == 2 * layers and "mv_gemm_skinny_fold" not in seen[0]
-    assert seen[1].count("mv_gemm_skinny_fold") == 2 * layers - 1          # the last product has the final norm behind it
+    # (the first norm has the embedding in front of it, the last product the final norm behind it)
+    assert seen[0].count("mv_gemm_skinny_norm") == 1 and seen[0].count("mv_gemm_skinny_fold") == 2 * layers - 1
+    assert seen[0].count("mv_gemm_skinny_scaled") == 2 * layers - 1 and seen[0].count("mv_add_rmsnorm") == 1
+    assert seen[1].count("mv_gemm_skinny_fold") == 2 * layers - 1
     assert seen[1].count("mv_gemm_skinny_scaled") == 2 * layers - 1 and seen[1].count("mv_add_rmsnorm") == 2
     assert "mv_gemm_skinny_fold" not in seen[2] and seen[2].count("mv_add_rmsnorm") == 2 * layers + 1
     assert len(got) == 130
