@@ -555,17 +555,18 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     __syncthreads();
     if (!sh_last) return;
 #define AF_PEEK(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-    // each thread adds up one element of one column; the rows of up to eight splits, with their
+    // each thread adds up one element of one column; the rows of up to sixteen splits, with their
     // maxima and sums, are in flight at once (one round trip for the usual split counts)
+    constexpr int MB = 16;
     for (int idx = threadIdx.x; idx < ncols * D; idx += blockDim.x) {
         const int col = idx / D, d = idx - col * D;
         const int tok = t0 + col / G, head = kvh * G + col % G;
         const float* base = partials + ((size_t)tok * H + head) * nsplit * (D + 2);
         float m = -INFINITY, l = 0.f, a = 0.f;
-        for (int j0 = 0; j0 < n_active; j0 += 8) {
-            float v[8], mz[8], lz[8];
+        for (int j0 = 0; j0 < n_active; j0 += MB) {
+            float v[MB], mz[MB], lz[MB];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < MB; ++u) {
                 int z = z_first + j0 + u;
                 if (z >= nsplit) z -= nsplit;
                 const float* row = base + (size_t)z * (D + 2);
@@ -576,14 +577,14 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
             }
             float mb = m;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) mb = fmaxf(mb, mz[u]);
+            for (int u = 0; u < MB; ++u) mb = fmaxf(mb, mz[u]);
             const float m_safe = (mb == -INFINITY) ? 0.f : mb;
             const float corr = exp2f(m - m_safe);     // exp2(-inf) = 0
             l *= corr;
             a *= corr;
             m = mb;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < MB; ++u) {
                 const float w = exp2f(mz[u] - m_safe);
                 l += w * lz[u];
                 a += w * v[u];
