@@ -10,8 +10,9 @@
 //   out^T    = V^T P^T   A operand: 16 d x 32 keys of the transposed value page,
 //                        B operand: 32 keys x 16 columns of the probabilities.
 // The probabilities a lane needs for the second product are exactly the scores it holds after
-// the first: its eight k-slots are bound to the keys {4g..4g+3} of two neighbouring 16-key
-// tiles (g = l/16), and the value operand is loaded for the same keys, so nothing is shuffled.
+// the first: the rows of the two score tiles of a 32-key block interleave in groups of four keys
+// (row 4g+r of tile t is key 8g+4t+r, g = l/16), so lane group g ends up with the keys 8g..8g+7,
+// eight neighbours of a value row: one 16-byte load per value operand, and nothing is shuffled.
 // Each column keeps its own running maximum and sum (online softmax, base 2).
 //
 // The W waves of a workgroup (4 or 8) take the 32-key blocks in turn, each with the K operands
@@ -310,37 +311,52 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         const int rel = pidx - p_first;
         return rel < n_cached ? sh_pages[rel] : bt[pidx];
     };
+    // Which keys a lane's operand slots hold: row rho of score tile t is key 8 (rho / 4) + 4 t + rho % 4 of
+    // the block, so that after the first product lane group g holds the probabilities of keys 8 g ..
+    // 8 g + 7 (slot 4 t + r is key 8 g + 4 t + r) — eight neighbours in a value row, one 16-byte load
+    // per operand, and still nothing is shuffled between the products. The block's two halves of 16
+    // keys may lie in different pages: a key row of either tile lies in half rho / 8, a lane group's
+    // values in half g / 2.
     struct Operands {
-        int page[2];
+        int page[2];   // of the block's halves
         Frag k[2][DS];
         Frag v[DT];
     };
+    const int k_half = i / 8, v_half = g / 2;
     auto fetch = [&](int b, Operands& op) {
         int slot0[2];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int key0 = 32 * b + 16 * t;
+        for (int h = 0; h < 2; ++h) {
+            const int key0 = 32 * b + 16 * h;
             const int pidx = key0 / page_size;
-            op.page[t] = (b < b_end && key0 <= hi_w) ? page_of(pidx) : -1;
-            slot0[t] = key0 - pidx * page_size;
+            op.page[h] = (b < b_end && key0 <= hi_w) ? page_of(pidx) : -1;
+            slot0[h] = key0 - pidx * page_size;
         }
+        const int kpage = k_half ? op.page[1] : op.page[0];
+        const int vpage = v_half ? op.page[1] : op.page[0];
+        if (kpage >= 0) {
+            const size_t head = (size_t)kpage * Hkv + kvh;
+            const int slot = (k_half ? slot0[1] : slot0[0]) + 8 * ((i / 4) % 2) + i % 4;   // of tile 0; tile 1 four on
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            if (op.page[t] >= 0) {
-                const size_t head = (size_t)op.page[t] * Hkv + kvh;
-                const bf16* kptr = k_pages + ((head * page_size + slot0[t] + i) * D + 8 * g);
+            for (int t = 0; t < 2; ++t) {
+                const bf16* kptr = k_pages + ((head * page_size + slot + 4 * t) * D + 8 * g);
 #pragma unroll
                 for (int s = 0; s < DS; ++s) op.k[t][s].u = *reinterpret_cast<const uint4*>(kptr + 32 * s);
-                const bf16* vptr = v_pages + (head * D + i) * page_size + slot0[t] + 4 * g;
+            }
+        } else {
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-                    op.v[dt].h[t] = *reinterpret_cast<const uint2*>(vptr + (size_t)16 * dt * page_size);
-            } else {
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int s = 0; s < DS; ++s) op.k[t][s].u = uint4{0u, 0u, 0u, 0u};
+        }
+        if (vpage >= 0) {
+            const size_t head = (size_t)vpage * Hkv + kvh;
+            const bf16* vptr = v_pages + (head * D + i) * page_size + (v_half ? slot0[1] : slot0[0]) + 8 * (g % 2);
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) op.v[dt].h[t] = uint2{0u, 0u};
-            }
+            for (int dt = 0; dt < DT; ++dt) op.v[dt].u = *reinterpret_cast<const uint4*>(vptr + (size_t)16 * dt * page_size);
+        } else {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) op.v[dt].u = uint4{0u, 0u, 0u, 0u};
         }
     };
     auto compute = [&](int b, Operands& op) {
@@ -348,32 +364,33 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         if (FUSED && owns_new && b == b_new) {   // the newest key and value come from the registers
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                if (base + 16 * t + i == hi_w) {
+                if (base + 8 * (i / 4) + 4 * t + i % 4 == hi_w) {
 #pragma unroll
                     for (int s = 0; s < DS; ++s) op.k[t][s] = knew[s];
                 }
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (base + 16 * t + 4 * g + r == hi_w) {
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) op.v[dt].s[t * 4 + r] = vnew[dt];
-                    }
             }
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (base + 8 * g + e == hi_w) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) op.v[dt].s[e] = vnew[dt];
+                }
         }
+        const bool v_live = (v_half ? op.page[1] : op.page[0]) >= 0;     // the half of this lane's probabilities
         // scores^T for two tiles of 16 keys
         float p[2][4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             floatx4_t sacc = floatx4_t{0.f, 0.f, 0.f, 0.f};
-            if (op.page[t] >= 0) {
+            if (op.page[0] >= 0 || op.page[1] >= 0) {
 #pragma unroll
                 for (int s = 0; s < DS; ++s)
                     sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.k[t][s].v, qop[0][s].v, sacc, 0, 0, 0);
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int key = base + 16 * t + 4 * g + r;
-                const bool ok = op.page[t] >= 0 && col_ok[0] && key <= col_pos[0] && key >= col_lo[0];
+                const int key = base + 8 * g + 4 * t + r;
+                const bool ok = v_live && col_ok[0] && key <= col_pos[0] && key >= col_lo[0];
                 p[t][r] = ok ? sacc[r] * sc_mul : -INFINITY;
             }
         }
@@ -407,10 +424,8 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (base + 16 * t + 4 * g + r > hi_w) op.v[dt].s[t * 4 + r] = 0;
+                for (int e = 0; e < 8; ++e)
+                    if (base + 8 * g + e > hi_w) op.v[dt].s[e] = 0;
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
