@@ -17,6 +17,12 @@ _NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
 
 # largest number of rows the weight-streaming product takes in one launch
 SKINNY_MAX_M = 64
+# ... and up to this many rows against small weights (the layers of a 0.6B-sized model): between 65 and
+# 96 rows the engine's products, with the norms and the activation folded into them, still beat the
+# library's with kernels of their own between them (a step of 72 / 80 / 96 sequences 3.2 / 4.4 / 2.3 %
+# faster; at 112 and 128 rows nothing is gained)
+SKINNY_WIDE_MAX_M = 96
+SKINNY_WIDE_MAX_WEIGHT = 8 * 1024 * 1024
 # most rows of one launch of it
 SKINNY_LAUNCH_ROWS = 512
 # the kernel that shares activation rows through LDS and splits K over workgroups takes over from
@@ -422,7 +428,7 @@ class Ops:
                                   defer_sum=defer_sum and out.dtype == self.dtype and out.is_contiguous())
             if done:
                 return done if isinstance(done, SplitSum) else None
-            if M > SKINNY_MAX_M and self._library_serves(out) and \
+            if not self.streams_rows(M, N, K) and self._library_serves(out) and \
                     self._library_allowed(M, N, K, bias is not None, out.dtype) and self._library_product(a, w, bias, out):
                 return
             if fold is not None and self._fold_serves(fold, out, M, N):
@@ -449,6 +455,12 @@ class Ops:
         self._note("mv_gemm_ref", self._size(a, w, out), 2 * M * N * K)
         self.lib.call("mv_gemm_ref", a.data_ptr(), lda, self.code, w.data_ptr(), K, wcode, _ptr(bias),
                       out.data_ptr(), ldc, _CODES[out.dtype], M, N, K, self._stream())
+
+    @staticmethod
+    def streams_rows(M: int, N: int, K: int) -> bool:
+        """Whether the weight-streaming product is the engine's choice for M rows against an [N, K]
+        weight (before the library and the K-splitting kernel have had their say)."""
+        return M <= SKINNY_MAX_M or (M <= SKINNY_WIDE_MAX_M and N * K <= SKINNY_WIDE_MAX_WEIGHT)
 
     def prefers_library(self, M: int, N: int, K: int, gated: bool = False) -> bool:
         """Whether a product of few rows against this weight is left to the library (see
@@ -541,7 +553,8 @@ class Ops:
 
     @staticmethod
     def wants_mid(M: int, N: int, K: int) -> bool:
-        """Whether a product of M rows with an [N, K] weight goes to the kernel that splits K."""
+        """Whether a product of M rows with an [N, K] weight goes to the kernel that splits K (it takes
+        up to 64 rows)."""
         if M > SKINNY_MAX_M or K % 128:
             return False
         return (N * K >= MID_ALWAYS_WEIGHT and K >= MID_ALWAYS_K) or (N * K >= MID_MIN_WEIGHT and M >= MID_MIN_M)
@@ -556,18 +569,18 @@ class Ops:
         rows), this is taken: the product behind reads finished bf16 rows instead of normalising
         them in every workgroup (0.6B sizes: a step of 1, 8, 16 sequences 5, 3, 4 % faster)."""
         if not (self.use_fast_kernels and self.dtype == torch.bfloat16 and self.lib.has("mv_gemm_skinny_fold")
-                and self.lib.has("mv_gemm_skinny_scaled") and 0 < rows <= SKINNY_MAX_M and width % 4 == 0):
+                and self.lib.has("mv_gemm_skinny_scaled") and 0 < rows <= SKINNY_WIDE_MAX_M and width % 4 == 0):
             return False
         if consumer is None:
-            return True
+            return rows <= SKINNY_MAX_M
         n, k, gated = consumer
-        return (k == width and k % 32 == 0 and not (gated and n % 2)
+        return (k == width and self.streams_rows(rows, n, k) and k % 32 == 0 and not (gated and n % 2)
                 and not (self.wants_mid(rows, n, k) and self.lib.has("mv_gemm_mid"))
                 and not self.prefers_library(rows, n, k, gated=gated))
 
     def _fold_serves(self, fold, out: torch.Tensor, M: int, N: int) -> bool:
         resid = fold.stream.resid
-        return (M <= SKINNY_MAX_M and out.dtype == self.dtype and self.lib.has("mv_gemm_skinny_fold")
+        return (M <= SKINNY_WIDE_MAX_M and out.dtype == self.dtype and self.lib.has("mv_gemm_skinny_fold")
                 and resid.dtype == torch.float32 and resid.shape == (M, N) and resid.stride(1) == 1
                 and fold.weight.numel() == N and fold.weight.is_contiguous()
                 and fold.weighted.shape == (M, N) and fold.weighted.stride(1) == 1 and fold.weighted.dtype == self.dtype
@@ -582,7 +595,8 @@ class Ops:
         mean square; False if the shape is not taken (nothing has been done then)."""
         a = rows.weighted
         M, K = a.shape
-        if (not self.use_fast_kernels or not self.lib.has("mv_gemm_skinny_scaled") or M == 0 or M > SKINNY_MAX_M
+        if (not self.use_fast_kernels or not self.lib.has("mv_gemm_skinny_scaled") or M == 0
+                or not self.streams_rows(M, w.shape[0], K)
                 or w.dtype != torch.bfloat16 or not w.is_contiguous() or w.shape[1] != K or K % 32
                 or a.stride(1) != 1 or (M > 1 and a.stride(0) % 8) or a.data_ptr() % 16
                 or out.stride(1) != 1 or out.dtype != torch.bfloat16 or (swiglu and w.shape[0] % 2)):
@@ -673,7 +687,8 @@ class Ops:
         if self.prefers_library(M, two_i, K, gated=True) and self._library_allowed(M, two_i, K, False):
             return False
         # with the library's product at hand, more rows than one workgroup takes go there
-        if (M > SKINNY_LAUNCH_ROWS or M == 0 or (M > SKINNY_MAX_M and self._library_allowed(M, two_i, K, False))
+        if (M > SKINNY_LAUNCH_ROWS or M == 0
+                or (not self.streams_rows(M, two_i, K) and self._library_allowed(M, two_i, K, False))
                 or w_gate_up.dtype != torch.bfloat16 or K % 32 or two_i % 2
                 or a.stride(1) != 1 or (M > 1 and a.stride(0) % 8) or a.data_ptr() % 16
                 or not w_gate_up.is_contiguous() or w_gate_up.shape[1] != K):

@@ -788,11 +788,11 @@ def test_gemm_weight_streaming_many_rows(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,with_bias,out_dtype", [
-    (65, 1024, 2048, True, torch.bfloat16), (200, 336, 1024, False, torch.bfloat16),
+    (97, 1024, 2048, True, torch.bfloat16), (65, 4096, 4096, False, torch.bfloat16), (200, 336, 1024, False, torch.bfloat16),
     (2048, 6144, 1024, False, torch.bfloat16), (300, 4096, 12288, True, torch.bfloat16),
     (2048, 51200, 5120, False, torch.bfloat16), (128, 151936, 1024, False, torch.float32),
     (1, 151936, 1024, False, torch.float32), (8, 151936, 1024, False, torch.float32), (40, 151936, 1024, True, torch.float32),
-    (70, 1001, 96, True, torch.float32), (400, 50021, 4096, False, torch.float32)])
+    (100, 1001, 96, True, torch.float32), (400, 50021, 4096, False, torch.float32)])
 def test_gemm_through_the_library(M, N, K, with_bias, out_dtype):
     """More than 64 rows outside graphs, and any number of rows into float32 against a very large
     weight (the logits): the library's product, called directly. The largest bf16 shape is one for
@@ -1060,7 +1060,8 @@ def test_gemm_with_fused_add_and_norm(M, N, K, swiglu, with_delta):
 
 @pytest.mark.parametrize("M,N,K,N2,swiglu", [(64, 1024, 2048, 4096, False), (17, 1024, 3072, 3072, True),
                                              (40, 224, 96, 333, False), (33, 96, 64, 56, True),
-                                             (8, 4096, 4096, 6144, False), (20, 992, 1024, 100, False)])
+                                             (8, 4096, 4096, 6144, False), (20, 992, 1024, 100, False),
+                                             (80, 1024, 2048, 4096, False), (96, 1024, 3072, 3072, True)])
 @pytest.mark.parametrize("with_bias", [False, True])
 @pytest.mark.parametrize("consumer", ["product", "rows"])
 def test_residual_add_and_norm_folded_into_the_products_around_them(M, N, K, N2, swiglu, with_bias, consumer):
@@ -1085,7 +1086,8 @@ def test_residual_add_and_norm_folded_into_the_products_around_them(M, N, K, N2,
     b1 = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
     w2 = (torch.randn((2 * N2 if swiglu else N2), N, generator=g) / math.sqrt(N)).to(torch.bfloat16)
     b2 = torch.randn(N2, generator=g).to(torch.bfloat16) if (with_bias and not swiglu) else None
-    assert not ops.can_fuse_norm(M, N) and ops.can_fold_norm(M, N)
+    assert not ops.can_fuse_norm(M, N) and ops.can_fold_norm(M, N, (w2.shape[0], N, swiglu))
+    assert not ops.can_fold_norm(97, N, (w2.shape[0], N, swiglu)) and not ops.can_fold_norm(80, 4096, (6144, 4096, False))
     stream = HiddenStream(dev(resid).clone(), torch.full((M, N), float("nan"), device="cuda"))
     assert norm.fold(stream, None) is None                      # nobody said what comes behind the norm
     assert norm.fold(stream, None, (200 * 1000, N, False)) is None or N * 200 * 1000 < 96 * 1000 * 1000   # the library's

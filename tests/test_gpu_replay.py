@@ -161,14 +161,15 @@ def test_first_tokens_and_single_token_requests(cases):
 
 def test_which_kernels_take_the_norms(cases):
     """The residual add and the norm between two products, by the number of rows of the step (bfloat16,
-    sizes the MFMA products take): up to 64 rows the product in front adds and weights and the
-    product behind divides (the first norm of a step of up to 16 rows, which has no product in
-    front, runs inside the product behind it); above that they are a kernel of their own. Seen in what the kernel front end launches; the logits of
+    sizes the MFMA products take): up to 64 rows (96 against weights as small as these) the product in
+    front adds and weights and the product behind divides (the first norm of a step of up to 16 rows,
+    which has no product in front, runs inside the product behind it); above that they are a kernel
+    of their own. Seen in what the kernel front end launches; the logits of
     every one of these steps agree with the plain model."""
     case = cases[("D128", "mild")]
     toks = case.reqs["r2"]
-    assert len(toks) >= 130
-    cuts = [0, 8, 48, 130]                         # portions of 8, 40 and 82 tokens
+    assert len(toks) >= 133
+    cuts = [0, 8, 48, 133]                         # portions of 8, 40 and 85 tokens
     steps = [{"step": i, "entries": [{"id": "x", "tokens": toks[a:b], "want": list(range(b - a))}], "end": []}
              for i, (a, b) in enumerate(zip(cuts, cuts[1:]))]
     runner = runner_for(case, "bfloat16", steps)
@@ -190,8 +191,8 @@ def test_which_kernels_take_the_norms(cases):
     assert seen[0].count("mv_gemm_skinny_scaled") == 2 * layers - 1 and seen[0].count("mv_add_rmsnorm") == 1
     assert seen[1].count("mv_gemm_skinny_fold") == 2 * layers - 1
     assert seen[1].count("mv_gemm_skinny_scaled") == 2 * layers - 1 and seen[1].count("mv_add_rmsnorm") == 2
-    assert "mv_gemm_skinny_fold" not in seen[2] and seen[2].count("mv_add_rmsnorm") == 2 * layers + 1
-    assert len(got) == 130
+    assert seen[2].count("mv_gemm_skinny_fold") == 2 * layers - 1 and seen[2].count("mv_add_rmsnorm") == 2   # small weights: up to 96 rows
+    assert len(got) == 133
     for (rid, pos), row in got.items():
         assert rel_err(row, case.want["r2"][pos]) <= case.tol("bfloat16")
 
