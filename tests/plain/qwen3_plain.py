@@ -33,7 +33,7 @@ def rope_cos_sin(positions: torch.Tensor, rotary_dim: int, theta: float, dtype=t
     takes cosine and sine of those float32 angles in ``dtype``. Returns (cos, sin), each
     [n, rotary_dim / 2]."""
     inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float) / rotary_dim))
-    freqs = torch.einsum("i,j->ij", positions.to(torch.float), inv_freq)
+    freqs = torch.einsum("i,j->ij", positions.to(torch.float), inv_freq.to(positions.device))
     return freqs.to(dtype).cos(), freqs.to(dtype).sin()
 
 
@@ -57,7 +57,7 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
     Hkv = k.shape[1]
     group = H // Hkv
     out = torch.empty_like(q)
-    idx = torch.arange(n)
+    idx = torch.arange(n, device=q.device)
     allowed = idx[None, :] <= idx[:, None]
     if window is not None:
         allowed &= idx[None, :] >= idx[:, None] - window
@@ -147,23 +147,25 @@ def decoder_layer(cfg: Dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tensor
 
 
 def forward(cfg: Dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=torch.float64,
-            first_position: int = 0, rnd=_identity) -> torch.Tensor:
+            first_position: int = 0, rnd=_identity, device=None) -> torch.Tensor:
     """minivllm/models/models/qwen3.py:178-190,206-220 — embed, layers, final norm, head (tied
     to the embedding when ``tie_word_embeddings``, qwen3.py:203-204). Returns the logits of every
     position, [n, vocab]. ``first_position`` shifts all positions (for invariance tests).
     ``rnd`` is applied to every activation a reduced-precision implementation would store
     (outputs of projections, norms, rotary embedding, attention, activation); with
     ``round_to_bfloat16`` the result shows how far bfloat16 storage alone moves the logits of
-    this model and input, which is what an engine's bfloat16 error is measured against."""
-    w = {k: v.to(dtype) for k, v in weights.items()}
-    ids = torch.tensor(tokens, dtype=torch.long)
-    positions = torch.arange(first_position, first_position + len(tokens))
+    this model and input, which is what an engine's bfloat16 error is measured against.
+    ``device``: where these tensor operations run (the CPU unless a test of very long sequences
+    says otherwise: a square of scores per head is slow there); the result is on the CPU."""
+    w = {k: v.to(device=device, dtype=dtype) for k, v in weights.items()}
+    ids = torch.tensor(tokens, dtype=torch.long, device=device)
+    positions = torch.arange(first_position, first_position + len(tokens), device=device)
     x = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
         x = decoder_layer(cfg, w, i, x, positions, rnd)
     x = rnd(rms_norm(x, w["model.norm.weight"], cfg.get("rms_norm_eps", 1e-6)))
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
-    return x @ head.T
+    return (x @ head.T).cpu()
 
 
 # ---------------------------------------------------------------------------------------

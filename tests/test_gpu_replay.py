@@ -12,19 +12,22 @@ import pytest
 import torch
 
 import trace_tools
-from helpers import (TINY, TOL_F32, bf16_tolerance, make_weights, plain_logits, plain_logits_bf16, random_tokens,
-                     rel_err, write_model_dir)
+from helpers import (TINY, TOL_F32, bf16_tolerance, f32_tolerance, make_weights, plain_logits, plain_logits_bf16,
+                     plain_logits_f32, random_tokens, rel_err, write_model_dir)
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-STORED = {"A": torch.float32, "B": torch.bfloat16, "C": torch.bfloat16, "D128": torch.bfloat16, "D64": torch.bfloat16}
+STORED = {"A": torch.float32, "B": torch.bfloat16, "C": torch.bfloat16, "D128": torch.bfloat16, "D64": torch.bfloat16,
+          "W64": torch.bfloat16}
 LENGTHS = {"A": [70, 5, 33, 17, 1 + 32, 49], "B": [91, 40, 66, 2, 58, 35], "C": [50, 36, 77],
-           "D128": [70, 5, 133, 17, 49], "D64": [91, 40, 66, 2, 158]}
+           "D128": [70, 5, 133, 17, 49], "D64": [91, 40, 66, 2, 158], "W64": [120, 44, 90, 3, 77]}
 # D128 and D64 have the head sizes the MFMA attention kernels serve (on pages of 16 and 32) and widths
 # the MFMA products serve: in bfloat16 every cutting below runs the serving kernels with them
-PAGE = {"A": 16, "B": 16, "C": 16, "D128": 16, "D64": 32}
-NAMES = ["A", "B", "C", "D128", "D64"]
+# W64 is the head size 64 again with a window of 38 keys on two of its three layers, shorter than its
+# longest requests: the same kernels with a window, on pages the window gives back while a request runs
+PAGE = {"A": 16, "B": 16, "C": 16, "D128": 16, "D64": 32, "W64": 16}
+NAMES = ["A", "B", "C", "D128", "D64", "W64"]
 # sharp: the q/k norm weights are scaled so that attention is peaked and one lost or wrong key shows;
 # rounding is amplified with it, so the bfloat16 bound of these cases is wide. mild: the same case with
 # the weights as drawn, where the bfloat16 bound is at most 2e-2 and a small systematic error shows.
@@ -128,7 +131,7 @@ def test_mixed(cases, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["B", "D128"])
+@pytest.mark.parametrize("name", ["B", "D128", "W64"])
 def test_mixed_with_poisoned_pages(cases, name, dtype):
     """The mixed cutting with the debugging switch that fills every page with NaN when it changes
     hands: a kernel that reads a slot nobody has written since (masked or not: 0 x NaN is NaN), or a
@@ -213,17 +216,18 @@ def test_long_decoding(cases):
         assert worst <= tol[dtype]
 
 
+@pytest.mark.parametrize("kind", ["sharp", "mild"])
 @pytest.mark.parametrize("head_dim,page_size", [(128, 16), (64, 32), (48, 16)])
-def test_contexts_beyond_a_thousand_tokens(tmp_path, head_dim, page_size):
+def test_contexts_beyond_a_thousand_tokens(tmp_path, head_dim, page_size, kind):
     """Requests of 1100 to 2300 tokens: prompts in portions of up to 400 tokens, then a hundred and
     more decoded one by one across the lengths at which the decode graphs and the prompt kernel
     change their launch (1024, 2048), three live at a time beside each other. Sharp attention: a
-    far key that is lost shows."""
+    far key that is lost shows. Mild: the weights as drawn, where the bfloat16 bound is 2e-2 at most."""
     cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 96,
            "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": head_dim, "intermediate_size": 160,
            "vocab_size": 211, "max_position_embeddings": 4096, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
            "tie_word_embeddings": False, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
-    weights = make_weights(cfg, seed=head_dim, stored=torch.bfloat16, qk_gain=2.5)
+    weights = make_weights(cfg, seed=head_dim, stored=torch.bfloat16, qk_gain=GAINS[kind])
     path = write_model_dir(str(tmp_path / "long"), cfg, weights)
     lengths = {"a": 1100, "b": 2300, "c": 1290, "d": 2100}
     reqs = {rid: random_tokens(cfg, n, seed=n) for rid, n in lengths.items()}
@@ -239,7 +243,9 @@ def test_contexts_beyond_a_thousand_tokens(tmp_path, head_dim, page_size):
         assert len(got) == sum(lengths.values())
         worst = max(rel_err(row, want[rid][pos]) for (rid, pos), row in got.items())
         tol = TOL_F32 if dtype == "float32" else bf16_tolerance(bf16_err)
-        print(f"long contexts, head size {head_dim} [{dtype}]: worst relative error {worst:.3e} (allowed {tol:.3e})")
+        if kind == "mild" and dtype == "bfloat16":
+            tol = min(tol, MILD_BF16_BOUND)
+        print(f"long contexts, head size {head_dim}, {kind} [{dtype}]: worst relative error {worst:.3e} (allowed {tol:.3e})")
         assert worst <= tol
         runner.manager.check_invariants()
         assert all(pool.num_free == pool.num_pages for pool in runner.manager.pools)
@@ -271,17 +277,19 @@ def test_trace_run_program(cases, tmp_path):
         case.check(got, dtype, "bin/trace_run mixed")
 
 
-def test_layer_sizes_of_the_0_6b_shape(tmp_path):
+@pytest.mark.parametrize("kind", ["sharp", "mild"])
+def test_layer_sizes_of_the_0_6b_shape(tmp_path, kind):
     """The layer sizes of Qwen3-0.6B (hidden 1024, 16/8 heads of 128, intermediate 3072, vocabulary
     151936, tied head, theta 1e6) with four layers, in all four cuttings (whole, the last 32 tokens
     one by one, portions down to two tokens, mixed with a second request on recycled pages), in
     float32 and bfloat16, against the plain model. This is the shape the
-    MFMA kernels are tuned for (head size 128, K = 1024/2048/3072)."""
+    MFMA kernels are tuned for (head size 128, K = 1024/2048/3072). Sharp: q/k norm weights times 1.5;
+    mild: as drawn, with the bfloat16 bound at 2e-2 at most."""
     cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 4, "hidden_size": 1024,
            "num_attention_heads": 16, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 3072,
            "vocab_size": 151936, "max_position_embeddings": 40960, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
            "tie_word_embeddings": True, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
-    weights = make_weights(cfg, seed=6, stored=torch.bfloat16, std=0.02, qk_gain=1.5)
+    weights = make_weights(cfg, seed=6, stored=torch.bfloat16, std=0.02, qk_gain=1.5 if kind == "sharp" else 1.0)
     path = write_model_dir(str(tmp_path / "shape06"), cfg, weights)
     reqs = {"p": random_tokens(cfg, 83, seed=1), "q": random_tokens(cfg, 40, seed=2)}
     w64 = {k: v.double() for k, v in weights.items()}            # converted once: the table is large
@@ -295,12 +303,150 @@ def test_layer_sizes_of_the_0_6b_shape(tmp_path):
     from minivllm_amd.engine.trace import TraceRunner
     for dtype in ("float32", "bfloat16"):
         tol = TOL_F32 if dtype == "float32" else bf16_tolerance(bf16_err)
+        if kind == "mild" and dtype == "bfloat16":
+            tol = min(tol, MILD_BF16_BOUND)
         for what, steps in cuttings.items():
             runner = TraceRunner(path, dtype, trace_tools.max_live_tokens(steps), page_size=16)
             got = trace_tools.collect(steps, runner.run_step)
             worst = max(rel_err(row, want[rid][pos]) for (rid, pos), row in got.items())
-            print(f"0.6B layer sizes, {what} [{dtype}]: {len(got)} rows, worst relative error {worst:.3e} "
+            print(f"0.6B layer sizes, {kind}, {what} [{dtype}]: {len(got)} rows, worst relative error {worst:.3e} "
                   f"(allowed {tol:.3e})")
             assert len(got) == (123 if what != "last 32 one by one" else 66) and worst <= tol
             del runner
             torch.cuda.empty_cache()
+
+
+def _check_rows(got, want, tol, what):
+    worst, where = 0.0, None
+    for (rid, pos), row in got.items():
+        e = rel_err(row, want[rid][pos])
+        if e > worst:
+            worst, where = e, (rid, pos)
+    print(f"{what}: {len(got)} rows, worst relative error {worst:.3e} at {where} (allowed {tol:.3e})")
+    assert worst <= tol, f"{what}: worst relative error {worst:.3e} at {where} exceeds {tol:.1e}"
+
+
+@pytest.mark.parametrize("kind", ["sharp", "mild"])
+def test_contexts_across_the_graph_caps(tmp_path, kind):
+    """Requests of 4,160, 8,260 and 16,450 tokens, three live: prompts in portions of up to 2,048
+    tokens side by side, then 110 tokens each decoded one by one, alone and in changing company, so
+    that the decode steps are planned for contexts of up to 4,096, 8,192, 16,384 and 32,768 keys (the
+    longest live context decides) and every request crosses one of these lengths while it decodes.
+    Head size 128 on pages of 16: in bfloat16 the MFMA kernels, the fused decode attention and its
+    key splits. Every row against the plain model (minivllm/models/layers/attention.py:84-91:
+    attention over all of a request's keys, whatever their number)."""
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 128,
+           "num_attention_heads": 2, "num_key_value_heads": 1, "head_dim": 128, "intermediate_size": 192,
+           "vocab_size": 211, "max_position_embeddings": 32768, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+           "tie_word_embeddings": False, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
+    # (sharp: q/k norm weights times 1.5, not 2.5: with heads of 128 over 16,000 keys, 2.5 makes scores of
+    # 70, and rounding q and k to bfloat16 alone then moves the logits by a quarter of their size)
+    weights = make_weights(cfg, seed=41, stored=torch.bfloat16, qk_gain=1.5 if kind == "sharp" else 1.0)
+    path = write_model_dir(str(tmp_path / "caps"), cfg, weights)
+    prompt_lens = {"a": 4050, "b": 8150, "c": 16340}
+    reqs = {rid: random_tokens(cfg, n + 110, seed=n) for rid, n in prompt_lens.items()}
+    want, bf16_err, f32_err = {}, 0.0, 0.0
+    for rid, toks in reqs.items():
+        # (the plain model's tensor operations on the GPU here: 16,450 x 16,450 scores a head in float64
+        # take a minute and a half on the CPU)
+        want[rid] = plain_logits(cfg, weights, toks, device="cuda")
+        emulated = plain_logits_bf16(cfg, weights, toks, device="cuda")
+        bf16_err = max(bf16_err, max(rel_err(emulated[p], want[rid][p]) for p in range(len(toks))))
+        emulated = plain_logits_f32(cfg, weights, toks, device="cuda")
+        f32_err = max(f32_err, max(rel_err(emulated[p], want[rid][p]) for p in range(len(toks))))
+        del emulated
+    subsets = [["a"], ["a", "b"], ["a", "b", "c"], ["b", "c"], ["c"], ["b"], ["a", "c"]]
+    steps = trace_tools.prompts_then_subsets(reqs, prompt_lens, subsets, seed=3, max_portion=2048)
+    from minivllm_amd.engine.trace import TraceRunner
+    for dtype in ("float32", "bfloat16"):
+        runner = TraceRunner(path, dtype, trace_tools.max_live_tokens(steps), page_size=16)
+        got = trace_tools.collect(steps, runner.run_step)
+        assert len(got) == sum(len(t) for t in reqs.values())
+        # (sharp attention over 16,000 keys has rows that the plain model itself, evaluated in float32,
+        # gets wrong by more than that: the float32 bound of the sharp copy comes from that; the mild copy keeps 3e-5)
+        tol = bf16_tolerance(bf16_err) if dtype == "bfloat16" else (TOL_F32 if kind == "mild" else f32_tolerance(f32_err))
+        if kind == "mild" and dtype == "bfloat16":
+            tol = min(tol, MILD_BF16_BOUND)
+        _check_rows(got, want, tol, f"contexts across the graph caps, {kind} [{dtype}]")
+        if dtype == "bfloat16":
+            caps = sorted({key[1] for key in runner.executor._graphs})
+            limit = runner.executor.config.max_model_len       # below 32,768: the pool's tokens
+            assert caps == [4096, 8192, 16384, limit], caps
+        runner.manager.check_invariants()
+        del runner
+        torch.cuda.empty_cache()
+
+
+def _crowd_case(case, n_requests, seed):
+    rng = np.random.default_rng(seed)
+    prompt_lens = {f"c{i}": int(rng.integers(4, 21)) for i in range(n_requests)}
+    reqs = {rid: random_tokens(case.cfg, n + int(rng.integers(14, 41)), seed=1000 * seed + i)
+            for i, (rid, n) in enumerate(prompt_lens.items())}
+    want = {rid: plain_logits(case.cfg, case.weights, toks) for rid, toks in reqs.items()}
+    emulated = {rid: plain_logits_bf16(case.cfg, case.weights, toks) for rid, toks in reqs.items()}
+    bf16_err = max(rel_err(emulated[r][p], want[r][p]) for r, t in reqs.items() for p in range(len(t)))
+    return reqs, prompt_lens, want, bf16_err
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_live", [70, 130])
+def test_crowded_steps(cases, n_live, dtype):
+    """70 and 130 requests live at once (head size 128): their prompts in small portions side by side,
+    portions beside decoded tokens, then decode-only steps of all of them, whose number falls to one
+    as the requests end: every graph bucket from 144 down (the reference's buckets,
+    minivllm/executor/graph.py:11-12), the decode attention with two workgroups a compute unit, the
+    norms folded into the products up to 96 rows and the library's products beyond."""
+    from minivllm_amd.engine.trace import TraceRunner
+    for case in both(cases, "D128"):
+        reqs, prompt_lens, want, bf16_err = _crowd_case(case, n_live, seed=n_live)
+        steps = trace_tools.crowd(reqs, prompt_lens, seed=n_live)
+        sizes = [len(st["entries"]) for st in steps if all(len(e["tokens"]) == 1 for e in st["entries"])]
+        assert max(sizes) == n_live and min(sizes) <= 8
+        runner = TraceRunner(case.dir, dtype, trace_tools.max_live_tokens(steps), page_size=case.page, max_live=n_live)
+        got = trace_tools.collect(steps, runner.run_step)
+        assert len(got) == sum(len(t) for t in reqs.values())
+        tol = TOL_F32 if dtype == "float32" else bf16_tolerance(bf16_err)
+        if case.kind == "mild" and dtype == "bfloat16":
+            tol = min(tol, MILD_BF16_BOUND)
+        _check_rows(got, want, tol, f"{n_live} live requests, {case.kind} [{dtype}]")
+        if dtype == "bfloat16":
+            buckets = {key[0] for key in runner.executor._graphs}
+            assert max(buckets) >= n_live and min(buckets) <= 8 and len(buckets) >= 5
+        runner.manager.check_invariants()
+        assert all(pool.num_free == pool.num_pages for pool in runner.manager.pools)
+        del runner
+        torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_beyond_the_last_graph_bucket(cases, dtype):
+    """260 live requests: more than the largest graph bucket holds (256), so their decode steps run
+    without a graph; the step of the 256 that are left afterwards is replayed from one."""
+    from minivllm_amd.engine.trace import TraceRunner
+    case = cases[("D128", "mild")]
+    rng = np.random.default_rng(260)
+    lengths = {f"m{i}": int(rng.integers(3, 9)) + (3 if i >= 4 else 2) for i in range(260)}
+    reqs = {rid: random_tokens(case.cfg, n, seed=5000 + i) for i, (rid, n) in enumerate(lengths.items())}
+    want = {rid: plain_logits(case.cfg, case.weights, toks) for rid, toks in reqs.items()}
+    emulated = {rid: plain_logits_bf16(case.cfg, case.weights, toks) for rid, toks in reqs.items()}
+    bf16_err = max(rel_err(emulated[r][p], want[r][p]) for r, t in reqs.items() for p in range(len(t)))
+    steps = []
+    prompt = {rid: n - (3 if i >= 4 else 2) for i, (rid, n) in enumerate(lengths.items())}
+    steps.append({"step": 0, "entries": [{"id": r, "tokens": t[:prompt[r]], "want": list(range(prompt[r]))}
+                                         for r, t in reqs.items()], "end": []})
+    for j in range(3):
+        entries, ended = [], []
+        for r, t in reqs.items():
+            p = prompt[r] + j
+            if p < len(t):
+                entries.append({"id": r, "tokens": [t[p]], "want": [0]})
+                if p + 1 == len(t):
+                    ended.append(r)
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    assert [len(s["entries"]) for s in steps] == [260, 260, 260, 256]
+    runner = TraceRunner(case.dir, dtype, trace_tools.max_live_tokens(steps), page_size=case.page, max_live=260)
+    got = trace_tools.collect(steps, runner.run_step)
+    assert len(got) == sum(lengths.values())
+    tol = TOL_F32 if dtype == "float32" else min(bf16_tolerance(bf16_err), MILD_BF16_BOUND)
+    _check_rows(got, want, tol, f"260 live requests [{dtype}]")
+    assert {key[0] for key in runner.executor._graphs} == {256}

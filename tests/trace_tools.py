@@ -120,3 +120,78 @@ def collect(steps: List[dict], run_step: Callable[[dict], Optional[np.ndarray]])
             pos.pop(rid, None)
     return out
 
+
+
+def crowd(reqs: Dict[str, List[int]], prompt_lens: Dict[str, int], seed: int = 0, max_portion: int = 9,
+          sit_out: float = 0.0) -> List[dict]:
+    """Every request is live from the first step on. Prompts go in portions of random size
+    (2..max_portion); a request whose prompt is in decodes one token a step until its tokens run out.
+    With requests of different lengths the steps go from many prompt portions side by side, through
+    portions beside decoded tokens, to decode-only steps whose number of sequences falls from all
+    requests to one. ``sit_out``: chance that a live request is left out of a step."""
+    rng = np.random.default_rng(seed)
+    live = list(reqs.keys())
+    done_upto = {rid: 0 for rid in reqs}
+    steps = []
+    while live:
+        entries, ended = [], []
+        for rid in list(live):
+            if sit_out and len(live) > 1 and rng.random() < sit_out:
+                continue
+            toks, p = reqs[rid], done_upto[rid]
+            if p < prompt_lens[rid]:
+                n = min(int(rng.integers(2, max_portion + 1)), prompt_lens[rid] - p)
+                if prompt_lens[rid] - p - n == 1:
+                    n += 1
+            else:
+                n = 1
+            chunk = toks[p:p + n]
+            done_upto[rid] = p + n
+            entries.append({"id": rid, "tokens": chunk, "want": list(range(len(chunk)))})
+            if done_upto[rid] == len(toks):
+                ended.append(rid)
+                live.remove(rid)
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
+
+
+def prompts_then_subsets(reqs: Dict[str, List[int]], prompt_lens: Dict[str, int], subsets: Sequence[Sequence[str]],
+                         seed: int = 0, max_portion: int = 2048, want_prompt_rows: bool = True) -> List[dict]:
+    """All requests live at once: first their prompts in portions of random size (2..max_portion), side
+    by side; then decode-only steps whose participants follow ``subsets`` in turn (a request that has
+    no token left is dropped from a subset), until every request has brought all its tokens. Which
+    requests share a decode step decides the longest context of the step, so the subsets take the
+    step through every launch plan the context lengths select."""
+    rng = np.random.default_rng(seed)
+    done_upto = {rid: 0 for rid in reqs}
+    steps: List[dict] = []
+    while any(done_upto[r] < prompt_lens[r] for r in reqs):
+        entries = []
+        for rid, toks in reqs.items():
+            p = done_upto[rid]
+            if p >= prompt_lens[rid]:
+                continue
+            n = min(int(rng.integers(2, max_portion + 1)), prompt_lens[rid] - p)
+            if prompt_lens[rid] - p - n == 1:
+                n += 1
+            chunk = toks[p:p + n]
+            done_upto[rid] = p + n
+            want = list(range(len(chunk))) if want_prompt_rows else []
+            entries.append({"id": rid, "tokens": chunk, "want": want})
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+    k = 0
+    while any(done_upto[r] < len(reqs[r]) for r in reqs):
+        subset = [r for r in subsets[k % len(subsets)] if done_upto[r] < len(reqs[r])]
+        k += 1
+        if not subset:
+            continue
+        entries, ended = [], []
+        for rid in subset:
+            p = done_upto[rid]
+            entries.append({"id": rid, "tokens": [reqs[rid][p]], "want": [0]})
+            done_upto[rid] = p + 1
+            if p + 1 == len(reqs[rid]):
+                ended.append(rid)
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
