@@ -70,6 +70,7 @@ struct FusedInput {
     float eps;
     int unit_offset;
     const float* table;     // [positions, D] or null
+    const float* rows;      // [tokens, D] = the table rows of the step's positions, gathered once a step, or null
     int store;
     const int* token_seq;   // rows that belong to no sequence (< 0) are left alone
 };
@@ -155,6 +156,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     } raw[ROUNDS];
     const int hw = threadIdx.x / 32, hj = threadIdx.x % 32;   // (FUSED) this lane's half wave and place in it
     float head_w[ROUNDS][E], rot_c[E], rot_s[E];
+    int first_a0 = -1, first_a1 = -1, first_b0 = -1, first_b1 = -1;   // page ids of the halves of the wave's first two blocks
     if (FUSED) {
         // a decode step: row t of the step is the one token of sequence t (or padding). Everything
         // that does not depend on the position is asked for before the position is looked at.
@@ -181,9 +183,31 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
                 }
             }
         }
+        if (fz.rows != nullptr) {   // the step's rotation rows: no need to know the position first
+            const float* cs = fz.rows + (size_t)t0 * D + (E * hj) % (D / 2);
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                rot_c[e] = cs[e];
+                rot_s[e] = cs[D / 2 + e];
+            }
+        }
         if (window < 0) {
+            // Without a window a wave's blocks are split * W + wave, + nsplit * W, ...: whatever the
+            // sequence's length. The page ids of its first two blocks come straight from the block
+            // table (uniform over the wave: scalar loads), so that their keys and values can be asked
+            // for as soon as the position is known; the ids of all later blocks go to LDS meanwhile.
             const int* bt0 = block_table + (size_t)seq * bt_width;
             int n = bt_width < max_pages ? bt_width : max_pages;
+            const int wv = __builtin_amdgcn_readfirstlane(wave);
+            auto lookup = [&](int key0) -> int {     // (any page of the table, also beyond the planned context)
+                const int pidx = key0 / page_size;
+                return pidx < bt_width ? bt0[pidx] : -1;
+            };
+            const int key_a = 32 * (split * W + wv), key_b = key_a + 32 * nsplit * W;
+            first_a0 = lookup(key_a);
+            first_a1 = lookup(key_a + 16);
+            first_b0 = lookup(key_b);
+            first_b1 = lookup(key_b + 16);
             if (n > AF_MAX_CACHED_PAGES) n = AF_MAX_CACHED_PAGES;
             for (int p = threadIdx.x; p < n; p += blockDim.x) sh_pages[p] = bt0[p];
         }
@@ -234,7 +258,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     if (FUSED) {   // known without asking the other lanes
         hi_w = pos0;
         lo_w = (window >= 0 && hi_w - window > 0) ? hi_w - window : 0;
-        if (fz.table != nullptr) {   // asked for before the keys, so that preparing the heads does not wait for keys
+        if (fz.table != nullptr && fz.rows == nullptr) {   // asked for before the keys, so that preparing the heads does not wait for keys
             const float* cs = fz.table + (size_t)(hi_w >= 0 ? hi_w : 0) * D + (E * hj) % (D / 2);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
@@ -304,8 +328,9 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         if (n_cached > AF_MAX_CACHED_PAGES) n_cached = AF_MAX_CACHED_PAGES;
         for (int r = threadIdx.x; r < n_cached; r += blockDim.x)
             sh_pages[r] = p_first + r < bt_width ? bt[p_first + r] : -1;
+        __syncthreads();
     }
-    __syncthreads();
+    // (FUSED without a window: the ids in LDS are first used behind the barrier of the head preparation)
     auto page_of = [&](int pidx) -> int {
         if (pidx >= bt_width) return -1;
         const int rel = pidx - p_first;
@@ -323,13 +348,14 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         Frag v[DT];
     };
     const int k_half = i / 8, v_half = g / 2;
-    auto fetch = [&](int b, Operands& op) {
+    // given: the caller has the page ids of the block's halves already (pg0, pg1); else they are looked up
+    auto fetch = [&](int b, Operands& op, bool given, int pg0, int pg1) {
         int slot0[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int key0 = 32 * b + 16 * h;
             const int pidx = key0 / page_size;
-            op.page[h] = (b < b_end && key0 <= hi_w) ? page_of(pidx) : -1;
+            op.page[h] = (b < b_end && key0 <= hi_w) ? (given ? (h ? pg1 : pg0) : page_of(pidx)) : -1;
             slot0[h] = key0 - pidx * page_size;
         }
         const int kpage = k_half ? op.page[1] : op.page[0];
@@ -432,8 +458,11 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
             acc_o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.v[dt].v, pop.v, acc_o[0][dt], 0, 0, 0);
     };
 
+    // two blocks are on their way before anything else is done with the position
     Operands oa, ob;
-    fetch(b_begin, oa);
+    const bool direct = FUSED && window < 0;
+    fetch(b_begin, oa, direct, first_a0, first_a1);
+    if (b_begin + b_step < b_end) fetch(b_begin + b_step, ob, direct, first_b0, first_b1);
     if (FUSED) {
         // while those loads are in flight: the group's query heads (and the new key, in the workgroup
         // that will meet it) are prepared by half a wave each and handed round through LDS
@@ -442,8 +471,8 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
             if (r * HW > G) break;
             const int h = hw + r * HW;
             if (h < G || (h == G && wg_owns_new))          // uniform over the half wave, and the exchange stays inside it
-                prepare_head_spread<D>(raw[r].s, hj, fz.has_norm != 0, head_w[r], fz.eps, fz.table != nullptr, rot_c, rot_s,
-                                       &sh_heads[h][E * hj]);
+                prepare_head_spread<D>(raw[r].s, hj, fz.has_norm != 0, head_w[r], fz.eps,
+                                       fz.table != nullptr || fz.rows != nullptr, rot_c, rot_s, &sh_heads[h][E * hj]);
         }
         __syncthreads();
 #pragma unroll
@@ -470,11 +499,14 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         }
     }
     for (int b = b_begin; b < b_end; b += 2 * b_step) {
-        fetch(b + b_step, ob);
         compute(b, oa);
         if (b + b_step >= b_end) break;
-        fetch(b + 2 * b_step, oa);
+        // Beyond the last block a fetch loads nothing and clears the registers. A wave of a grid that
+        // fits the chip has two or three blocks and skips that; in the long loops of crowded grids the
+        // straight line is faster (the branch costs the compiler its exact wait counts).
+        if (OCC != 1 || b + 2 * b_step < b_end) fetch(b + 2 * b_step, oa, false, -1, -1);
         compute(b + b_step, ob);
+        if (OCC != 1 || b + 3 * b_step < b_end) fetch(b + 3 * b_step, ob, false, -1, -1);
     }
 
     // the sum of a column is spread over the four lane groups
@@ -702,13 +734,16 @@ extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long
 // [q | k | v] product (one token a sequence; row t of qkv belongs to sequence t): per-head RMSNorm
 // (q_weight / k_weight, or null for none) and rotation by the table row of the position
 // (half-split pairs over the whole head, or null for none) happen on the way into the kernel;
+// `rows` [tokens, D], when given, holds the table's rows of the step's positions (row t for token t),
+// gathered once a step, so that no layer has to wait for the position before it can ask for the angles;
 // with store_kv the new key and value are written to their page slot as well.
 extern "C" int mv_attention_decode_fused(const void* qkv, long qkv_stride, int q_off, int k_off, int v_off, void* out,
                                          long out_stride, void* k_pages, void* v_pages, const int* block_table,
                                          int bt_width, int page_size, const int* positions, const int* cu_seqlens,
                                          int n_seqs, int H, int Hkv, int D, float scale, int window,
                                          const void* q_weight, const void* k_weight, int weight_dtype, float eps,
-                                         int unit_offset, const float* table, int store_kv, float* partials,
+                                         int unit_offset, const float* table, const float* rows, int store_kv,
+                                         float* partials,
                                          int* counters, int nsplit, int max_pages, int waves, const int* token_seq,
                                          hipStream_t stream) {
     if (int rc = check_common("attention_decode_fused", qkv_stride, out_stride, page_size, bt_width, H, Hkv, D))
@@ -724,8 +759,10 @@ extern "C" int mv_attention_decode_fused(const void* qkv, long qkv_stride, int q
                              ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0),
                "attention_decode_fused: bad norm weights (missing, unknown type or not 16-byte aligned) or eps");
     MV_REQUIRE(table == nullptr || ((uintptr_t)table % 16) == 0, "attention_decode_fused: the table is not 16-byte aligned");
+    MV_REQUIRE(rows == nullptr || (table != nullptr && ((uintptr_t)rows % 16) == 0),
+               "attention_decode_fused: rotation rows come with their table and are 16-byte aligned");
     FusedInput fz{(const bf16*)qkv, qkv_stride, q_off, k_off, v_off, WeightPtr{q_weight, weight_dtype},
-                  WeightPtr{k_weight, weight_dtype}, has_norm, eps, unit_offset, table, store_kv ? 1 : 0, token_seq};
+                  WeightPtr{k_weight, weight_dtype}, has_norm, eps, unit_offset, table, rows, store_kv ? 1 : 0, token_seq};
     return decode_common(true, fz, nullptr, 0, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size,
                          positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, partials, counters, nsplit, max_pages,
                          waves, token_seq, stream);

@@ -27,6 +27,42 @@ extern "C" int mv_embedding(const int* ids, const void* table, int table_dtype, 
     return mv_check_launch("embedding");
 }
 
+// The embedding and, in the same launch, a second gather of float rows: out2[n, :] = table2[ids2[n], :]
+// (the rows of a position table at the step's positions, say). The first kernel of a step carries it,
+// so that it costs no launch of its own.
+__global__ void embedding_gather_kernel(const int* __restrict__ ids, WeightPtr table, float* __restrict__ resid, int h,
+                                        int vocab, float scale, const int* __restrict__ ids2,
+                                        const float* __restrict__ table2, float* __restrict__ out2, int h2, int rows2) {
+    const int row = blockIdx.x;
+    if (blockIdx.y == 0) {
+        const int id = ids[row];
+        const bool valid = id >= 0 && id < vocab;
+        float* dst = resid + (size_t)row * h;
+        const size_t base = (size_t)(valid ? id : 0) * h;
+        for (int d = threadIdx.x; d < h; d += blockDim.x) dst[d] = valid ? table.at(base + d) * scale : 0.f;
+    } else {
+        const int id = ids2[row];
+        const bool valid = id >= 0 && id < rows2;
+        const float* src = table2 + (size_t)(valid ? id : 0) * h2;
+        float* dst = out2 + (size_t)row * h2;
+        for (int d = threadIdx.x; d < h2; d += blockDim.x) dst[d] = valid ? src[d] : 0.f;
+    }
+}
+
+extern "C" int mv_embedding_gather(const int* ids, const void* table, int table_dtype, float* resid, int n, int h,
+                                   int vocab, float scale, const int* ids2, const float* table2, float* out2, int h2,
+                                   int rows2, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && h > 0 && vocab > 0, "embedding: bad sizes n=%d h=%d vocab=%d", n, h, vocab);
+    MV_REQUIRE(mv_valid_dtype(table_dtype), "embedding: bad table dtype %d", table_dtype);
+    MV_REQUIRE(ids2 != nullptr && table2 != nullptr && out2 != nullptr && h2 > 0 && rows2 > 0,
+               "embedding: the second gather needs ids, a table of %d rows of %d and an output", rows2, h2);
+    if (n == 0) return 0;
+    WeightPtr w{table, table_dtype};
+    hipLaunchKernelGGL(embedding_gather_kernel, dim3(n, 2), dim3(256), 0, stream, ids, w, resid, h, vocab, scale, ids2,
+                       table2, out2, h2, rows2);
+    return mv_check_launch("embedding_gather");
+}
+
 // Eight consecutive elements, read and written 16 bytes (bf16) or 32 bytes (float) at a time.
 template <typename T> struct Vec8;
 template <> struct Vec8<bf16> {

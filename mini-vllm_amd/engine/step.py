@@ -98,6 +98,8 @@ class StepContext:
         self._kv: Dict[int, "KVView"] = {}
         self._state: Dict[int, torch.Tensor] = {}
         self.page_size = 0
+        # rows that a position encoding had gathered for this step (PositionEncoding.step_gather), by part
+        self.position_rows: Dict[object, torch.Tensor] = {}
 
     def kv(self, call: int) -> KVView:
         try:

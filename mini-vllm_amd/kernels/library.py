@@ -90,11 +90,14 @@ _OPTIONAL_SIGNATURES = {
                                     c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     # qkv, stride, q_off, k_off, v_off, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size,
     # positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, q_weight, k_weight, weight_dtype, eps, unit_offset,
-    # table, store_kv, partials, counters, nsplit, max_pages, waves, token_seq, stream
+    # table, rows, store_kv, partials, counters, nsplit, max_pages, waves, token_seq, stream
     "mv_attention_decode_fused": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p,
                                           c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                          c_float, c_int, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_int,
-                                          c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+                                          c_float, c_int, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p,
+                                          c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    # ids, table, table_dtype, resid, n, h, vocab, scale, ids2, table2, out2, h2, rows2, stream
+    "mv_embedding_gather": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
+                                    c_void_p, c_int, c_int, c_void_p]),
     "mv_attention_prefill": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                      c_int, c_void_p]),

@@ -201,17 +201,46 @@ class Ops:
             raise KernelLibraryError(f"{what} has dtype {t.dtype}, expected {self.dtype}")
 
     # ------------------------------------------------------------------------------------
-    def embedding(self, ids: torch.Tensor, table: torch.Tensor, resid: torch.Tensor, scale: float = 1.0) -> None:
-        """resid[n] = table[ids[n]] * scale; ids int32 [n], resid float32 [n, h]."""
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor, resid: torch.Tensor, scale: float = 1.0,
+                  gather: Optional[tuple] = None) -> None:
+        """resid[n] = table[ids[n]] * scale; ids int32 [n], resid float32 [n, h].
+
+        ``gather`` = (index int32 [>= n], float32 table [rows, w], float32 out [n, w]) rides on the same
+        launch: out[n] = table[index[n]] (rows outside the table give zeros)."""
         _dev(ids, "ids"); _dev(table, "embedding table"); _dev(resid, "residual")
         n, h = resid.shape
         if ids.dtype != torch.int32 or ids.numel() < n or resid.dtype != torch.float32:
             raise KernelLibraryError("embedding: ids must be int32 [>= n] and the residual float32 [n, h]")
         if table.dim() != 2 or table.shape[1] != h or not table.is_contiguous() or not resid.is_contiguous():
             raise KernelLibraryError(f"embedding: table {tuple(table.shape)} does not fit residual {tuple(resid.shape)}")
+        if gather is not None:
+            index, table2, out2 = gather
+            self._check_gather(index, table2, out2, n)
+            self._note("mv_embedding", n * h * (table.element_size() + 4) + n * 4 + n * (8 * out2.shape[1] + 4))
+            self.lib.call("mv_embedding_gather", ids.data_ptr(), table.data_ptr(), _weight_code(table, "embedding table"),
+                          resid.data_ptr(), n, h, table.shape[0], float(scale), index.data_ptr(), table2.data_ptr(),
+                          out2.data_ptr(), table2.shape[1], table2.shape[0], self._stream())
+            return
         self._note("mv_embedding", n * h * (table.element_size() + 4) + n * 4)
         self.lib.call("mv_embedding", ids.data_ptr(), table.data_ptr(), _weight_code(table, "embedding table"),
                       resid.data_ptr(), n, h, table.shape[0], float(scale), self._stream())
+
+    @staticmethod
+    def _check_gather(index: torch.Tensor, table: torch.Tensor, out: torch.Tensor, n: int) -> None:
+        _dev(index, "gather index"); _dev(table, "gather table"); _dev(out, "gathered rows")
+        if index.dtype != torch.int32 or index.numel() < n:
+            raise KernelLibraryError("gather: the index must be int32 with a row for every token")
+        if (table.dtype != torch.float32 or table.dim() != 2 or not table.is_contiguous() or out.dtype != torch.float32
+                or out.shape != (n, table.shape[1]) or not out.is_contiguous()):
+            raise KernelLibraryError(f"gather: float32 table {tuple(table.shape)} does not fit float32 rows {tuple(out.shape)}")
+
+    def gather_rows(self, index: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+        """out[n] = table[index[n]] for a float32 table (rows outside it give zeros)."""
+        n = out.shape[0]
+        self._check_gather(index, table, out, n)
+        self._note("mv_embedding", n * (8 * out.shape[1] + 4))
+        self.lib.call("mv_embedding", index.data_ptr(), table.data_ptr(), DTYPE_F32, out.data_ptr(), n, table.shape[1],
+                      table.shape[0], 1.0, self._stream())
 
     def add_rmsnorm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional[torch.Tensor],
                     eps: float, out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
@@ -799,11 +828,12 @@ class Ops:
                                head_dim: int, scale: float, window: Optional[int], plan,
                                q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                                rope_table: Optional[torch.Tensor], interleaved: bool, store_kv: bool,
-                               unit_offset: bool = False) -> bool:
+                               unit_offset: bool = False, rope_rows: Optional[torch.Tensor] = None) -> bool:
         """A decode step's attention straight from the raw rows ``qkv`` = [q | k | v] (or [q] alone
         without ``store_kv``): per-head norm, rotation, cache write and attention in one kernel.
         Returns False, having done nothing, when the step or the sizes are not taken; the caller
-        then runs ``qk_norm_rope_store`` and ``attention``."""
+        then runs ``qk_norm_rope_store`` and ``attention``. ``rope_rows`` float32 [tokens, D]: the rows of
+        ``rope_table`` at the step's positions, when something gathered them earlier in the step."""
         if (not self.use_fast_kernels or plan is None or not plan.decode_only
                 or not self.lib.has("mv_attention_decode_fused")):
             return False
@@ -840,13 +870,17 @@ class Ops:
         _dev(block_table, "block table")
         if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
             raise KernelLibraryError("attention: the block table must be a contiguous int32 matrix")
+        if rope_rows is not None and (rope_table is None or rope_rows.dtype != torch.float32 or not rope_rows.is_cuda
+                                      or rope_rows.shape != (n, D) or not rope_rows.is_contiguous()
+                                      or rope_rows.data_ptr() % 16):
+            rope_rows = None
         nsplit, partials = self._decode_split(plan, n, H, Hkv, D)
         self._note_attention("mv_attention_decode_fused", plan, n, H, Hkv, D, 2, splits=nsplit)
         self.lib.call("mv_attention_decode_fused", qkv.data_ptr(), stride, 0, H * D, (H + Hkv) * D, out.data_ptr(), os_,
                       k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n, H, Hkv, D, float(scale),
                       -1 if window is None else int(window), _ptr(q_weight), _ptr(k_weight), wcode, float(eps),
-                      int(unit_offset), _ptr(rope_table), int(store_kv), _ptr(partials),
+                      int(unit_offset), _ptr(rope_table), _ptr(rope_rows), int(store_kv), _ptr(partials),
                       self._split_counters(n * Hkv, partials), nsplit, -(-max(1, plan.max_context_len) // page_size),
                       DECODE_ATTENTION_WAVES, token_seq.data_ptr(), self._stream())
         return True

@@ -92,6 +92,7 @@ class CausalLM:
         self.head = head_cls(plan.head, fetch(None, "head", head_cls.tensors(plan.head)), rt)
 
         position_parts: Dict[object, object] = {}
+        self.position_parts = position_parts
         self.graph_safe = True          # every part allows its forward to be captured in a graph
         self.blocks = []
         self.mixers = []
@@ -158,7 +159,16 @@ class CausalLM:
         rt, plan = self.rt, self.plan
         n = ctx.n_tokens
         resid = rt.workspace.get("resid", (n, plan.hidden_size), torch.float32)
-        self.embedding.forward(ctx, resid)
+        # what position encodings want gathered for the whole step rides on the first kernel
+        ctx.position_rows = {}
+        gathers = [job for job in (part.step_gather(ctx) for part in self.position_parts.values()
+                                   if hasattr(part, "step_gather")) if job is not None]
+        if gathers and getattr(self.embedding, "carries_gather", False):
+            self.embedding.forward(ctx, resid, gather=gathers.pop(0))
+        else:
+            self.embedding.forward(ctx, resid)
+        for index, table, out in gathers:
+            rt.ops.gather_rows(index, table, out)
         stream = HiddenStream(resid, rt.workspace.get("resid.spare", (n, plan.hidden_size), torch.float32))
         for call_index, call in enumerate(plan.calls):
             block = self.blocks[call.layer]

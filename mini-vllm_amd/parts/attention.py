@@ -127,7 +127,8 @@ class Attention(Mixer):
             if ops.attention_decode_fused(qkv, attn, kv.k_pages, kv.v_pages, kv.block_table, kv.page_size,
                                           ctx.positions, ctx.token_seq, spec.num_heads, spec.num_kv_heads,
                                           spec.head_dim, spec.scale, spec.window, plan, self.q_norm, self.k_norm,
-                                          spec.qk_norm_eps, table, interleaved, not spec.shares_kv):
+                                          spec.qk_norm_eps, table, interleaved, not spec.shares_kv,
+                                          rope_rows=ctx.position_rows.get(self.position)):
                 y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
                 return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True, fold=fold) or y
         ops.qk_norm_rope_store(

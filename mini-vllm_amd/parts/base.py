@@ -386,6 +386,13 @@ class PositionEncoding(Part):
         """In place on q [n, H, D] and k [n, Hkv, D] views, for encodings without a table."""
         raise NotImplementedError
 
+    def step_gather(self, ctx):
+        """Asked once per step, in front of the layers: (index int32 [tokens], float32 table [rows, w],
+        float32 out [tokens, w]) when the encoding wants ``out[t] = table[index[t]]`` prepared for the
+        step (it leaves ``out`` in ``ctx.position_rows[self]`` for its mixers), else None. The
+        model lets the step's first kernel carry the gather."""
+        return None
+
 
 class Mixer(Part):
     """forward(x, ctx, call) -> y: mixes information along the sequence. ``call`` identifies
@@ -413,7 +420,11 @@ class FeedForward(Part):
 
 
 class Embedding(Part):
-    """forward(ctx, resid): fills the float32 residual stream [tokens, hidden] from ``ctx.token_ids``."""
+    """forward(ctx, resid): fills the float32 residual stream [tokens, hidden] from ``ctx.token_ids``.
+    An embedding that declares ``carries_gather = True`` takes ``gather=`` (see
+    ``PositionEncoding.step_gather``) and runs it in its own launch; for any other the model runs
+    the gather as a kernel of its own."""
+    carries_gather: ClassVar[bool] = False
 
     def forward(self, ctx, resid: torch.Tensor) -> None:
         raise NotImplementedError

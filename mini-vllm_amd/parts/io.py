@@ -22,6 +22,7 @@ from .plan import EmbeddingSpec, HeadSpec
 @register_embedding(EmbeddingSpec.kind)
 class TokenEmbedding(Embedding):
     spec_class = EmbeddingSpec
+    carries_gather = True
 
     @classmethod
     def tensors(cls, spec: EmbeddingSpec) -> Dict[str, TensorDecl]:
@@ -31,8 +32,8 @@ class TokenEmbedding(Embedding):
         self.spec, self.rt = spec, rt
         self.table = tensors["weight"]
 
-    def forward(self, ctx, resid: torch.Tensor) -> None:
-        self.rt.ops.embedding(ctx.token_ids, self.table, resid, self.spec.scale)
+    def forward(self, ctx, resid: torch.Tensor, gather=None) -> None:
+        self.rt.ops.embedding(ctx.token_ids, self.table, resid, self.spec.scale, gather=gather)
 
 
 @register_head(HeadSpec.kind)

@@ -44,3 +44,15 @@ class RotaryEmbedding(PositionEncoding):
 
     def rotary(self) -> Optional[Tuple[torch.Tensor, bool]]:
         return self.table, self.spec.interleaved
+
+    def step_gather(self, ctx):
+        """In a step of single decoded tokens every layer needs the table's rows at the same few
+        positions: they are gathered once, in front of the layers, so that no layer has to wait for a
+        position before it can ask for its angles."""
+        plan = ctx.attention_plan
+        if plan is None or not plan.decode_only or self.spec.interleaved or not self.rt.ops.use_fast_kernels:
+            return None
+        rows = self.rt.workspace.get(f"rotary.rows.{self.spec.rotary_dim}.{self.spec.theta}",
+                                     (ctx.n_tokens, self.spec.rotary_dim), torch.float32)
+        ctx.position_rows[self] = rows
+        return ctx.positions, self.table, rows

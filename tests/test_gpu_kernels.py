@@ -588,10 +588,14 @@ def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
                                                        (True, True, False)])
 @pytest.mark.parametrize("max_context", [None, 40000])
 @pytest.mark.parametrize("splits", [None, 1, 5, 64])
-def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_rope, store, max_context, splits):
+@pytest.mark.parametrize("gathered", [False, True])
+def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_rope, store, max_context, splits, gathered):
     """A decode step from the raw [q | k | v] rows: per-head norm, rotation, cache write and attention
     in one kernel. The slot of the new position holds NaN before (unless the cache is another
-    layer's and already complete), the finished key and value afterwards."""
+    layer's and already complete), the finished key and value afterwards. ``gathered``: the rotation
+    angles come as rows gathered for the step's tokens (the padding row's are NaN), not from the table."""
+    if gathered and not with_rope:
+        pytest.skip("no rotation, no rows")
     ops = ops_for(torch.bfloat16)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(21)
@@ -660,11 +664,16 @@ def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_ro
     rows = raw if store else raw[:, :H * D].contiguous()
     qkv = dev(torch.cat([rows, torch.full((1, rows.shape[1]), float("nan"), dtype=dtype)]))
     bt_rows = torch.cat([bt[live], torch.full((1, bt.shape[1]), -1, dtype=torch.int32)]).contiguous()
+    rope_rows = None
+    if gathered:
+        rope_rows = torch.full((n + 1, D), float("nan"), dtype=torch.float32, device="cuda")
+        ops.gather_rows(dev(positions), table, rope_rows[:n])
+        assert torch.equal(rope_rows[:n].cpu(), table.cpu()[positions.long()])
     took = ops.attention_decode_fused(qkv, out, kp, vp, dev(bt_rows), ps,
                                       dev(torch.cat([positions, torch.zeros(1, dtype=torch.int32)])),
                                       dev(torch.tensor(list(range(n)) + [-1], dtype=torch.int32)), H, Hkv, D, scale,
                                       window, plan, dev(qw) if with_norm else None, dev(kw) if with_norm else None,
-                                      eps, table, False, store)
+                                      eps, table, False, store, rope_rows=rope_rows)
     assert took
     out = out[:n]
     seqs = torch.arange(n, dtype=torch.int32)
