@@ -10,7 +10,8 @@ has them (``model``, ``max_model_len``, ``max_num_batched_tokens``, ``max_num_ba
   as given (the reference treats it as an upper cap, executor.py:46);
 * ``use_cuda_graph`` keeps its name; the decode step is captured in a HIP graph;
 * the executor never writes into this object (the reference's does, executor.py:49);
-* ``prefill_chunk``, ``enable_prefix_caching``, ``num_scheduler_steps``, ``launch_ahead``, ``seed`` have no
+* ``prefill_chunk``, ``enable_prefix_caching``, ``num_scheduler_steps``, ``launch_ahead``, ``seed``,
+  ``prompt_graph_max_tokens`` have no
   counterpart there (its scheduler runs whole prompts and one decoded token a step, scheduler.py:26-89).
 """
 from __future__ import annotations
@@ -74,6 +75,10 @@ class EngineConfig:
     # reference does, minivllm/executor/graph.py:24-58) instead of at a graph's first use, which
     # makes that step wait for the recording
     capture_graphs_at_start: bool = False
+    # steps that hold prompt portions (alone or beside decoded tokens) of up to this many tokens are
+    # replayed from graphs too, recorded at first use per (token bucket, sequence bucket, context cap):
+    # such steps are bound by the host's launches, not by the device (0: only decode steps use graphs)
+    prompt_graph_max_tokens: int = 2048
     # debugging: fill a cache page with NaN when it is handed out for new content and (without
     # prefix reuse, which revives given-back pages) when its last holder gives it back, so that a
     # kernel that reads a slot nobody has written since, or a page that is no longer the request's,
@@ -95,6 +100,8 @@ class EngineConfig:
             raise ValueError(f"max_num_batched_tokens must be >= 1, got {self.max_num_batched_tokens}")
         if self.max_num_batched_seqs < 1:
             raise ValueError(f"max_num_batched_seqs must be >= 1, got {self.max_num_batched_seqs}")
+        if self.prompt_graph_max_tokens < 0:
+            raise ValueError(f"prompt_graph_max_tokens must be >= 0, got {self.prompt_graph_max_tokens}")
         if self.prefill_chunk is not None and self.prefill_chunk < 1:
             raise ValueError(f"prefill_chunk must be >= 1, got {self.prefill_chunk}")
         if self.kv_cache_block_size < 1:

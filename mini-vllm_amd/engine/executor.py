@@ -37,6 +37,13 @@ from .step import AttentionPlan, KVView, SeqStep, StepContext
 logger = logging.getLogger(__name__)
 
 GRAPH_BUCKETS = [1, 2, 4, 8] + list(range(16, 257, 16))     # as the reference's (graph.py:11-12)
+# token counts that steps with prompt portions are padded to when they are replayed from a graph:
+# at most an eighth more than the step holds
+TOKEN_BUCKETS = (list(range(16, 129, 16)) + list(range(160, 257, 32)) + list(range(320, 513, 64))
+                 + list(range(640, 1025, 128)) + list(range(1280, 2049, 256)) + list(range(2560, 4097, 512))
+                 + list(range(5120, 8193, 1024)))
+# graphs of such steps kept at a time (the one used longest ago goes first)
+MIXED_GRAPHS_KEPT = 64
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -145,6 +152,8 @@ class Executor:
         self._graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, StepContext, torch.Tensor, torch.Tensor]] = {}
         self._graph_pool = None
         self._repeat_graphs: Dict[Tuple[int, int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
+        # steps with prompt portions: (token bucket, sequence bucket, logit rows, context cap) -> graph
+        self._mixed_graphs: Dict[Tuple[int, int, int, int], Tuple] = {}
         self._graph_workspace: Optional[Workspace] = None
         # what each recorded graph holds, by kind of node (see _record)
         self.graph_census: Dict[Tuple, Dict[str, int]] = {}
@@ -205,6 +214,7 @@ class Executor:
                                    for name, shape in need.page_shapes(self.page_size).items()}
         self._graphs.clear()
         self._repeat_graphs.clear()
+        self._mixed_graphs.clear()
 
     def _warmup(self, num_tokens: int) -> None:
         """One dry step of ``num_tokens`` tokens against a throw-away cache, so that every scratch
@@ -283,22 +293,25 @@ class Executor:
                                      f"{s.start + n - 1} needs {last_page + 1}")
 
     def _fill(self, seqs: Sequence[SeqStep], pad_to: Optional[int] = None, bt_widths: Optional[List[int]] = None,
-              lookahead: int = 0, extra_words: int = 0, check_pages: bool = True):
+              lookahead: int = 0, extra_words: int = 0, check_pages: bool = True, pad_tokens: Optional[int] = None,
+              pad_rows: Optional[int] = None):
         """Packs the step's integers into one int32 array. Returns (array, offsets dict, facts).
-        ``lookahead`` extends the check of the block tables to positions that later runs of a
-        repeated step touch; ``extra_words`` leaves room at the end (offset "extra", 8-byte aligned)."""
+        ``pad_to`` pads sequences (and, unless ``pad_tokens`` / ``pad_rows`` say otherwise, tokens and
+        logit rows) to a graph's size with inert rows. ``lookahead`` extends the check of the block
+        tables to positions that later runs of a repeated step touch; ``extra_words`` leaves room at
+        the end (offset "extra", 8-byte aligned)."""
         S = len(seqs)
         q_lens = [len(s.tokens) for s in seqs]
         N = sum(q_lens)
         Sp = pad_to if pad_to is not None else S
-        Np = pad_to if pad_to is not None else N
+        Np = pad_tokens if pad_tokens is not None else (pad_to if pad_to is not None else N)
         want_rows: List[int] = []
         base = 0
         for s, n in zip(seqs, q_lens):
             want_rows.extend(base + w for w in s.want)
             base += n
         M = len(want_rows)
-        Mp = pad_to if pad_to is not None else M
+        Mp = pad_rows if pad_rows is not None else (pad_to if pad_to is not None else M)
         widths = bt_widths or [max(1, max(len(s.block_tables[g]) for s in seqs)) for g in range(len(self.groups))]
         off = {}
         cur = 0
@@ -433,9 +446,15 @@ class Executor:
             self._flush_poison()
         S = len(seqs)
         decode_only = all(len(s.tokens) == 1 for s in seqs)
-        if (self.config.use_cuda_graph and self.model.graph_safe and decode_only and S <= GRAPH_BUCKETS[-1]
-                and all(len(s.want) == 1 for s in seqs)):
-            return self._step_graph(seqs)
+        if self.config.use_cuda_graph and self.model.graph_safe and S <= GRAPH_BUCKETS[-1]:
+            if decode_only and all(len(s.want) == 1 for s in seqs):
+                return self._step_graph(seqs)
+            # prompt portions, alone or beside decoded tokens: short ones are bound by the host's
+            # launches, so they are replayed from a graph of their size class too
+            n_tokens = sum(len(s.tokens) for s in seqs)
+            if (n_tokens <= min(self.config.prompt_graph_max_tokens, TOKEN_BUCKETS[-1])
+                    and all(len(s.want) <= 1 for s in seqs)):
+                return self._step_mixed_graph(seqs, n_tokens)
         arr, off, facts = self._fill(seqs)
         meta = self._upload(arr)
         ctx = self._context(meta, off, facts, seqs)
@@ -475,6 +494,34 @@ class Executor:
         self._upload(arr, dst=meta)
         graph.replay()
         return logits[:S]
+
+    def _step_mixed_graph(self, seqs: Sequence[SeqStep], n_tokens: int) -> torch.Tensor:
+        """A step with prompt portions from the graph of its size class: tokens and sequences are
+        padded with inert rows up to the class's sizes, the kernels' grids are those of the worst
+        cut the class holds. A class is recorded at its first use."""
+        S = len(seqs)
+        Sp = next(b for b in GRAPH_BUCKETS if b >= S)
+        Np = next(b for b in TOKEN_BUCKETS if b >= n_tokens)
+        M = sum(len(s.want) for s in seqs)
+        Mp = Sp if M else 0                      # no wanted row: the graph ends in front of the head
+        longest = max(s.start + len(s.tokens) for s in seqs)
+        cap = 1024
+        while cap < longest:
+            cap *= 2
+        cap = min(cap, max(self.config.max_model_len, 1))
+        widths = [self.max_pages_per_seq] * len(self.groups)
+        arr, off, facts = self._fill(seqs, pad_to=Sp, pad_tokens=Np, pad_rows=Mp, bt_widths=widths)
+        key = (Np, Sp, Mp, cap)
+        entry = self._mixed_graphs.pop(key, None)
+        if entry is None:
+            entry = self._capture(Sp, cap, arr, off, facts, seqs, mixed_key=key)
+            while len(self._mixed_graphs) >= MIXED_GRAPHS_KEPT:
+                self._mixed_graphs.pop(next(iter(self._mixed_graphs)))
+        self._mixed_graphs[key] = entry              # (the newest at the end)
+        graph, ctx, meta, logits = entry
+        self._upload(arr, dst=meta)
+        graph.replay()
+        return logits[:M]
 
     # ------------------------------------------------------------------------------------
     # a decode step run several times in a row on the device
@@ -607,11 +654,12 @@ class Executor:
         self._repeat_graphs[key] = entry
         return entry
 
-    def _padding_step(self, bucket: int) -> StepContext:
-        """A context of ``bucket`` padding rows: every kernel runs, none touches the cache."""
+    def _padding_step(self, bucket: int, tokens: Optional[int] = None) -> StepContext:
+        """A context of ``bucket`` padding sequences and ``tokens`` padding rows (``bucket`` if not
+        given): every kernel runs, none touches the cache."""
         widths = [self.max_pages_per_seq] * len(self.groups)
         dummy = [SeqStep(tokens=[0], start=0, block_tables=[[0]] * len(self.groups), state_slot=0, want=[0])]
-        arr, off, facts = self._fill(dummy, pad_to=bucket, bt_widths=widths)
+        arr, off, facts = self._fill(dummy, pad_to=bucket, pad_tokens=tokens, bt_widths=widths)
         o, size = off["token_seq"]
         arr[o:o + size] = -1
         o, size = off["logit_rows"]
@@ -623,8 +671,9 @@ class Executor:
         return self._context(meta, off, facts, dummy)
 
     def _prepare_graph_workspace(self) -> None:
-        """One scratch area for all graphs, sized by a step of padding rows at the largest batch the
-        graphs serve; should a later graph need a larger buffer, the old one stays alive for the
+        """One scratch area for all graphs, sized by steps of padding rows at the largest sizes the
+        graphs serve (a decode step of the largest batch, a step with prompt portions of the largest
+        size class); should a later graph need a larger buffer, the old one stays alive for the
         graphs that hold it."""
         if self._graph_workspace is not None:
             return
@@ -637,6 +686,14 @@ class Executor:
             pad_ctx = self._padding_step(largest)
             pad_ctx.attention_plan.max_context_len = self.config.max_model_len
             self.model.forward(pad_ctx)
+            most = min(self.config.prompt_graph_max_tokens, self.config.max_num_batched_tokens, TOKEN_BUCKETS[-1])
+            if most > largest:
+                tokens = next(b for b in TOKEN_BUCKETS if b >= most)
+                pad_ctx = self._padding_step(largest, tokens=tokens)
+                plan = pad_ctx.attention_plan
+                plan.decode_only, plan.max_q_len, plan.q_lens, plan.bound = False, tokens, (), (tokens, largest)
+                plan.max_context_len = self.config.max_model_len
+                self.model.forward(pad_ctx)
             torch.cuda.synchronize()
         finally:
             self.rt.workspace = eager_workspace
@@ -649,6 +706,15 @@ class Executor:
         only, and must be clean then."""
         for library in (True, False):
             self.ops.library_in_graphs = library
+            if not library:
+                # the engine's own products take over shapes the library had so far: run them once
+                # outside a capture, where their kernels are loaded and their scratch may still grow
+                was_frozen, self._graph_workspace.frozen = self._graph_workspace.frozen, False
+                try:
+                    body()
+                    torch.cuda.synchronize()
+                finally:
+                    self._graph_workspace.frozen = was_frozen
             self.ops.ledger = []
             try:
                 graph = torch.cuda.CUDAGraph(keep_graph=True)
@@ -721,8 +787,15 @@ class Executor:
         o, size = off["positions"]
         arr[o:o + size] = 0
 
-    def _capture(self, bucket: int, cap: int, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep]):
-        logger.info("capturing the decode graph for %d sequences, contexts up to %d", bucket, cap)
+    def _capture(self, bucket: int, cap: int, arr: np.ndarray, off, facts, seqs: Sequence[SeqStep],
+                 mixed_key: Optional[Tuple[int, int, int, int]] = None):
+        """Records the graph of a decode step of ``bucket`` sequences, or (``mixed_key`` = (tokens,
+        sequences, logit rows, cap)) of a step with prompt portions of that size class."""
+        if mixed_key is None:
+            logger.info("capturing the decode graph for %d sequences, contexts up to %d", bucket, cap)
+        else:
+            logger.info("capturing the graph of steps of up to %d tokens of %d sequences, contexts up to %d",
+                        mixed_key[0], mixed_key[1], cap)
         eager_workspace = self.rt.workspace
         self.ops.for_graph = True
         try:
@@ -732,12 +805,19 @@ class Executor:
             self._upload(arr, dst=meta)
             ctx = self._context(meta, off, facts, seqs)
             # the graph serves every context length up to its cap
-            ctx.attention_plan.max_context_len = cap
+            plan = ctx.attention_plan
+            plan.max_context_len = cap
+            if mixed_key is not None:
+                # ... and every cut of its size class: nothing recorded may follow this step's own lengths
+                plan.decode_only, plan.max_q_len, plan.q_lens = False, mixed_key[0], ()
+                plan.bound = (mixed_key[0], mixed_key[1])
+                ctx.q_lens = ctx.starts = ctx.host_state_slots = None
             self.model.forward(ctx)                # loads every kernel before the capture
             torch.cuda.synchronize()
             self._graph_workspace.frozen = True    # the eager run above sized everything: nothing is allocated now
             result = []
-            graph = self._record(lambda: result.append(self.model.forward(ctx)), (bucket, cap))
+            graph = self._record(lambda: result.append(self.model.forward(ctx)),
+                                 (bucket, cap) if mixed_key is None else ("mixed",) + mixed_key)
             logits = result[-1]
         finally:
             self._graph_workspace.frozen = False
@@ -745,5 +825,6 @@ class Executor:
             self.ops.for_graph = False
         torch.cuda.synchronize()
         entry = (graph, ctx, meta, logits)
-        self._graphs[(bucket, cap)] = entry
+        if mixed_key is None:
+            self._graphs[(bucket, cap)] = entry
         return entry

@@ -64,10 +64,21 @@ class AttentionPlan:
     # decode steps: over how many workgroups a sequence's keys are dealt out; None lets the launch
     # rule choose (tests force counts)
     decode_splits: Optional[int] = None
+    # steps recorded into a graph that serves any cut of up to (tokens, sequences): the kernels' grids
+    # are then sized for the worst cut, not for ``q_lens`` (workgroups without work end at once)
+    bound: Optional[tuple] = None
     # for measurement: keys in the cache of the step's sequences after the step (summed), and the
     # number of (query, visible key) pairs without windows
     kv_tokens: int = 0
     attention_pairs: int = 0
+
+    def units(self, unit_tokens: int) -> int:
+        """Runs of up to ``unit_tokens`` consecutive tokens of one sequence in the step: counted from
+        the host's lengths, or the most that any cut within ``bound`` can have."""
+        if self.bound is not None:
+            tokens, seqs = self.bound
+            return tokens // unit_tokens + seqs
+        return sum(-(-ql // unit_tokens) for ql in self.q_lens)
 
 
 class StepContext:

@@ -913,7 +913,7 @@ class Ops:
         for cand in (2, 1):
             u = self.lib.dll.mv_attention_prefill_unit_tokens(group, cand)
             if u > 0:
-                units = sum(-(-ql // u) for ql in plan.q_lens)
+                units = plan.units(u)
                 if cand == 2 and units * Hkv < 2 * COMPUTE_UNITS and \
                         self.lib.dll.mv_attention_prefill_unit_tokens(group, 1) > 0:
                     continue

@@ -347,6 +347,58 @@ def test_graphs_of_many_sequences_hold_library_products_and_no_memset_node(model
     print(f"graphs of {S} sequences: {recorded['library']} library products recorded, nodes {census}")
 
 
+def test_a_graph_with_a_memset_node_is_recorded_again_without_library_products(models, monkeypatch):
+    """Should a library product leave a memset node in a graph, the graph is thrown away and recorded
+    again with the engine's own products only (after one eager run of them, outside any capture). No
+    library product has ever done so here, so the census is made to report one on the first look:
+    the second recording must hold no library product and replay to the logits of eager steps."""
+    from minivllm_amd.engine.trace import TraceRunner
+    from minivllm_amd.kernels.library import KernelLibrary
+    from minivllm_amd.kernels.ops import Ops
+    cfg, w, path = models["B"]
+    S = 70
+    toks = {f"s{i}": random_tokens(cfg, 12 + i % 5, seed=300 + i) for i in range(S)}
+    looks, in_capture = {"n": 0}, {"library": 0}
+    real_census, real_offer = Ops.graph_census, KernelLibrary.offer
+
+    def census(self, raw_graph):
+        counts = real_census(self, raw_graph)
+        looks["n"] += 1
+        if looks["n"] == 1:
+            counts = dict(counts, memset=1)
+        return counts
+
+    def offer(self, name, *args):
+        if name == "mv_gemm_lt" and torch.cuda.is_current_stream_capturing():
+            in_capture["library"] += 1
+        return real_offer(self, name, *args)
+
+    runs = {}
+    for use_graph in (False, True):
+        if use_graph:
+            monkeypatch.setattr(Ops, "graph_census", census)
+            monkeypatch.setattr(KernelLibrary, "offer", offer)
+        r = TraceRunner(path, "bfloat16", 64 * S, page_size=16, use_graph=use_graph, max_live=128)
+        r.executor.config.prompt_graph_max_tokens = 0          # the decode graph is the first one recorded
+        for rid, t in toks.items():
+            r.run_step({"step": 0, "entries": [{"id": rid, "tokens": t[:8], "want": []}], "end": []})
+        rows = []
+        for p in range(8, 11):
+            out = r.run_step({"step": p, "entries": [{"id": rid, "tokens": [t[p]], "want": [0]}
+                                                      for rid, t in toks.items()], "end": []})
+            rows.append(out.copy())
+            torch.cuda.synchronize()
+        runs[use_graph] = np.stack(rows)
+        if use_graph:
+            assert looks["n"] == 2 and r.executor.graph_census[(80, 1024)]["memset"] == 0
+            first_pass = in_capture["library"]
+            assert first_pass > 0
+        del r
+    assert rel_err(runs[True], runs[False]) <= 2e-2
+    # nothing of the library's went into the second recording (the counter saw the first pass only)
+    assert in_capture["library"] == first_pass
+
+
 def test_graphs_recorded_when_the_engine_starts(models):
     """With ``capture_graphs_at_start`` every decode graph the configuration can ask for exists before
     the first request; serving then records nothing, and gives the tokens it gives without."""

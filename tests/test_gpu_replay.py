@@ -131,6 +131,31 @@ def test_mixed(cases, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+def test_steps_with_prompt_portions_from_graphs(cases, name, dtype):
+    """Portions of changing size, and portions beside decoded tokens on recycled pages, where every
+    entry wants its last row only, as generation does: such steps are replayed from graphs recorded
+    per size class (tokens and sequences padded with inert rows, grids sized for the worst cut of
+    the class). Every returned row against the plain model, and the same rows without graphs."""
+    for case in both(cases, name):
+        prompt_lens = {rid: max(2, len(t) - 12) if len(t) > 3 else len(t) for rid, t in case.reqs.items()}
+        cuttings = {"portions": trace_tools.portions(case.reqs),
+                    "mixed": trace_tools.mixed(case.reqs, prompt_lens, max_live=4 if name != "C" else 2, seed=4)}
+        for what, steps in cuttings.items():
+            steps = trace_tools.only_last_rows(steps)
+            runner = runner_for(case, dtype, steps)
+            got = trace_tools.collect(steps, runner.run_step)
+            case.check(got, dtype, f"tiny {name} {case.kind} {what} from graphs")
+            assert len(got) == sum(len(st["entries"]) for st in steps)
+            classes = list(runner.executor._mixed_graphs)
+            assert classes and all(runner.executor.graph_census[("mixed",) + key]["memset"] == 0 for key in classes)
+            eager = trace_tools.collect(steps, runner_for(case, dtype, steps, use_graph=False).run_step)
+            worst = max(rel_err(got[k], eager[k]) for k in got)
+            assert worst <= (1e-6 if dtype == "float32" else 2e-2), f"graphs against eager steps: {worst:.3e}"
+            runner.manager.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "D128", "W64"])
 def test_mixed_with_poisoned_pages(cases, name, dtype):
     """The mixed cutting with the debugging switch that fills every page with NaN when it changes

@@ -195,3 +195,8 @@ def prompts_then_subsets(reqs: Dict[str, List[int]], prompt_lens: Dict[str, int]
                 ended.append(rid)
         steps.append({"step": len(steps), "entries": entries, "end": ended})
     return steps
+
+
+def only_last_rows(steps: List[dict]) -> List[dict]:
+    """The same steps, each entry wanting the logits of its last token only (what generation asks for)."""
+    return [dict(st, entries=[dict(e, want=[len(e["tokens"]) - 1]) for e in st["entries"]]) for st in steps]
