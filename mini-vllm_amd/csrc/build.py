@@ -29,7 +29,7 @@ ARCH = "gfx950"
 COMMON_SOURCES = ["runtime.hip", "elementwise.hip", "gemm_ref.hip", "attention_ref.hip", "sampling.hip"]
 VARIANT_SOURCES: Dict[str, List[str]] = {
     "f32": COMMON_SOURCES,
-    "bf16": COMMON_SOURCES + ["gemm_skinny.hip", "gemm_mid.hip", "gemm_lt.hip", "attention_fast.hip",
+    "bf16": COMMON_SOURCES + ["gemm_skinny.hip", "gemm_mid.hip", "gemm_tile.hip", "gemm_lt.hip", "attention_fast.hip",
                               "attention_prefill.hip"],
 }
 # libraries a variant links against

@@ -23,7 +23,7 @@ PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
 # entry point -> (pattern of the kernel names it launches, the most launches one call makes)
 KERNELS_OF: Dict[str, Tuple[str, int]] = {
-    "mv_embedding": (r"\bembedding_kernel", 1),
+    "mv_embedding": (r"\bembedding(_gather)?_kernel", 1),
     "mv_add_rmsnorm": (r"\badd_rmsnorm(_vec)?_kernel", 1),
     "mv_add_rmsnorm_split": (r"\badd_rmsnorm(_vec)?_kernel", 1),
     "mv_rmsnorm": (r"\brmsnorm_kernel", 1),
@@ -37,6 +37,7 @@ KERNELS_OF: Dict[str, Tuple[str, int]] = {
     "mv_scale_rows": (r"\bscale_rows_kernel", 1),
     "mv_gemm_ref": (r"\bgemm_nt_kernel", 1),
     "mv_gemm_mid": (r"\bgemm_mid(_reduce)?_kernel", 2),
+    "mv_gemm_tile": (r"\bgemm_(tile|mid_reduce)_kernel", 2),
     "mv_gemm_lt": (r"^((Custom_)?Cijk_|void hipblaslt|hipblaslt|.*rocblaslt)", 3),
     "mv_attention_ref": (r"\battention_ref_kernel", 1),
     "mv_attention_decode": (r"\battention_(decode(_wave)?|merge(_range)?)_kernel", 2),

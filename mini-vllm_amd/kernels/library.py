@@ -85,6 +85,16 @@ _OPTIONAL_SIGNATURES = {
     # A, lda, W, bias, C, ldc, c_dtype, M, N, K, swiglu, work, work_floats, stream
     "mv_gemm_mid": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                             c_void_p, c_long, c_void_p]),
+    "mv_gemm_tile_workspace": (c_long, [c_int, c_int, c_int, c_int, c_int]),
+    "mv_gemm_tile_splits": (c_int, [c_int, c_int, c_int, c_int, c_int]),
+    # A, lda, W, bias, C, ldc, c_dtype, M, N, K, gated, work, work_floats, force, stream
+    "mv_gemm_tile": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
+                             c_void_p, c_long, c_int, c_void_p]),
+    # A, lda, W, M, N, K, work, work_floats, force, stream
+    "mv_gemm_tile_sums": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_void_p]),
+    # A, lda, W, bias, C, ldc, c_dtype, M, N, K, gated, partial, P, eps, stream
+    "mv_gemm_tile_scaled": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int,
+                                    c_int, c_void_p, c_int, c_float, c_void_p]),
     "mv_attention_decode": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
                                     c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),

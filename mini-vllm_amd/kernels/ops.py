@@ -45,6 +45,27 @@ LIBRARY_TALL_WEIGHT = 96 * 1000 * 1000
 # weights for fewer than 16 rows (8B-sized: 44 against 46 us at 8 rows, 49 against 46 at 16); from
 # this size on the library and a separate activation kernel win at every number of rows
 LIBRARY_TALL_WEIGHT_GATED = 240 * 1000 * 1000
+# The tiled MFMA product (gemm_tile.hip) takes the steps between the weight-streaming kernels and the
+# library, where it is ahead of both (measured on MI355X, weights rotating so that they come from memory):
+# a gated pair with the activation in its epilogue from 32 rows on (0.6B sizes at 64 rows: 7.7 us
+# against the weight-streaming kernel's 11.4 and the library's 13.8 with the activation as a kernel of
+# its own; at 1,024 rows 21.6 against 24.6; level from 1,536 on), for weights of 64 MB and more up to 128
+# rows (8B sizes at 64 rows 44 against 51 us; at 256 the library is ahead); a plain product against a
+# small weight with at least 4,096 rows (enough tiles without splitting K) from 40 to 512 rows (0.6B qkv
+# at 64 rows 6.8 against 7.8 us, at 256 rows 7.2 against the library's 9.0; weights with fewer rows go to
+# the library, which is a tenth ahead there); any plain product against a weight of 16 MB and more from
+# 33 to 256 rows (8B sizes at 128 rows: down 33 against the library's 67 us, o 16 against 23, qkv 22 against 25).
+TILE_MIN_WEIGHT = 4 * 1024 * 1024             # bytes: smaller weights were not measured and stay where they were
+TILE_GATED_MIN_M = 32
+TILE_GATED_MAX_M = 1536
+TILE_GATED_BIG_WEIGHT = 64 * 1024 * 1024      # bytes
+TILE_GATED_BIG_MAX_M = 128
+TILE_SMALL_MIN_M = 40
+TILE_SMALL_MAX_M = 512
+TILE_SMALL_MIN_N = 4096
+TILE_BIG_WEIGHT = 16 * 1024 * 1024            # bytes
+TILE_BIG_MIN_M = 33
+TILE_BIG_MAX_M = 256
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
@@ -167,6 +188,7 @@ class Ops:
         self._lt_work: Optional[torch.Tensor] = None        # the library's workspace
         self._split_pending: Optional[SplitSum] = None     # partial sums in the work area nobody has used yet
         self._mid_retired: list = []
+        self._tile_work: Optional[torch.Tensor] = None     # partial sums of the tiled product when it splits K
         self._sample_work: Optional[torch.Tensor] = None
         self._attn_counters: Optional[torch.Tensor] = None
         # measurement: with a list here, every launch leaves (entry point, bytes it has to move,
@@ -452,6 +474,13 @@ class Ops:
                 and self._library_allowed(M, N, K, bias is not None, out.dtype)
                 and self._library_product(a, w, bias, out)):
             return None
+        if fast and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.wants_tile(M, N, K):
+            if defer_sum and out.dtype == self.dtype and out.is_contiguous():
+                pending = self._gemm_tile_sums(a, lda, w, bias, out, M, N, K)
+                if pending is not None:
+                    return pending
+            if self.gemm_tile(a, w, out, bias):
+                return None
         if fast and K % 32 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.lib.has("mv_gemm_skinny"):
             done = self._gemm_mid(a, lda, w, bias, out, ldc, M, N, K, swiglu=False,
                                   defer_sum=defer_sum and out.dtype == self.dtype and out.is_contiguous())
@@ -580,6 +609,85 @@ class Ops:
                       self._stream())
         return True
 
+    def wants_tile(self, M: int, N: int, K: int, gated: bool = False) -> bool:
+        """Whether M rows against an [N, K] weight (``gated``: the packed gate/up pair) go to the tiled
+        product (see TILE_GATED_MIN_M)."""
+        if not (self.use_fast_kernels and self.lib.has("mv_gemm_tile")) or K % 64 or M * N >= 1 << 31:
+            return False
+        weight_bytes = 2 * N * K
+        if weight_bytes < TILE_MIN_WEIGHT:
+            return False
+        if gated:
+            # (the largest pairs, 32B-sized ones, stream faster through the library at any number of rows)
+            if N % 2 or M < TILE_GATED_MIN_M or N * K >= LIBRARY_TALL_WEIGHT_GATED:
+                return False
+            return M <= (TILE_GATED_MAX_M if weight_bytes < TILE_GATED_BIG_WEIGHT else TILE_GATED_BIG_MAX_M)
+        if self.prefers_library(M, N, K):
+            return False
+        if weight_bytes >= TILE_BIG_WEIGHT:
+            return TILE_BIG_MIN_M <= M <= TILE_BIG_MAX_M
+        return N >= TILE_SMALL_MIN_N and TILE_SMALL_MIN_M <= M <= TILE_SMALL_MAX_M
+
+    def _gemm_tile_sums(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                        M: int, N: int, K: int):
+        """The tiled product of a shape whose K is split, left as partial sums (``SplitSum``) for the
+        residual add + norm behind it; None when the shape is not split or the sums cannot be kept."""
+        splits = int(self.lib.dll.mv_gemm_tile_splits(M, N, K, 0, 0))
+        if splits <= 1 or not self.lib.has("mv_add_rmsnorm_split"):
+            return None
+        need = splits * M * N
+        if self._mid_work is None or self._mid_work.numel() < need:
+            if torch.cuda.is_current_stream_capturing():
+                return None                                    # no allocation inside a capture
+            if self._split_pending is not None:
+                self._split_pending.materialize()
+            if self._mid_work is not None:
+                self._mid_retired.append(self._mid_work)       # captured graphs may hold its address
+            self._mid_work = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=a.device)
+        if self._split_pending is not None:
+            self._split_pending.materialize()                  # its sums are about to be overwritten
+        self._note("mv_gemm_tile", self._size(a, w) + 4 * M * N * splits, 2 * M * N * K)
+        self.lib.call("mv_gemm_tile_sums", a.data_ptr(), lda, w.data_ptr(), M, N, K, self._mid_work.data_ptr(),
+                      self._mid_work.numel(), 0, self._stream())
+        pending = SplitSum(self, out, self._mid_work, splits, bias)
+        self._split_pending = pending
+        return pending
+
+    def gemm_tile(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                  gated: bool = False, force: int = 0) -> bool:
+        """out[M, N] = a @ w^T (+ bias), or with ``gated`` out[M, N / 2] = silu(a Wg^T) * (a Wu^T), by the
+        engine's tiled MFMA product for many rows. False, with nothing done, when the shape is not taken.
+        ``force`` fixes the tile and the split of K (measurements)."""
+        if not (self.use_fast_kernels and self.lib.has("mv_gemm_tile")):
+            return False
+        M, K = a.shape
+        N = w.shape[0]
+        n_out = N // 2 if gated else N
+        if (M == 0 or K % 64 or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not w.is_contiguous()
+                or w.shape[1] != K or a.stride(1) != 1 or (M > 1 and a.stride(0) % 8) or a.data_ptr() % 16
+                or w.data_ptr() % 16 or out.shape != (M, n_out) or out.stride(1) != 1
+                or out.dtype not in (torch.bfloat16, torch.float32) or (gated and (N % 2 or bias is not None))
+                or (bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N))
+                or M * N >= 1 << 31):
+            return False
+        need = int(self.lib.dll.mv_gemm_tile_workspace(M, N, K, int(gated), force))
+        if need < 0:
+            return False
+        work = None
+        if need > 0:
+            if self._tile_work is None or self._tile_work.numel() < need:
+                if torch.cuda.is_current_stream_capturing():
+                    return False                               # no allocation inside a capture
+                if self._tile_work is not None:
+                    self._mid_retired.append(self._tile_work)  # captured graphs may hold its address
+                self._tile_work = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=a.device)
+            work = self._tile_work
+        self._note("mv_gemm_tile", self._size(a, w, out) + 8 * need, 2 * M * N * K)
+        self.lib.call("mv_gemm_tile", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias), out.data_ptr(),
+                      out.stride(0) if M > 1 else n_out, _CODES[out.dtype], M, N, K, int(gated), _ptr(work),
+                      0 if work is None else work.numel(), force, self._stream())
+        return True
+
     @staticmethod
     def wants_mid(M: int, N: int, K: int) -> bool:
         """Whether a product of M rows with an [N, K] weight goes to the kernel that splits K (it takes
@@ -639,6 +747,14 @@ class Ops:
             return False
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N):
             return False
+        if (self.wants_tile(M, w.shape[0], K, gated=swiglu) and self.lib.has("mv_gemm_tile_scaled") and w.data_ptr() % 16 == 0
+                and int(self.lib.dll.mv_gemm_tile_splits(M, w.shape[0], K, int(swiglu), 0)) == 1):
+            rows.take()
+            self._note("mv_gemm_tile", self._size(a, w, out) + M * rows.P * 4, 2 * M * w.shape[0] * K)
+            self.lib.call("mv_gemm_tile_scaled", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias),
+                          out.data_ptr(), out.stride(0) if M > 1 else N, _CODES[out.dtype], M, w.shape[0], K, int(swiglu),
+                          rows.partial.data_ptr(), rows.P, rows.eps, self._stream())
+            return True
         rows.take()
         self._note("mv_gemm_skinny_scaled", self._size(a, w, out) + M * rows.P * 4, 2 * M * w.shape[0] * K)
         self.lib.call("mv_gemm_skinny_scaled", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), _ptr(bias),
@@ -713,6 +829,8 @@ class Ops:
             return False
         M, K = a.shape
         two_i = w_gate_up.shape[0]
+        if self.wants_tile(M, two_i, K, gated=True) and self.gemm_tile(a, w_gate_up, out, None, gated=True):
+            return True
         if self.prefers_library(M, two_i, K, gated=True) and self._library_allowed(M, two_i, K, False):
             return False
         # with the library's product at hand, more rows than one workgroup takes go there

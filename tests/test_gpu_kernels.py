@@ -726,13 +726,13 @@ def test_gemm_weight_streaming(out_dtype, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,swiglu,out_dtype", [
-    (17, 3100, 4096, False, torch.bfloat16), (64, 4096, 3072, False, torch.bfloat16),
-    (40, 6144, 2048, False, torch.float32), (64, 6144, 2048, True, torch.bfloat16),
-    (33, 2 * 1571, 4096, True, torch.bfloat16), (20, 151936 // 4, 1024, False, torch.float32),
+    (17, 3100, 4096, False, torch.bfloat16), (32, 4096, 3072, False, torch.bfloat16),
+    (30, 6144, 2048, False, torch.float32), (31, 6144, 2048, True, torch.bfloat16),
+    (25, 2 * 1571, 4096, True, torch.bfloat16), (20, 151936 // 4, 1024, False, torch.float32),
     (9, 3100, 4096, False, torch.bfloat16), (1, 5120, 25600, False, torch.bfloat16),
     (3, 2 * 12032, 5120, True, torch.bfloat16)])
 def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dtype):
-    """9 to 64 rows against a weight of tens of megabytes, any number of rows up to 64 against one
+    """9 to 32 rows against a weight of tens of megabytes, any number of rows up to 64 against one
     of hundreds: the kernel that shares the activation rows through LDS and splits K over
     workgroups (partial sums added in a fixed order)."""
     ops = ops_for(torch.bfloat16)
@@ -797,7 +797,7 @@ def test_gemm_weight_streaming_many_rows(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,with_bias,out_dtype", [
-    (97, 1024, 2048, True, torch.bfloat16), (65, 4096, 4096, False, torch.bfloat16), (200, 336, 1024, False, torch.bfloat16),
+    (97, 1024, 2048, True, torch.bfloat16), (300, 4096, 4096, False, torch.bfloat16), (200, 336, 1024, False, torch.bfloat16),
     (2048, 6144, 1024, False, torch.bfloat16), (300, 4096, 12288, True, torch.bfloat16),
     (2048, 51200, 5120, False, torch.bfloat16), (128, 151936, 1024, False, torch.float32),
     (1, 151936, 1024, False, torch.float32), (8, 151936, 1024, False, torch.float32), (40, 151936, 1024, True, torch.float32),
@@ -828,6 +828,107 @@ def test_gemm_through_the_library(M, N, K, with_bias, out_dtype):
     tol = OP_TOL[torch.bfloat16] if out_dtype == torch.bfloat16 else 3e-6
     assert rel_err(out[:, cols].float().cpu().numpy(), want.cpu().numpy()) <= tol
     assert bool(torch.isfinite(out.float()).all())
+
+
+TILE_SHAPES = {"auto": 0, "128x128": 40401, "128x128 deep": 140401, "64x128": 20401, "128x64": 40201, "64x64": 20201,
+               "64x64 K/3": 20203, "128x128 K/2": 40402, "64x128 K/4": 20404}
+
+
+@pytest.mark.parametrize("M,N,K,gated,out_dtype,with_bias", [
+    (65, 4096, 1024, False, torch.bfloat16, True), (200, 333, 1024, False, torch.float32, True),
+    (130, 2 * 1571, 4096, True, torch.bfloat16, False), (33, 1024, 3072, False, torch.bfloat16, False),
+    (256, 6144, 1024, True, torch.bfloat16, False), (1000, 520, 192, False, torch.bfloat16, True),
+    (40, 2 * 96, 64, True, torch.float32, False), (513, 136, 512, False, torch.float32, False)])
+@pytest.mark.parametrize("shape", list(TILE_SHAPES))
+def test_gemm_tiled(M, N, K, gated, out_dtype, with_bias, shape):
+    """The tiled product for many rows at every tile it has (rows and columns that are no multiple
+    of a tile, a K of one to 64 chunks, split or not), plain and as a gated pair with the activation
+    in its epilogue, against float64; rows in a wider buffer give the same bits."""
+    if gated and shape == "128x64":
+        pytest.skip("a gated pair has no 128 x 64 tile")
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(31)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = ((2 if gated else 1) * torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
+    full = a.double() @ w.double().T
+    if gated:
+        want = torch.nn.functional.silu(full[:, :N // 2]) * full[:, N // 2:]
+    else:
+        want = full + b.double() if with_bias else full
+    n_out = N // 2 if gated else N
+    out = torch.full((M, n_out), float("nan"), dtype=out_dtype, device="cuda")
+    assert ops.gemm_tile(dev(a), dev(w), out, dev(b) if with_bias else None, gated, TILE_SHAPES[shape])
+    tol = 3e-6 if out_dtype == torch.float32 else OP_TOL[torch.bfloat16]
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= tol
+    wide = torch.zeros(M, K + 40, dtype=torch.bfloat16)
+    wide[:, :K] = a
+    out_w = torch.full((M, n_out + 12), float("nan"), dtype=out_dtype, device="cuda")[:, :n_out]
+    assert ops.gemm_tile(dev(wide)[:, :K], dev(w), out_w, dev(b) if with_bias else None, gated, TILE_SHAPES[shape])
+    assert torch.equal(out_w, out)
+
+
+@pytest.mark.parametrize("M,N,K,gated,with_bias", [(64, 4096, 1024, False, True), (96, 6144, 1024, True, False),
+                                                   (40, 4100, 512, False, False), (33, 2 * 1571, 1024, True, False)])
+# (each of these weights has at least 4 MB: smaller ones stay with the weight-streaming kernel)
+def test_gemm_tiled_behind_a_folded_norm(M, N, K, gated, with_bias):
+    """Rows that the product in front left weighted but not divided by their root mean square: the
+    tiled product divides its output rows (before the bias, before the gate)."""
+    from minivllm_amd.kernels.ops import WeightedRows
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(37)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = ((2 if gated else 1) * torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
+    P, eps = 7, 1e-5
+    partial = torch.rand(M, P, generator=g) * K / P * 1.7
+    rinv = torch.rsqrt(partial.double().sum(1, keepdim=True) / K + eps)
+    full = (a.double() @ w.double().T) * rinv
+    want = torch.nn.functional.silu(full[:, :N // 2]) * full[:, N // 2:] if gated else (full + b.double() if with_bias else full)
+
+    class Fold:
+        norm = None
+    fold = Fold()
+    fold.weighted, fold.partial, fold.eps, fold.normed = dev(a), dev(partial.float().contiguous()), eps, None
+    rows = WeightedRows(ops, fold, P)
+    n_out = N // 2 if gated else N
+    out = torch.full((M, n_out), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.ledger = []
+    try:
+        if gated:
+            assert ops.gemm_swiglu(rows, dev(w), out)
+        else:
+            ops.gemm(rows, dev(w), out, dev(b) if with_bias else None)
+        assert [line[0] for line in ops.ledger] == ["mv_gemm_tile"], ops.ledger
+    finally:
+        ops.ledger = None
+    assert rows.used
+    assert rel_err(out.float().cpu().numpy(), want.numpy()) <= OP_TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("M,N,K,gated,kernel", [
+    (64, 4096, 1024, False, "mv_gemm_tile"), (300, 4096, 1024, False, "mv_gemm_tile"), (600, 4096, 1024, False, "mv_gemm_lt"),
+    (32, 4096, 1024, False, "mv_gemm_skinny"), (100, 1024, 2048, False, "mv_gemm_lt"), (64, 4096, 4096, False, "mv_gemm_tile"),
+    (200, 4096, 12288, False, "mv_gemm_tile"), (32, 4096, 4096, False, "mv_gemm_mid"), (40, 6144, 1024, True, "mv_gemm_tile"),
+    (1024, 6144, 1024, True, "mv_gemm_tile"), (24, 6144, 1024, True, "mv_gemm_skinny_swiglu"),
+    (40, 1024, 256, True, "mv_gemm_skinny_swiglu"),
+    (100, 24576, 4096, True, "mv_gemm_tile"), (200, 24576, 4096, True, None)])
+def test_which_product_takes_which_rows(M, N, K, gated, kernel):
+    """Between the weight-streaming kernels (few rows) and the library (many), the tiled product."""
+    ops = ops_for(torch.bfloat16)
+    a = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    out = torch.empty(M, N // 2 if gated else N, dtype=torch.bfloat16, device="cuda")
+    ops.ledger = []
+    try:
+        if gated:
+            assert ops.gemm_swiglu(a, w, out) == (kernel is not None)
+        else:
+            ops.gemm(a, w, out)
+        seen = [line[0] for line in ops.ledger]
+    finally:
+        ops.ledger = None
+    assert seen == ([kernel] if kernel else []), seen
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 3072, 1024), (40, 100, 96), (64, 560, 256)])
@@ -1185,12 +1286,22 @@ def test_partial_sums_of_a_product_go_straight_into_the_norm(M, N, K, with_bias,
 
 
 def test_kernels_that_load_straight_into_lds_repeat_their_results():
-    """The K-splitting product and the prompt attention bring operands into LDS with loads whose
-    completion they wait for by count. A wait that came too early would show as results that differ
-    from call to call; here many calls in a row give the same bits."""
+    """The K-splitting product, the tiled product and the prompt attention bring operands into LDS with
+    loads whose completion they wait for by count. A wait that came too early would show as results
+    that differ from call to call; here many calls in a row give the same bits."""
     ops = ops_for(torch.bfloat16)
     g = torch.Generator().manual_seed(31)
-    for M, N, K in ((64, 4096, 4096), (9, 3100, 8192), (33, 12288, 2048)):
+    for M, N, K, gated in ((64, 4096, 4096, False), (200, 4096, 1024, False), (96, 6144, 1024, True), (256, 4096, 12288, False),
+                           (1024, 6144, 1024, True)):
+        a = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
+        w = dev((torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16))
+        first = torch.empty(M, N // 2 if gated else N, dtype=torch.bfloat16, device="cuda")
+        assert ops.wants_tile(M, N, K, gated) and ops.gemm_tile(a, w, first, None, gated)
+        for _ in range(30):
+            again = torch.empty_like(first)
+            assert ops.gemm_tile(a, w, again, None, gated)
+            assert torch.equal(first, again)
+    for M, N, K in ((32, 4096, 4096), (9, 3100, 8192), (30, 12288, 2048)):
         a = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
         w = dev((torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16))
         ops._mid_work = None
