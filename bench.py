@@ -260,11 +260,15 @@ def emit_kernels(llm, cfg, args) -> int:
             print()
         sp = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
         llm.submit(random_prompt(vocab, args.prefill_tokens, args.seed + 100), sp)
+        before = set(ex.graph_ledger)
         ex.ops.ledger = []
         try:
             while llm.has_unfinished():
                 llm.step()
-            ledger = roofline.launches(ex.ops.ledger)
+            # a prompt step that is replayed from a graph leaves its launches with the graph it recorded
+            recorded = [k for k in ex.graph_ledger if k not in before and k and k[0] == "mixed"]
+            lines = ex.graph_ledger[recorded[-1]] if recorded else ex.ops.ledger
+            ledger = roofline.launches(lines)
         finally:
             ex.ops.ledger = None
         title = f"prefill of one {args.prefill_tokens}-token prompt, qwen3-{args.shape} shape"

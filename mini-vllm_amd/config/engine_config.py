@@ -32,7 +32,9 @@ def compute_dtype_name(engine_dtype: Optional[str], model_dtype: Optional[str], 
     name = engine_dtype or model_dtype or "bfloat16"
     if name not in COMPUTE_DTYPES:
         raise ConfigError(f"{where}: the model names the dtype {name!r}; the engine computes in bfloat16 or float32 "
-                          f"and picks neither silently: state dtype='bfloat16' or dtype='float32' (--dtype)")
+                          f"and picks neither silently: state dtype='bfloat16' or dtype='float32' (--dtype). Tensors "
+                          f"stored in {name} are not converted on the way in either: a {name} checkpoint has to be "
+                          f"saved again in bfloat16 or float32 before it can be served")
     return name
 
 
@@ -57,7 +59,9 @@ class EngineConfig:
     eos_token_ids: Optional[Tuple[int, ...]] = None
 
     # ---- cache -------------------------------------------------------------------------
-    kv_cache_num_blocks: Optional[int] = None
+    # pages of the cache pools: None sizes them from the memory left; a number gives every cache group
+    # that many; a sequence names one count per group (a group that gives pages back early needs fewer)
+    kv_cache_num_blocks: Optional[object] = None
     kv_cache_block_size: int = 16
     gpu_memory_utilization: float = 0.5
     enable_prefix_caching: bool = False
@@ -106,8 +110,11 @@ class EngineConfig:
             raise ValueError(f"prefill_chunk must be >= 1, got {self.prefill_chunk}")
         if self.kv_cache_block_size < 1:
             raise ValueError(f"kv_cache_block_size must be >= 1, got {self.kv_cache_block_size}")
-        if self.kv_cache_num_blocks is not None and self.kv_cache_num_blocks < 1:
-            raise ValueError(f"kv_cache_num_blocks must be >= 1, got {self.kv_cache_num_blocks}")
+        if self.kv_cache_num_blocks is not None:
+            counts = [self.kv_cache_num_blocks] if isinstance(self.kv_cache_num_blocks, int) else list(self.kv_cache_num_blocks)
+            if not counts or any(not isinstance(n, int) or n < 1 for n in counts):
+                raise ValueError(f"kv_cache_num_blocks must be >= 1 (one count, or one per cache group), "
+                                 f"got {self.kv_cache_num_blocks}")
         if not (0.0 < self.gpu_memory_utilization <= 1.0):
             raise ValueError(f"gpu_memory_utilization must be in (0, 1], got {self.gpu_memory_utilization}")
         if self.eos_token_ids is not None:

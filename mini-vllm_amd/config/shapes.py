@@ -21,6 +21,20 @@ QWEN3_SHAPES: Dict[str, Dict[str, Any]] = {
 }
 
 
+def named_shapes() -> Dict[str, Dict[str, Any]]:
+    """Every named shape as a raw config.json dictionary, ``architectures`` included: the registry
+    picks the architecture from it, as it does for a model folder. Another architecture's shapes are
+    added here."""
+    return {name: qwen3_shape(name) for name in QWEN3_SHAPES}
+
+
+def named_shape(name: str, **overrides) -> Dict[str, Any]:
+    shapes = named_shapes()
+    if name not in shapes:
+        raise KeyError(f"unknown shape {name!r} (known: {sorted(shapes)})")
+    return dict(shapes[name], **overrides)
+
+
 def qwen3_shape(name: str, **overrides) -> Dict[str, Any]:
     """The raw config dictionary of a named shape (``architectures`` and a position limit included)."""
     if name not in QWEN3_SHAPES:

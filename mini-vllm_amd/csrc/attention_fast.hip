@@ -683,7 +683,7 @@ static int decode_common(bool fused, const FusedInput& fz, const void* q, long q
     // 256 registers a lane, which costs it three spilled ones at head size 128): one's set-up and
     // tail overlap the other's stream of keys, 4-6 % on a step of 64 to 256 sequences. A grid that
     // fits the chip at once keeps all registers.
-    const int occ = ((long)n_seqs * Hkv > 256 && nsplit == 1) ? 2 : 1;
+    const int occ = ((long)n_seqs * Hkv > mv_compute_units() && nsplit == 1) ? 2 : 1;
 #define AF_LAUNCH(DD, WW, FF)                                                                                     \
     do {                                                                                                          \
         if constexpr (WW == 4) {                                                                                  \

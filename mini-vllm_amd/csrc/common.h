@@ -159,6 +159,7 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 extern "C" const char* mv_last_error();
 int mv_fail(const char* fmt, ...);
 int mv_check_launch(const char* what);
+int mv_compute_units();     // of the current device (runtime.hip)
 
 #define MV_REQUIRE(cond, ...)                      \
     do {                                           \

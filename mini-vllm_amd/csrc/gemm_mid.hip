@@ -30,7 +30,7 @@ union Frag {
 #define GM_KC 128          // columns of a chunk
 #endif
 #define GM_KS (GM_KC / 32)  // MFMA steps of a chunk
-#define GM_COMPUTE_UNITS 256
+#define GM_COMPUTE_UNITS mv_compute_units()
 
 #define GM_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 15) | (((N) >> 4) << 14))
 

@@ -33,7 +33,7 @@ union Frag {
 
 #define SK_MAX_WAVES 8
 #define SK_MAX_ROWS 512      // up to 64 rows per workgroup, more rows are dealt out to groups of workgroups
-#define SK_COMPUTE_UNITS 256
+#define SK_COMPUTE_UNITS mv_compute_units()
 #ifndef SK_STAGE_FRAGS
 #define SK_STAGE_FRAGS 8    // 16-byte operand loads per lane in one register stage of the main loop
 #endif

@@ -312,7 +312,7 @@ struct TilePlan {
     int tiles_m, tiles_n;
 };
 
-#define GT_COMPUTE_UNITS 256
+#define GT_COMPUTE_UNITS mv_compute_units()
 
 // The tile and the number of splits of K, by rules read off measurements on MI355X (weights of 4 MB to
 // 500 MB, 33 to 2,048 rows). Weights below 16 MB: the largest tile no taller than the rows need that

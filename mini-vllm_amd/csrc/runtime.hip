@@ -35,6 +35,27 @@ extern "C" int mv_built_dtypes() {
 
 extern "C" int mv_abi_version() { return 1; }
 
+// Compute units of the current device, asked once (the launch rules size their grids in rounds of
+// one workgroup a compute unit); 256 if the device does not say. MV_COMPUTE_UNITS overrides it,
+// for a process that is confined to part of the chip.
+int mv_compute_units() {
+    static int units = 0;
+    if (units > 0) return units;
+    int n = 0;
+    const char* env = getenv("MV_COMPUTE_UNITS");
+    if (env != nullptr) n = atoi(env);
+    if (n <= 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+    }
+    units = n > 0 ? n : 256;
+    return units;
+}
+
+extern "C" int mv_device_compute_units() { return mv_compute_units(); }
+
 // A kernel that does nothing: a graph of these, each depending on the one before, shows what a
 // dependent launch costs on the device whatever it computes (the floor of a decode step that is a
 // chain of small kernels).

@@ -26,7 +26,7 @@ import torch
 
 from ..cache.manager import CacheManager, GroupSpec, groups_from_needs
 from ..config.engine_config import EngineConfig, compute_dtype_name
-from ..kernels.ops import dtype_from_name, get_ops
+from ..kernels.ops import Ops, dtype_from_name
 from ..models.causal_lm import CausalLM, expected_tensors
 from ..models.registry import Architecture, load_config
 from ..parts.base import Runtime, Workspace
@@ -126,7 +126,10 @@ class Executor:
                 logger.warning("%d matrices of %s are stored in 32-bit and stay so: products with them run on the "
                                "exact kernel, not on the MFMA kernels (first: %s); store the model in bfloat16 for "
                                "serving speed", len(wide), where, wide[0])
-        self.ops = get_ops(self.dtype)
+        # an engine has its kernels' front end to itself: what it keeps between launches (scratch areas,
+        # the counters of the decode attention's key splits, the state of a recording) is then never
+        # shared with another engine of the process
+        self.ops = Ops(self.dtype)
         self.rt = Runtime(device=self.device, dtype=self.dtype, ops=self.ops, workspace=Workspace(self.device),
                           max_positions=config.max_model_len)
         tensors = DeviceTensors(source, self.device)
@@ -165,15 +168,47 @@ class Executor:
         self.kv_pages: Dict[int, Dict[str, torch.Tensor]] = {}     # per call with a cache need: its page tensors by name
         self._poison: Dict[int, List[int]] = {}                    # debug_poison_pages: pages to fill, per group
         self.state_tensors: Dict[int, torch.Tensor] = {}
-        self.num_pages = 0
+        self.num_pages = 0                                         # of the largest pool
+        self.group_pages: List[int] = [0] * len(self.groups)       # pages of each group's pool
         self._allocate_memory()
 
     # ------------------------------------------------------------------------------------
     # memory
     # ------------------------------------------------------------------------------------
-    def bytes_per_page(self) -> int:
-        item = torch.empty((), dtype=self.dtype).element_size()
-        return sum(n.bytes_per_token(item) for n in self.needs if n is not None) * self.page_size
+    def bytes_per_page(self, group: Optional[int] = None) -> int:
+        """Bytes one page index takes over all calls (of one group, or of all groups together)."""
+        calls = range(len(self.needs)) if group is None else self.groups[group].calls
+        return sum(self.needs[c].bytes_per_token(self.dtype) for c in calls if self.needs[c] is not None) * self.page_size
+
+    def _pages_a_request_holds(self, group: int) -> int:
+        """Most pages one request can hold in a group at a time (see Retention.most_pages_held)."""
+        portion = min(self.config.max_num_batched_tokens, self.config.max_model_len)
+        held = self.groups[group].retention.most_pages_held(self.config.max_model_len, self.page_size, portion)
+        return self.max_pages_per_seq if held is None else max(1, min(int(held), self.max_pages_per_seq))
+
+    def _pool_sizes(self, budget_bytes: int) -> List[int]:
+        """Pages per group within ``budget_bytes``: every pool as large as the largest, except that a
+        group never gets more pages than all live requests together can hold in it (a group that
+        gives pages back early is bounded by that long before the memory is)."""
+        n_groups = len(self.groups)
+        caps = [self.config.max_num_batched_seqs * self._pages_a_request_holds(g) for g in range(n_groups)]
+        per = [max(1, self.bytes_per_page(g)) for g in range(n_groups)]
+        sizes: List[Optional[int]] = [None] * n_groups
+        left = budget_bytes
+        while True:
+            open_groups = [g for g in range(n_groups) if sizes[g] is None]
+            if not open_groups:
+                break
+            common = left // sum(per[g] for g in open_groups)
+            capped = [g for g in open_groups if caps[g] <= common]
+            if not capped:
+                for g in open_groups:
+                    sizes[g] = int(common)
+                break
+            for g in capped:
+                sizes[g] = caps[g]
+                left -= caps[g] * per[g]
+        return [int(n) for n in sizes]
 
     def _allocate_memory(self) -> None:
         cfg = self.config
@@ -183,35 +218,42 @@ class Executor:
                 self.state_tensors[call] = torch.zeros((self.num_state_slots,) + tuple(dims), dtype=dt,
                                                        device=self.device)
         if cfg.kv_cache_num_blocks is not None:
-            num_pages = cfg.kv_cache_num_blocks
+            given = cfg.kv_cache_num_blocks
+            sizes = [int(given)] * len(self.groups) if isinstance(given, int) else [int(n) for n in given]
+            if len(sizes) != len(self.groups):
+                raise ValueError(f"kv_cache_num_blocks names {len(sizes)} pools, the model has {len(self.groups)} cache groups")
         else:
             self._warmup(cfg.max_num_batched_tokens)
             torch.cuda.synchronize()
             free, total = torch.cuda.mem_get_info(self.device)
             used = total - free
-            per_page = max(1, self.bytes_per_page())
             budget = int(total * cfg.gpu_memory_utilization) - used
-            num_pages = budget // per_page
-            if num_pages < 1:
+            sizes = self._pool_sizes(budget) if self.groups else []
+            if sizes and min(sizes) < 1:
                 raise RuntimeError(f"no memory left for the cache: {used / 2**30:.1f} GiB are in use, "
                                    f"gpu_memory_utilization {cfg.gpu_memory_utilization} of "
                                    f"{total / 2**30:.1f} GiB allows {budget / 2**30:.2f} GiB more")
-            # never more than every request at full length can use
-            num_pages = min(num_pages, cfg.max_num_batched_seqs * self.max_pages_per_seq)
-        self._allocate_pages(num_pages)
-        logger.info("allocated %d cache pages of %d tokens (%.2f GiB)", num_pages, self.page_size,
-                    num_pages * self.bytes_per_page() / 2 ** 30)
+        self._allocate_pages(sizes)
+        logger.info("allocated cache pools of %s pages of %d tokens (%.2f GiB)", sizes, self.page_size,
+                    sum(n * self.bytes_per_page(g) for g, n in enumerate(sizes)) / 2 ** 30)
         if cfg.capture_graphs_at_start and cfg.use_cuda_graph and self.model.graph_safe:
             self.capture_graphs()
 
-    def _allocate_pages(self, num_pages: int) -> None:
+    def _allocate_pages(self, sizes) -> None:
+        """Page tensors ``[pages, *shape]`` for every call with a cache need, in the element types the
+        need names, as many pages as the call's group has (``sizes``: one count, or one per group)."""
+        if isinstance(sizes, int):
+            sizes = [sizes] * len(self.groups)
         self.kv_pages.clear()
-        self.num_pages = num_pages
-        for call, need in enumerate(self.needs):
-            if need is None:
-                continue
-            self.kv_pages[call] = {name: torch.zeros((num_pages,) + tuple(shape), dtype=self.dtype, device=self.device)
-                                   for name, shape in need.page_shapes(self.page_size).items()}
+        self.group_pages = [int(n) for n in sizes]
+        self.num_pages = max(self.group_pages, default=0)
+        for g, spec in enumerate(self.groups):
+            for call in spec.calls:
+                need = self.needs[call]
+                dtypes = need.page_dtypes(self.dtype)
+                self.kv_pages[call] = {name: torch.zeros((self.group_pages[g],) + tuple(shape), dtype=dtypes[name],
+                                                         device=self.device)
+                                       for name, shape in need.page_shapes(self.page_size).items()}
         self._graphs.clear()
         self._repeat_graphs.clear()
         self._mixed_graphs.clear()
@@ -242,7 +284,7 @@ class Executor:
         """A manager for this executor's pages and state slots."""
         if enable_prefix_caching is None:
             enable_prefix_caching = self.config.enable_prefix_caching
-        manager = CacheManager(self.groups, self.num_pages, self.page_size, self.num_state_slots,
+        manager = CacheManager(self.groups, list(self.group_pages), self.page_size, self.num_state_slots,
                                enable_prefix_caching=enable_prefix_caching, has_state=self.has_state)
         if self.config.debug_poison_pages:
             self._poison = {g: [] for g in range(len(self.groups))}
@@ -373,9 +415,9 @@ class Executor:
             idx = np.arange(w, dtype=np.int64)[None, :]
             touched = (idx >= first_page[:, None]) & (idx <= last_page[:, None])
             ids = bt[:S][touched]
-            if check_pages and ids.size and (ids.min() < 0 or ids.max() >= self.num_pages):
+            if check_pages and ids.size and (ids.min() < 0 or ids.max() >= self.group_pages[g]):
                 raise ValueError(f"cache group {g}: a block table names a page outside the pool of "
-                                 f"{self.num_pages} (or one that was given back) where the step reads or writes")
+                                 f"{self.group_pages[g]} (or one that was given back) where the step reads or writes")
         if N and (tok[:N].min() < 0 or tok[:N].max() >= self.vocab_size):
             raise ValueError(f"token ids must lie in [0, {self.vocab_size})")
         facts = dict(S=S, N=N, M=M, Sp=Sp, Np=Np, Mp=Mp, q_lens=q_lens, widths=widths)

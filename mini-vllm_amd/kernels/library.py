@@ -85,6 +85,7 @@ _OPTIONAL_SIGNATURES = {
     # A, lda, W, bias, C, ldc, c_dtype, M, N, K, swiglu, work, work_floats, stream
     "mv_gemm_mid": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                             c_void_p, c_long, c_void_p]),
+    "mv_device_compute_units": (c_int, []),
     "mv_gemm_tile_workspace": (c_long, [c_int, c_int, c_int, c_int, c_int]),
     "mv_gemm_tile_splits": (c_int, [c_int, c_int, c_int, c_int, c_int]),
     # A, lda, W, bias, C, ldc, c_dtype, M, N, K, gated, work, work_floats, force, stream

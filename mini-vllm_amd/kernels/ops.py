@@ -73,14 +73,14 @@ FUSED_NORM_MAX_CHUNKS = 32
 # the sampler's first pass: workgroups that share a row, and the rows its scratch is made for
 SAMPLE_CHUNKS = 32
 SAMPLE_WORK_ROWS = 1024
-# compute units of the device the launch heuristics are tuned for
+# compute units of the device the launch heuristics were tuned on; an ``Ops`` asks its device
 COMPUTE_UNITS = 256
 # context length from which the prompt attention uses two key groups per workgroup
 PREFILL_TWO_GROUPS_FROM = 1024
 # waves per workgroup of the decode attention
 DECODE_ATTENTION_WAVES = 4
-# the workgroup kernel splits a sequence's keys until about this many workgroups are in flight
-DECODE_SPLIT_WORKGROUPS = 256
+# the workgroup kernel splits a sequence's keys until about one workgroup for every compute unit is
+# in flight (``Ops.compute_units``)
 # (sequence, kv head) pairs of one decode step whose keys may be split over workgroups
 SPLIT_COUNTERS = 1 << 16
 # from this many tokens on, value rows are written to their pages 16 tokens of a kv head at a time
@@ -178,6 +178,8 @@ class Ops:
         self.lib = library.load(library.variant_of(_NAMES[dtype]))
         self.use_fast_kernels = dtype == torch.bfloat16
         self.use_library_gemm = dtype == torch.bfloat16
+        # compute units of the device: grids are sized in rounds of one workgroup each
+        self.compute_units = int(self.lib.dll.mv_device_compute_units()) if torch.cuda.is_available() else COMPUTE_UNITS
         # set by the executor while it records a graph; library products take part in a recording
         # while ``library_in_graphs`` holds (see _library_allowed)
         self.for_graph = False
@@ -914,7 +916,9 @@ class Ops:
         """One counter for every (sequence, kv head) of a decode step whose keys are split over
         workgroups: the workgroups count themselves in and the last one adds the partial results up.
         The counters are zero between launches (the last workgroup puts its counter back), so they are
-        cleared once, here; launches that share them must follow each other on one stream."""
+        cleared once, here; launches that share them must follow each other on one stream. They belong
+        to this ``Ops`` (an engine has its own), and a launch that fails clears them again
+        (``_decode_launch``)."""
         if partials is None:
             return None
         if self._attn_counters is None:
@@ -923,17 +927,31 @@ class Ops:
             raise ValueError(f"a decode step of {n} (sequence, kv head) pairs exceeds the {SPLIT_COUNTERS} split counters")
         return self._attn_counters.data_ptr()
 
+    def _decode_launch(self, entry: str, *args) -> None:
+        """Launches a decode attention; should the launch fail, the split counters are put back to
+        zero (outside a capture) before the error goes on: a launch that stopped half-way may have
+        left some counted."""
+        try:
+            self.lib.call(entry, *args)
+        except Exception:
+            if self._attn_counters is not None and not torch.cuda.is_current_stream_capturing():
+                try:
+                    torch.cuda.synchronize()
+                    self._attn_counters.zero_()
+                except Exception:
+                    pass
+            raise
+
     def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int):
         """Over how many workgroups a decode step deals a sequence's keys out, and the work area for
         their partial results: (nsplit, partials). The keys go round in groups of 128 (a block of 32
         to each of a workgroup's four waves), so a split beyond the number of such groups in the
         planned context would only add workgroups that end at once. The count is a property of the
-        plan (a captured graph keeps it): about DECODE_SPLIT_WORKGROUPS workgroups in flight, one for
-        every compute unit (measured on MI355X with 8 kv heads at contexts of 1,100: 512 and 1,024
+        plan (a captured graph keeps it): about one workgroup in flight for every compute unit (measured on MI355X with 8 kv heads at contexts of 1,100: 512 and 1,024
         workgroups are 5 and 18 % slower at batch 8; batch 64 is fastest without a split)."""
         ctx = max(1, plan.max_context_len)
         forced = getattr(plan, "decode_splits", None)
-        nsplit = forced if forced else max(1, min(DECODE_SPLIT_WORKGROUPS // max(1, n_seqs * Hkv), -(-ctx // 128), 64))
+        nsplit = forced if forced else max(1, min(self.compute_units // max(1, n_seqs * Hkv), -(-ctx // 128), 64))
         partials = None
         if nsplit > 1:
             rows = max(n_seqs * nsplit, 2048 // Hkv, 256)      # one size serves every batch of a graph set
@@ -994,7 +1012,7 @@ class Ops:
             rope_rows = None
         nsplit, partials = self._decode_split(plan, n, H, Hkv, D)
         self._note_attention("mv_attention_decode_fused", plan, n, H, Hkv, D, 2, splits=nsplit)
-        self.lib.call("mv_attention_decode_fused", qkv.data_ptr(), stride, 0, H * D, (H + Hkv) * D, out.data_ptr(), os_,
+        self._decode_launch("mv_attention_decode_fused", qkv.data_ptr(), stride, 0, H * D, (H + Hkv) * D, out.data_ptr(), os_,
                       k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n, H, Hkv, D, float(scale),
                       -1 if window is None else int(window), _ptr(q_weight), _ptr(k_weight), wcode, float(eps),
@@ -1015,7 +1033,7 @@ class Ops:
         if plan.decode_only and group <= 16:
             nsplit, partials = self._decode_split(plan, n_seqs, H, Hkv, D)
             self._note_attention("mv_attention_decode", plan, q.shape[0], H, Hkv, D, 2, splits=nsplit)
-            self.lib.call("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
+            self._decode_launch("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
                           _ptr(partials), self._split_counters(n_seqs * Hkv, partials), nsplit,
@@ -1032,7 +1050,7 @@ class Ops:
             u = self.lib.dll.mv_attention_prefill_unit_tokens(group, cand)
             if u > 0:
                 units = plan.units(u)
-                if cand == 2 and units * Hkv < 2 * COMPUTE_UNITS and \
+                if cand == 2 and units * Hkv < 2 * self.compute_units and \
                         self.lib.dll.mv_attention_prefill_unit_tokens(group, 1) > 0:
                     continue
                 nt, n_units = cand, units
@@ -1042,7 +1060,7 @@ class Ops:
         # two key groups per workgroup (eight waves) halve the walk over long contexts; they pay while
         # the grid leaves compute units waiting for the longest walk (measured on MI355X: faster up
         # to two workgroups per compute unit, slower beyond)
-        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_units * Hkv <= 2 * COMPUTE_UNITS else 1
+        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_units * Hkv <= 2 * self.compute_units else 1
         self._note_attention("mv_attention_prefill", plan, q.shape[0], H, Hkv, D, 2)
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
@@ -1107,6 +1125,8 @@ _OPS = {}
 
 
 def get_ops(dtype: torch.dtype) -> Ops:
+    """A front end shared by code outside any engine (tools, tests of single kernels). An engine makes
+    its own (``Ops(dtype)``): launches that share one must follow each other on one stream."""
     ops = _OPS.get(dtype)
     if ops is None:
         ops = _OPS[dtype] = Ops(dtype)

@@ -69,6 +69,13 @@ class Retention:
         (a request that needs more than its pool has is refused when it is submitted)."""
         return None
 
+    def most_pages_held(self, length: int, page_size: int, portion: int) -> Optional[int]:
+        """Most pages a request that grows to ``length`` tokens holds at one time when a step brings at
+        most ``portion`` of its tokens, if the rule can tell: the executor then gives the group's pool no
+        more pages than that for every request that can be live (a group that gives pages back early
+        needs a smaller pool than one that keeps everything). None: as many as ``length`` fills."""
+        return None
+
     def key(self) -> Tuple:
         """Calls whose needs have equal keys share a group: a pool and block tables of their own."""
         return (type(self).__name__,) + tuple(sorted(vars(self).items()))
@@ -88,6 +95,9 @@ class KeepAll(Retention):
     def most_pages(self, length: int, page_size: int) -> Optional[int]:
         return -(-length // page_size)
 
+    def most_pages_held(self, length: int, page_size: int, portion: int) -> Optional[int]:
+        return -(-length // page_size)
+
 
 @dataclass(frozen=True)
 class KeepWindow(Retention):
@@ -105,6 +115,11 @@ class KeepWindow(Retention):
         import numpy as np
         return np.maximum(0, np.asarray(next_positions, dtype=np.int64) - self.window) // page_size
 
+    def most_pages_held(self, length: int, page_size: int, portion: int) -> Optional[int]:
+        # while a portion runs: the window behind its first token, the portion itself, and the two
+        # pages that the ends of that range may only touch
+        return min(-(-length // page_size), (self.window + max(1, portion)) // page_size + 2)
+
 
 class CacheNeed:
     """Paged memory a mixer needs for each token of a request: which tensors a page consists of
@@ -117,17 +132,29 @@ class CacheNeed:
         """Name -> shape of one page of ``page_size`` token slots."""
         raise NotImplementedError
 
+    def page_dtypes(self, activation_dtype: torch.dtype) -> Dict[str, torch.dtype]:
+        """Name -> element type of each page tensor; the default keeps everything in the activation
+        type. A mixer that pages float32 or integer state names the type here."""
+        return {name: activation_dtype for name in self.page_shapes(1)}
+
     def group_key(self) -> Tuple:
         return self.retention.key()
 
-    def bytes_per_token(self, itemsize: int) -> int:
+    def bytes_per_token(self, activation_dtype) -> int:
+        """Bytes of cache one token takes in one call. (An ``int`` is read as the size of an element
+        of every tensor.)"""
+        if isinstance(activation_dtype, int):
+            sizes = {name: activation_dtype for name in self.page_shapes(1)}
+        else:
+            sizes = {name: torch.empty((), dtype=dt).element_size()
+                     for name, dt in self.page_dtypes(activation_dtype).items()}
         total = 0
-        for shape in self.page_shapes(1).values():
+        for name, shape in self.page_shapes(1).items():
             n = 1
             for d in shape:
                 n *= int(d)
-            total += n
-        return total * itemsize
+            total += n * sizes[name]
+        return total
 
 
 @dataclass(frozen=True)

@@ -39,7 +39,8 @@ class WeightError(ValueError):
         if unsupported_dtype:
             kinds = sorted({t for _, t in unsupported_dtype})
             lines.append(f"  unsupported dtype {', '.join(kinds)} ({len(unsupported_dtype)} tensors; the engine keeps "
-                         f"bfloat16 and float32 as stored and converts nothing else):")
+                         f"bfloat16 and float32 as stored and converts nothing else: save the checkpoint again in "
+                         f"bfloat16 or float32 to serve it):")
             lines += [f"    {n}: {t}" for n, t in unsupported_dtype]
         super().__init__("\n".join(lines))
 

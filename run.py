@@ -87,17 +87,21 @@ def main() -> int:
     ap.add_argument("--prompt", action="append", default=None, help="a text prompt (repeatable)")
     ap.add_argument("--prompt-ids", action="append", default=None, help="a prompt as comma-separated token ids")
     ap.add_argument("--no-chat-template", action="store_true", help="encode text prompts as they are")
-    ap.add_argument("--random-model", choices=["tiny", "0.6b"], default=None,
-                    help="write a random-weights model of this shape to a temporary folder and run it")
+    ap.add_argument("--random-model", default=None, metavar="SHAPE",
+                    help="write a random-weights model of this named shape (tiny, 0.6b, ...) to a temporary folder "
+                         "and run it; the architecture is the one the shape's config names")
     args = ap.parse_args()
     logging.basicConfig(format="%(asctime)s: %(message)s", level=logging.INFO, datefmt="%m-%d-%Y %H:%M:%S")
 
     from minivllm_amd import LLM
     tmp = None
     if args.random_model:
-        from minivllm_amd.config import Qwen3Config, qwen3_shape
+        from minivllm_amd.config import named_shape, named_shapes
+        from minivllm_amd.models import config_from_dict
         from minivllm_amd.weights import write_model_folder
-        cfg = Qwen3Config.from_dict(qwen3_shape(args.random_model))
+        if args.random_model not in named_shapes():
+            ap.error(f"--random-model: unknown shape {args.random_model!r} (known: {sorted(named_shapes())})")
+        arch, cfg = config_from_dict(named_shape(args.random_model))       # the registry picks the architecture
         tmp = tempfile.TemporaryDirectory()
         args.model = write_model_folder(os.path.join(tmp.name, "model"), cfg, seed=args.seed)
         logging.info("wrote a random %s model to %s", args.random_model, args.model)

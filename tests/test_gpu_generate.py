@@ -312,16 +312,14 @@ def test_graphs_of_many_sequences_hold_library_products_and_no_memset_node(model
     platform); replays must give what eager steps give."""
     from minivllm_amd.engine.trace import TraceRunner
     from minivllm_amd.kernels.library import KernelLibrary
-    from minivllm_amd.kernels.ops import get_ops
     cfg, w, path = models["B"]
     S = 70
     toks = {f"s{i}": random_tokens(cfg, 12 + i % 5, seed=900 + i) for i in range(S)}
-    ops = get_ops(torch.bfloat16)
     recorded = {"library": 0}
     real_offer = KernelLibrary.offer
 
     def offer(self, name, *args):
-        if name == "mv_gemm_lt" and ops.for_graph and torch.cuda.is_current_stream_capturing():
+        if name == "mv_gemm_lt" and torch.cuda.is_current_stream_capturing():
             recorded["library"] += 1
         return real_offer(self, name, *args)
 

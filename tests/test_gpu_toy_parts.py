@@ -447,8 +447,10 @@ def test_toy_routed_feed_forward_and_learned_positions():
 
 def define_chunk_toy():
     """A third toy architecture. Its mixer caches one tensor per token (the mixer's input itself, no
-    keys and values) and keeps it by a rule of its own: a query sees its own chunk of 12 tokens,
-    every page before that chunk goes back to the pool. Its layers have no feed-forward (a block
+    keys and values) and keeps it by a rule of its own: a query sees its own chunk of tokens (12 in
+    the first layer, 20 in the second, which also pages its tensor in float32 whatever the activation
+    type: two cache groups with pools of their own sizes), every page before that chunk goes back to
+    the pool. Its layers have no feed-forward (a block
     arrangement defined here wires a norm and a mixer only), its norm centres the row (not an RMS
     norm, so no kernel may fuse it as one), and its head caps the logits."""
     from minivllm_amd.config.model_config import ModelConfig
@@ -464,19 +466,28 @@ def define_chunk_toy():
         def first_kept_page(self, next_position, page_size):
             return (next_position // self.chunk) * self.chunk // page_size
 
+        def most_pages_held(self, length, page_size, portion):
+            # the chunk of the portion's first token up to the portion's last token
+            return min(-(-length // page_size), (self.chunk + portion) // page_size + 2)
+
     @dataclass(frozen=True)
     class InputCacheNeed(CacheNeed):
         retention: Retention
         hidden_size: int
+        in_float32: bool = False
 
         def page_shapes(self, page_size):
             return {"x": (page_size, self.hidden_size)}
+
+        def page_dtypes(self, activation_dtype):
+            return {"x": torch.float32 if self.in_float32 else activation_dtype}
 
     @dataclass(frozen=True)
     class ChunkMeanSpec(PartSpec):
         kind: ClassVar[str] = "toy_chunk_mean"
         hidden_size: int = 0
         chunk: int = 1
+        in_float32: bool = False
 
     class ChunkMean(Mixer):
         """y_t = W mean(x_s : chunk start <= s <= t), the x_s read back from the paged cache."""
@@ -488,7 +499,7 @@ def define_chunk_toy():
 
         @classmethod
         def cache_need(cls, spec):
-            return InputCacheNeed(KeepChunk(spec.chunk), spec.hidden_size)
+            return InputCacheNeed(KeepChunk(spec.chunk), spec.hidden_size, spec.in_float32)
 
         def __init__(self, spec, tensors, rt):
             self.spec, self.w = spec, tensors["w"]
@@ -502,7 +513,7 @@ def define_chunk_toy():
             for i, (n, start) in enumerate(zip(ctx.q_lens, ctx.starts)):
                 table = view.block_table[i].long()
                 pos = torch.arange(start, start + n, device=x.device)
-                pages[table[pos // ps], pos % ps] = x[base:base + n]
+                pages[table[pos // ps], pos % ps] = x[base:base + n].to(pages.dtype)
                 for j in range(n):
                     p = start + j
                     seen = torch.arange((p // C) * C, p + 1, device=x.device)
@@ -600,9 +611,10 @@ def define_chunk_toy():
     def plan(cfg):
         h = cfg.hidden_size
         norm = CentredNormSpec(size=h, eps=1e-5)
-        layer = LayerPlan(MixerOnlySpec(), ChunkMeanSpec(hidden_size=h, chunk=12), None, (("mixer", norm),))
+        first = LayerPlan(MixerOnlySpec(), ChunkMeanSpec(hidden_size=h, chunk=12), None, (("mixer", norm),))
+        second = LayerPlan(MixerOnlySpec(), ChunkMeanSpec(hidden_size=h, chunk=20, in_float32=True), None, (("mixer", norm),))
         return ModelPlan(hidden_size=h, vocab_size=cfg.vocab_size, max_positions=cfg.max_position_embeddings,
-                         embedding=EmbeddingSpec(cfg.vocab_size, h), layers=(layer, layer), calls=(Call(0), Call(1)),
+                         embedding=EmbeddingSpec(cfg.vocab_size, h), layers=(first, second), calls=(Call(0), Call(1)),
                          final_norm=norm, head=CappedHeadSpec(cfg.vocab_size, h, cap=3.0))
 
     def tensor_name(cfg, loc):
@@ -613,7 +625,7 @@ def define_chunk_toy():
     return arch, ChunkConfig()
 
 
-def chunk_plain(w: Dict[str, torch.Tensor], tokens, chunk=12, cap=3.0):
+def chunk_plain(w: Dict[str, torch.Tensor], tokens, chunks=(12, 20), cap=3.0):
     w = {k: v.double() for k, v in w.items()}
     x = w["embedding.weight"][torch.tensor(tokens)]
     n = len(tokens)
@@ -622,7 +634,7 @@ def chunk_plain(w: Dict[str, torch.Tensor], tokens, chunk=12, cap=3.0):
         c = v - v.mean(-1, keepdim=True)
         return c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + 1e-5) * weight
 
-    for layer in range(2):
+    for layer, chunk in enumerate(chunks):
         hcur = norm(x, w[f"layers.{layer}.norm.mixer.weight"])
         y = torch.stack([hcur[(t // chunk) * chunk:t + 1].mean(0) for t in range(n)])
         x = x + y @ w[f"layers.{layer}.mixer.w"].T
@@ -634,7 +646,9 @@ def test_toy_one_tensor_cache_with_its_own_retention_norm_block_and_head(dtype):
     """A mixer with a one-tensor cache and a third retention rule, a layer without feed-forward, a
     norm that is no RMS norm and a head that caps its logits: all defined in this file, built and
     stepped through the engine without a change to it; two requests beside each other in portions
-    and token by token, on a pool that holds them only because pages behind a chunk come back."""
+    and token by token, on pools that hold them only because pages behind a chunk come back. The two
+    layers keep chunks of different lengths, so they are two cache groups, each with a pool of its
+    own size, and the second pages its tensor in float32 whatever the activation type."""
     from minivllm_amd.config import EngineConfig
     from minivllm_amd.engine.executor import Executor
     from minivllm_amd.engine.step import SeqStep
@@ -650,10 +664,13 @@ def test_toy_one_tensor_cache_with_its_own_retention_norm_block_and_head(dtype):
     assert sorted(weights) == ["embedding.weight", "final_norm.weight", "head.weight", "layers.0.mixer.w",
                                "layers.0.norm.mixer.weight", "layers.1.mixer.w", "layers.1.norm.mixer.weight"]
     ex = Executor(EngineConfig(model="", dtype=dtype, max_model_len=128, kv_cache_block_size=8,
-                               kv_cache_num_blocks=8, max_num_batched_seqs=2),
+                               kv_cache_num_blocks=(8, 9), max_num_batched_seqs=2),
                   model=(arch, cfg, DictSource(weights)))
-    assert len(ex.groups) == 1 and ex.groups[0].retention.key() == ("KeepChunk", ("chunk", 12))
+    assert [g.retention.key() for g in ex.groups] == [("KeepChunk", ("chunk", 12)), ("KeepChunk", ("chunk", 20))]
     assert {n: tuple(t.shape) for n, t in ex.kv_pages[0].items()} == {"x": (8, 8, 64)}
+    assert {n: tuple(t.shape) for n, t in ex.kv_pages[1].items()} == {"x": (9, 8, 64)}
+    assert ex.kv_pages[0]["x"].dtype == ex.dtype and ex.kv_pages[1]["x"].dtype == torch.float32
+    assert ex.bytes_per_page(1) == 8 * 64 * 4
     mgr = ex.new_cache_manager(enable_prefix_caching=True)
     assert not mgr.prefix_caching                      # the rule does not keep everything
     rng = np.random.default_rng(2)
@@ -668,13 +685,15 @@ def test_toy_one_tensor_cache_with_its_own_retention_norm_block_and_head(dtype):
                 mgr.admit(rid)
             mgr.reserve(rid, len(toks))
             s = mgr.sequence(rid)
-            seqs.append(SeqStep(toks, s.num_computed, [mgr.block_table(rid, 0)], s.state_slot, list(range(len(toks)))))
+            seqs.append(SeqStep(toks, s.num_computed, [mgr.block_table(rid, 0), mgr.block_table(rid, 1)], s.state_slot,
+                                list(range(len(toks)))))
         out = ex.step(seqs).cpu().numpy()
         for rid, toks in entries:
             mgr.commit(rid, len(toks))
         mgr.check_invariants()
         return out
 
+    assert [p.num_pages for p in mgr.pools] == [8, 9]
     assert rel_err(run([("a", reqs["a"])]), want["a"]) <= tol           # whole: all 8 pages for one request
     mgr.release("a")
     done = {r: 0 for r in reqs}
@@ -696,4 +715,11 @@ def test_toy_one_tensor_cache_with_its_own_retention_norm_block_and_head(dtype):
     assert most_used <= 8 and sum(len(t) for t in reqs.values()) > 8 * 8
     for r in reqs:
         mgr.release(r)
-    assert mgr.pools[0].num_free == 8
+    assert [p.num_free for p in mgr.pools] == [8, 9]
+    # pools sized from the memory left: no group gets more pages than its live requests can hold at a
+    # time (two requests; steps of up to 16 tokens: a chunk and a portion, and the pages their ends touch)
+    auto = Executor(EngineConfig(model="", dtype=dtype, max_model_len=128, kv_cache_block_size=8, max_num_batched_seqs=2,
+                                 max_num_batched_tokens=16, gpu_memory_utilization=0.3),
+                    model=(arch, cfg, DictSource(weights)))
+    assert auto.group_pages == [2 * ((12 + 16) // 8 + 2), 2 * ((20 + 16) // 8 + 2)]
+    assert [p.num_pages for p in auto.new_cache_manager().pools] == auto.group_pages
