@@ -24,6 +24,9 @@ move, its operations and the share of the HBM and MFMA peaks these amount to.
 ``--only floor`` times a replayed graph of empty kernels: what every dependent launch of a decode step
 costs before it computes anything.
 
+``--only graphs`` records every decode graph the configuration can ask for ahead of serving and prints
+their number, the time and the device memory they took.
+
 ``--only serve`` runs a continuous-batching workload instead (``--requests`` requests, 256 by
 default, with prompt lengths uniform in 128..2048 and ``--gen-len`` generated tokens each, all
 submitted at once under a budget of ``--token-budget`` tokens a step) and prints its own line:
@@ -297,9 +300,12 @@ def main() -> int:
                     help="launch the next decode steps before the running ones' tokens are read (default: the engine's)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", "--mode", dest="only", choices=["all", "decode", "prefill", "serve", "floor"], default="all",
+    ap.add_argument("--only", "--mode", dest="only", choices=["all", "decode", "prefill", "serve", "floor", "graphs"],
+                    default="all",
                     help="measure one phase alone (for profiling); the line then lacks the other's fields. "
-                         "'serve': the continuous-batching workload; 'floor': what a dependent launch costs in a graph")
+                         "'serve': the continuous-batching workload; 'floor': what a dependent launch costs in a graph; "
+                         "'graphs': time and device memory of recording every decode graph ahead of serving "
+                         "(--max-seqs sequences, contexts up to --context)")
     ap.add_argument("--nodes", type=int, default=170, help="kernels in the graph of --only floor")
     ap.add_argument("--requests", type=int, default=256, help="requests of the serve workload")
     ap.add_argument("--gen-len", type=int, default=256, help="generated tokens per request of the serve workload")
@@ -352,6 +358,23 @@ def main() -> int:
                        "parallelism": "single-gpu"},
             "seconds": round(dt, 3), "prompt_tokens": prompt, "generated_tokens": gen,
             "total_tok_s": round((gen + prompt) / dt, 1), "preemptions": preempted}))
+        return 0
+    if args.only == "graphs":
+        live = args.max_seqs
+        llm, cfg = build_llm(args, shape, layers, max_seqs=live, num_pages=live + 64)
+        ex = llm.executor
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        t0 = time.perf_counter()
+        made = ex.capture_graphs()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        used = free0 - torch.cuda.mem_get_info()[0]
+        print(json.dumps({"metric": "decode graphs recorded ahead of serving", "value": made, "unit": "graphs", "n_gpus": 1,
+                          "seconds": round(dt, 2), "device_bytes": int(used), "ms_per_graph": round(dt / max(made, 1) * 1e3, 1),
+                          "config": {"model": f"qwen3-{args.shape}-shape-random", "layers": layers, "max_seqs": live,
+                                     "seq_len": args.context, "scheduler_steps": args.scheduler_steps,
+                                     "block_size": args.block_size}}))
         return 0
     llm, cfg = build_llm(args, shape, layers)
     if args.emit_kernels:

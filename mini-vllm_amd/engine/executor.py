@@ -779,7 +779,7 @@ class Executor:
     def capture_graphs(self) -> int:
         """Records, ahead of serving, every decode graph the configuration can ask for: batch-size
         buckets up to ``max_num_batched_seqs``, context caps up to ``max_model_len``, single steps
-        and rows of 2 to ``num_scheduler_steps`` (the reference records its buckets when the engine
+        and rows of ``num_scheduler_steps`` (the reference records its buckets when the engine
         starts, minivllm/executor/graph.py:24-58). Otherwise a graph is recorded at its first use,
         which makes that step wait. Returns the number of graphs recorded."""
         caps, cap = [], 1024
@@ -809,7 +809,7 @@ class Executor:
                     self._as_padding(arr, off)
                     self._capture(bucket, cap, arr, off, facts, seqs)
                     made += 1
-                for repeat in range(2, k + 1):          # a row is shorter when a request nears its last token
+                for repeat in ([k] if k > 1 else []):   # rows have the full length or the step runs once
                     if (bucket, cap, repeat) in self._repeat_graphs:
                         continue
                     arr, off, facts = self._fill(seqs, pad_to=bucket, bt_widths=widths, extra_words=7 * bucket,

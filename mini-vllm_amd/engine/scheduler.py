@@ -193,7 +193,9 @@ class Scheduler:
     def _decode_repeat(self, seqs: List[ScheduledSeq]) -> int:
         """How many times in a row the step may run: more than once only when it holds nothing
         but decoded tokens, nobody waits to be admitted or to go on with a prompt, and every
-        request has that many tokens to go and the pages for them (they are reserved here)."""
+        request has that many tokens to go and the pages for them (they are reserved here). A row has
+        the full length or the step runs once: the executor then needs two graphs per batch size and
+        context cap, not one for every length in between (the last few tokens of a request go step by step)."""
         k = self.max_decode_repeat
         if k <= 1 or self.waiting or len(seqs) != len(self.running) or not all(s.is_decode for s in seqs):
             return 1
@@ -206,7 +208,7 @@ class Scheduler:
             if all(sum(e[g] for e in extra) <= self.manager.pools[g].num_free for g in range(len(self.manager.groups))):
                 break
             k -= 1
-        if k <= 1:
+        if k < self.max_decode_repeat:
             return 1
         for s in seqs:
             self.manager.reserve(s.request.id, k)

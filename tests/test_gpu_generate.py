@@ -409,9 +409,9 @@ def test_graphs_recorded_when_the_engine_starts(models):
                 max_num_batched_tokens=64, max_num_batched_seqs=6, num_scheduler_steps=4)
     early = LLM(capture_graphs_at_start=True, **opts)
     ex = early.executor
-    # buckets 1, 2, 4, 8 (the first that holds 6), one context cap (max_model_len), single steps and rows of 2 to 4
+    # buckets 1, 2, 4, 8 (the first that holds 6), one context cap (max_model_len), single steps and whole rows of 4
     assert sorted(ex._graphs) == [(1, 96), (2, 96), (4, 96), (8, 96)]
-    assert sorted(ex._repeat_graphs) == [(b, 96, k) for b in (1, 2, 4, 8) for k in (2, 3, 4)]
+    assert sorted(ex._repeat_graphs) == [(b, 96, 4) for b in (1, 2, 4, 8)]   # a row is whole or one step
     assert all(c["memset"] == 0 for c in ex.graph_census.values())
     before = (sorted(ex._graphs), sorted(ex._repeat_graphs), {k: id(v[0]) for k, v in ex._repeat_graphs.items()})
     got = [o.token_ids for o in early.generate(prompts, params, use_tqdm=False)]

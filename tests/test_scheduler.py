@@ -321,9 +321,10 @@ def test_decode_steps_run_in_a_row():
         assert all(p.num_free == p.num_pages for p in e.manager.pools)
 
 
-def test_repeat_shrinks_to_the_free_pages():
-    """With pages for fewer positions than asked, the step repeats fewer times; nothing is preempted
-    for the sake of repeating."""
+def test_no_row_of_steps_without_the_pages_for_all_of_it():
+    """With pages for fewer positions than a full row needs, the step runs once (a row has the full
+    length or none: the executor keeps two graphs per size, not one per length); nothing is
+    preempted for the sake of repeating."""
     e = FakeEngine(num_pages=5, page_size=4, max_tokens=32, max_seqs=4, repeat=8)
     rng = random.Random(12)
     a = submit(e, [rng.randrange(VOCAB) for _ in range(7)], max_tokens=12, ignore_eos=True)
@@ -332,7 +333,8 @@ def test_repeat_shrinks_to_the_free_pages():
     assert a.completion_tokens == expected_output(a.prompt_tokens, 12)
     assert b.completion_tokens == expected_output(b.prompt_tokens, 3)
     assert e.sched.num_preemptions == 0
-    assert any(1 < st.repeat < 8 for st in e.steps)
+    assert all(st.repeat in (1, 8) for st in e.steps) and any(st.repeat == 1 and all(s.is_decode for s in st.seqs)
+                                                              for st in e.steps)
     assert all(p.num_free == p.num_pages for p in e.manager.pools)
 
 
