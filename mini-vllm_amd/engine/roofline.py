@@ -21,31 +21,33 @@ from typing import Dict, List, Optional, Sequence, Tuple
 PEAK_HBM_BYTES = 8.0e12
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-# entry point -> (pattern of the kernel names it launches, the most launches one call makes)
-KERNELS_OF: Dict[str, Tuple[str, int]] = {
-    "mv_embedding": (r"\bembedding(_gather)?_kernel", 1),
-    "mv_add_rmsnorm": (r"\badd_rmsnorm(_vec)?_kernel", 1),
-    "mv_add_rmsnorm_split": (r"\badd_rmsnorm(_vec)?_kernel", 1),
-    "mv_rmsnorm": (r"\brmsnorm_kernel", 1),
-    "mv_qk_norm_rope_store": (r"\b(qk_norm_rope_store(_vec)?_kernel|qkv_prompt_vec_kernel|store_v_pages_kernel)", 2),
-    "mv_swiglu": (r"\bswiglu(_vec)?_kernel", 1),
-    "mv_gemm_skinny": (r"\bgemm_skinny_kernel", 1),
-    "mv_gemm_skinny_norm": (r"\bgemm_skinny_kernel", 1),
-    "mv_gemm_skinny_swiglu": (r"\bgemm_skinny_kernel", 1),
-    "mv_gemm_skinny_fold": (r"\bgemm_skinny_kernel", 1),
-    "mv_gemm_skinny_scaled": (r"\bgemm_skinny_kernel", 1),
-    "mv_scale_rows": (r"\bscale_rows_kernel", 1),
-    "mv_gemm_ref": (r"\bgemm_nt_kernel", 1),
-    "mv_gemm_mid": (r"\bgemm_mid(_reduce)?_kernel", 2),
-    "mv_gemm_tile": (r"\bgemm_(tile|mid_reduce)_kernel", 2),
-    "mv_gemm_lt": (r"^((Custom_)?Cijk_|void hipblaslt|hipblaslt|.*rocblaslt)", 3),
-    "mv_attention_ref": (r"\battention_ref_kernel", 1),
-    "mv_attention_decode": (r"\battention_(decode(_wave)?|merge(_range)?)_kernel", 2),
-    "mv_attention_decode_fused": (r"\battention_(decode(_wave)?|merge(_range)?)_kernel", 2),
-    "mv_attention_prefill": (r"\battention_prefill_kernel", 1),
-    "mv_sample": (r"\bsample(_partial)?_kernel", 2),
+_LIBRARY = r"^((Custom_)?Cijk_|void hipblaslt|hipblaslt|.*rocblaslt)"
+# entry point -> (the kernel a call starts with, the kernel that may follow it within the same call, the
+# most kernels one call launches)
+KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
+    "mv_embedding": (r"\bembedding(_gather)?_kernel", None, 1),
+    "mv_add_rmsnorm": (r"\badd_rmsnorm(_vec)?_kernel", None, 1),
+    "mv_add_rmsnorm_split": (r"\badd_rmsnorm(_vec)?_kernel", None, 1),
+    "mv_rmsnorm": (r"\brmsnorm_kernel", None, 1),
+    "mv_qk_norm_rope_store": (r"\b(qk_norm_rope_store(_vec)?_kernel|qkv_prompt_vec_kernel)", r"\bstore_v_pages_kernel", 2),
+    "mv_swiglu": (r"\bswiglu(_vec)?_kernel", None, 1),
+    "mv_gemm_skinny": (r"\bgemm_skinny_kernel", None, 1),
+    "mv_gemm_skinny_norm": (r"\bgemm_skinny_kernel", None, 1),
+    "mv_gemm_skinny_swiglu": (r"\bgemm_skinny_kernel", None, 1),
+    "mv_gemm_skinny_fold": (r"\bgemm_skinny_kernel", None, 1),
+    "mv_gemm_skinny_scaled": (r"\bgemm_skinny_kernel", None, 1),
+    "mv_scale_rows": (r"\bscale_rows_kernel", None, 1),
+    "mv_gemm_ref": (r"\bgemm_nt_kernel", None, 1),
+    "mv_gemm_mid": (r"\bgemm_mid_kernel", r"\bgemm_mid_reduce_kernel", 2),
+    "mv_gemm_tile": (r"\bgemm_tile_kernel", r"\bgemm_mid_reduce_kernel", 2),
+    "mv_gemm_lt": (_LIBRARY, _LIBRARY, 3),
+    "mv_attention_ref": (r"\battention_ref_kernel", None, 1),
+    "mv_attention_decode": (r"\battention_decode(_wave)?_kernel", r"\battention_merge(_range)?_kernel", 2),
+    "mv_attention_decode_fused": (r"\battention_decode(_wave)?_kernel", r"\battention_merge(_range)?_kernel", 2),
+    "mv_attention_prefill": (r"\battention_prefill_kernel", None, 1),
+    "mv_sample": (r"\bsample(_partial)?_kernel", r"\bsample_kernel", 2),
 }
-_OURS = re.compile("|".join(f"(?:{p})" for p, _ in KERNELS_OF.values()))
+_OURS = re.compile("|".join(f"(?:{p})" for spec in KERNELS_OF.values() for p in spec[:2] if p))
 
 
 @dataclass
@@ -123,15 +125,18 @@ class Window:
 
 
 def _align(trace: Sequence[Tuple[str, float]], start: int, patterns, limits) -> Optional[Tuple[Window, int]]:
+    """``patterns``: per ledger line the kernel a launch starts with and the one that may follow it
+    (two products of the same kernel in a row are two launches, not one launch's pair)."""
     i, n = start, len(trace)
     times, names, other, other_count = [], [], 0.0, 0
-    for pat, limit in zip(patterns, limits):
+    for (pat, follow), limit in zip(patterns, limits):
         while i < n and not _OURS.search(trace[i][0]):
             other += trace[i][1]
             other_count += 1
             i += 1
         got_t, got_n = [], []
-        while i < n and len(got_t) < limit and pat.search(trace[i][0]):
+        while i < n and len(got_t) < limit and (pat if not got_t else follow) is not None \
+                and (pat if not got_t else follow).search(trace[i][0]):
             got_t.append(trace[i][1])
             got_n.append(trace[i][0])
             i += 1
@@ -144,9 +149,10 @@ def _align(trace: Sequence[Tuple[str, float]], start: int, patterns, limits) -> 
 
 def find_windows(trace: Sequence[Tuple[str, float]], ledger: Sequence[Launch], most: int = 256) -> List[Window]:
     """Every place in the trace where the kernels of ``ledger`` follow each other, the last first."""
-    patterns = [re.compile(KERNELS_OF[l.entry][0]) for l in ledger]
-    limits = [KERNELS_OF[l.entry][1] for l in ledger]
-    first = patterns[0]
+    patterns = [(re.compile(KERNELS_OF[l.entry][0]), re.compile(KERNELS_OF[l.entry][1]) if KERNELS_OF[l.entry][1] else None)
+                for l in ledger]
+    limits = [KERNELS_OF[l.entry][2] for l in ledger]
+    first = patterns[0][0]
     windows, taken_from = [], len(trace)
     for start in range(len(trace) - 1, -1, -1):
         if not first.search(trace[start][0]):

@@ -70,3 +70,25 @@ def test_one_step_of_a_row_and_errors(tmp_path):
     stats.write_text('"Name","Calls","TotalDurationNs"\n"k",1,5\n')
     with pytest.raises(ValueError, match="not a rocprofv3 kernel trace"):
         roofline.read_trace(str(stats))
+
+
+def test_two_products_of_one_kernel_in_a_row_are_two_launches(tmp_path):
+    """A product whose K is split launches its kernel and the one that adds the partial sums; the
+    same kernel twice in a row is two products, and only the second kind of kernel may follow within
+    a launch."""
+    step = [("mv_embedding", 100, 0), ("mv_gemm_tile", 4000, 8000), ("mv_gemm_tile", 2000, 4000),
+            ("mv_add_rmsnorm_split", 500, 0), ("mv_gemm_tile", 3000, 6000), ("mv_sample", 300, 600)]
+    kernels = [("void embedding_gather_kernel(int const*)", 1.0),
+               ("void gemm_tile_kernel<2, 4, true, 3, 2>(TileArgs)", 40.0),
+               ("void gemm_tile_kernel<2, 2, false, 4, 2>(TileArgs)", 20.0),
+               ("void add_rmsnorm_vec_kernel<bf16, true>(float*)", 5.0),
+               ("void gemm_tile_kernel<2, 2, false, 4, 2>(TileArgs)", 15.0),
+               ("void gemm_mid_reduce_kernel<bf16>(float const*)", 4.0),
+               ("void sample_kernel(float const*)", 2.0)]
+    path = str(tmp_path / "t_kernel_trace.csv")
+    write_trace(path, kernels * 3)
+    found = roofline.find_windows(roofline.read_trace(path), roofline.launches(step))
+    assert len(found) == 3
+    assert [len(t) for t in found[0].times] == [1, 1, 1, 1, 2, 1]
+    text = roofline.kernel_table(path, roofline.launches(step), "bfloat16", title="t")
+    assert "3 occurrences" in text
