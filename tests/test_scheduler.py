@@ -321,6 +321,30 @@ def test_decode_steps_run_in_a_row():
         assert all(p.num_free == p.num_pages for p in e.manager.pools)
 
 
+def test_decode_steps_list_the_longest_contexts_first():
+    """A step of decoded tokens only names its requests by falling context length (the attention's
+    workgroups start in that order); steps with prompt portions keep the order of arrival; the tokens
+    are what they are in any order."""
+    rng = random.Random(5)
+    lengths = (7, 30, 3, 18, 30, 11)
+    e = FakeEngine(num_pages=128, page_size=4, max_tokens=64, max_seqs=8, repeat=2)
+    reqs = [submit(e, [rng.randrange(VOCAB) for _ in range(n)], max_tokens=9 + i, ignore_eos=True) for i, n in enumerate(lengths)]
+    n = 0
+    while not e.sched.finished:
+        e.run_step()
+        n += 1
+        assert n < 1000
+    decode_steps = [st for st in e.steps if all(s.is_decode for s in st.seqs)]
+    assert decode_steps and any(len(st.seqs) == len(lengths) for st in decode_steps)
+    for st in decode_steps:
+        starts = [s.start for s in st.seqs]
+        assert starts == sorted(starts, reverse=True)
+    first = e.steps[0]
+    assert [s.request.id for s in first.seqs] == [r.id for r in reqs][:len(first.seqs)]
+    for i, r in enumerate(reqs):
+        assert r.completion_tokens == expected_output(r.prompt_tokens, 9 + i, ignore_eos=True)
+
+
 def test_no_row_of_steps_without_the_pages_for_all_of_it():
     """With pages for fewer positions than a full row needs, the step runs once (a row has the full
     length or none: the executor keeps two graphs per size, not one per length); nothing is
