@@ -55,17 +55,28 @@ LIBRARY_TALL_WEIGHT_GATED = 240 * 1000 * 1000
 # at 64 rows 6.8 against 7.8 us, at 256 rows 7.2 against the library's 9.0; weights with fewer rows go to
 # the library, which is a tenth ahead there); any plain product against a weight of 16 MB and more from
 # 33 to 256 rows (8B sizes at 128 rows: down 33 against the library's 67 us, o 16 against 23, qkv 22 against 25).
+# Below 33 rows it is ahead of the kernel that splits K over workgroups wherever that one was used (9 rows and
+# more: 8B sizes at 16 rows o 11.6 against 13.6 us, down 23.7 against 28.7, gate/up 41.9 against 47.7; 32B o at
+# 12 rows 19.7 against 23.3; in the model 8B decode at 12 / 16 / 32 sequences 9 / 10 / 3 % faster, 32B at 16
+# sequences 8 %), and at 8 rows against weights of 96 MB and more (32B down 53 against 64 us, 32B qkv 23 against
+# 29; 32B decode at batch 8 2.4 % faster) unless a norm can be folded into the weight-streaming product instead
+# (8B down: 24.9 us with the norm in it against 23.7 and a norm kernel of 5). Fewer rows stay where they were:
+# in the model a 32B step of one sequence was 2 % slower with the tiled product, and the gated 8B pair behind a
+# folded norm at 8 rows made the step 4 % slower although the product alone was 4 us faster.
 TILE_MIN_WEIGHT = 4 * 1024 * 1024             # bytes: smaller weights were not measured and stay where they were
 TILE_GATED_MIN_M = 32
 TILE_GATED_MAX_M = 1536
 TILE_GATED_BIG_WEIGHT = 64 * 1024 * 1024      # bytes
+TILE_GATED_BIG_MIN_M = 9
 TILE_GATED_BIG_MAX_M = 128
 TILE_SMALL_MIN_M = 40
 TILE_SMALL_MAX_M = 512
 TILE_SMALL_MIN_N = 4096
 TILE_BIG_WEIGHT = 16 * 1024 * 1024            # bytes
-TILE_BIG_MIN_M = 33
+TILE_BIG_MIN_M = 9
 TILE_BIG_MAX_M = 256
+TILE_HUGE_WEIGHT = 96 * 1024 * 1024           # bytes
+TILE_HUGE_MIN_M = 8
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
@@ -178,6 +189,7 @@ class Ops:
         self.lib = library.load(library.variant_of(_NAMES[dtype]))
         self.use_fast_kernels = dtype == torch.bfloat16
         self.use_library_gemm = dtype == torch.bfloat16
+        self.use_tiled_gemm = dtype == torch.bfloat16     # (a test of the kernels behind it switches it off)
         # compute units of the device: grids are sized in rounds of one workgroup each
         self.compute_units = int(self.lib.dll.mv_device_compute_units()) if torch.cuda.is_available() else COMPUTE_UNITS
         # set by the executor while it records a graph; library products take part in a recording
@@ -476,7 +488,8 @@ class Ops:
                 and self._library_allowed(M, N, K, bias is not None, out.dtype)
                 and self._library_product(a, w, bias, out)):
             return None
-        if fast and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.wants_tile(M, N, K):
+        if fast and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.wants_tile(
+                M, N, K, fold_offered=fold is not None and self._fold_serves(fold, out, M, N)):
             if defer_sum and out.dtype == self.dtype and out.is_contiguous():
                 pending = self._gemm_tile_sums(a, lda, w, bias, out, M, N, K)
                 if pending is not None:
@@ -611,23 +624,28 @@ class Ops:
                       self._stream())
         return True
 
-    def wants_tile(self, M: int, N: int, K: int, gated: bool = False) -> bool:
+    def wants_tile(self, M: int, N: int, K: int, gated: bool = False, fold_offered: bool = False) -> bool:
         """Whether M rows against an [N, K] weight (``gated``: the packed gate/up pair) go to the tiled
-        product (see TILE_GATED_MIN_M)."""
-        if not (self.use_fast_kernels and self.lib.has("mv_gemm_tile")) or K % 64 or M * N >= 1 << 31:
+        product (see TILE_GATED_MIN_M). ``fold_offered``: the caller could fold a norm into the
+        weight-streaming product instead, which keeps the few-row steps of the largest weights."""
+        if not (self.use_fast_kernels and self.use_tiled_gemm and self.lib.has("mv_gemm_tile")) or K % 64 or M * N >= 1 << 31:
             return False
         weight_bytes = 2 * N * K
         if weight_bytes < TILE_MIN_WEIGHT:
             return False
         if gated:
             # (the largest pairs, 32B-sized ones, stream faster through the library at any number of rows)
-            if N % 2 or M < TILE_GATED_MIN_M or N * K >= LIBRARY_TALL_WEIGHT_GATED:
+            if N % 2 or N * K >= LIBRARY_TALL_WEIGHT_GATED:
                 return False
-            return M <= (TILE_GATED_MAX_M if weight_bytes < TILE_GATED_BIG_WEIGHT else TILE_GATED_BIG_MAX_M)
+            if weight_bytes >= TILE_GATED_BIG_WEIGHT:
+                return TILE_GATED_BIG_MIN_M <= M <= TILE_GATED_BIG_MAX_M
+            return TILE_GATED_MIN_M <= M <= TILE_GATED_MAX_M
         if self.prefers_library(M, N, K):
             return False
         if weight_bytes >= TILE_BIG_WEIGHT:
-            return TILE_BIG_MIN_M <= M <= TILE_BIG_MAX_M
+            if M < TILE_BIG_MIN_M:
+                return M >= TILE_HUGE_MIN_M and weight_bytes >= TILE_HUGE_WEIGHT and not fold_offered
+            return M <= TILE_BIG_MAX_M
         return N >= TILE_SMALL_MIN_N and TILE_SMALL_MIN_M <= M <= TILE_SMALL_MAX_M
 
     def _gemm_tile_sums(self, a: torch.Tensor, lda: int, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,

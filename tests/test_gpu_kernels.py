@@ -732,10 +732,13 @@ def test_gemm_weight_streaming(out_dtype, M, N, K):
     (9, 3100, 4096, False, torch.bfloat16), (1, 5120, 25600, False, torch.bfloat16),
     (3, 2 * 12032, 5120, True, torch.bfloat16)])
 def test_gemm_for_a_few_dozen_rows_against_large_weights(M, N, K, swiglu, out_dtype):
-    """9 to 32 rows against a weight of tens of megabytes, any number of rows up to 64 against one
-    of hundreds: the kernel that shares the activation rows through LDS and splits K over
-    workgroups (partial sums added in a fixed order)."""
-    ops = ops_for(torch.bfloat16)
+    """The kernel that shares the activation rows through LDS and splits K over workgroups (partial
+    sums added in a fixed order): it serves what the tiled product does not take (gated pairs of a few
+    dozen megabytes below 32 rows, the largest weights below 8 rows, K no multiple of 64), and here,
+    with the tiled product switched off, everything it used to."""
+    from minivllm_amd.kernels.ops import Ops
+    ops = Ops(torch.bfloat16)
+    ops.use_tiled_gemm = False        # (the tiled product has taken most of these shapes over: see test_which_product_...)
     g = torch.Generator().manual_seed(19)
     a = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
@@ -909,7 +912,10 @@ def test_gemm_tiled_behind_a_folded_norm(M, N, K, gated, with_bias):
 @pytest.mark.parametrize("M,N,K,gated,kernel", [
     (64, 4096, 1024, False, "mv_gemm_tile"), (300, 4096, 1024, False, "mv_gemm_tile"), (600, 4096, 1024, False, "mv_gemm_lt"),
     (32, 4096, 1024, False, "mv_gemm_skinny"), (100, 1024, 2048, False, "mv_gemm_lt"), (64, 4096, 4096, False, "mv_gemm_tile"),
-    (200, 4096, 12288, False, "mv_gemm_tile"), (32, 4096, 4096, False, "mv_gemm_mid"), (40, 6144, 1024, True, "mv_gemm_tile"),
+    (200, 4096, 12288, False, "mv_gemm_tile"), (32, 4096, 4096, False, "mv_gemm_tile"), (40, 6144, 1024, True, "mv_gemm_tile"),
+    (9, 4096, 4096, False, "mv_gemm_tile"), (8, 4096, 4096, False, "mv_gemm_skinny"), (8, 4096, 12288, False, "mv_gemm_tile"),
+    (7, 4096, 12288, False, "mv_gemm_skinny"), (4, 5120, 25600, False, "mv_gemm_mid"), (12, 24576, 4096, True, "mv_gemm_tile"),
+    (8, 24576, 4096, True, "mv_gemm_skinny_swiglu"), (20, 6144, 2048, True, "mv_gemm_mid"),
     (1024, 6144, 1024, True, "mv_gemm_tile"), (24, 6144, 1024, True, "mv_gemm_skinny_swiglu"),
     (40, 1024, 256, True, "mv_gemm_skinny_swiglu"),
     (100, 24576, 4096, True, "mv_gemm_tile"), (200, 24576, 4096, True, None)])
@@ -1301,17 +1307,21 @@ def test_kernels_that_load_straight_into_lds_repeat_their_results():
             again = torch.empty_like(first)
             assert ops.gemm_tile(a, w, again, None, gated)
             assert torch.equal(first, again)
-    for M, N, K in ((32, 4096, 4096), (9, 3100, 8192), (30, 12288, 2048)):
-        a = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
-        w = dev((torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16))
-        ops._mid_work = None
-        first = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
-        ops.gemm(a, w, first)
-        assert ops._mid_work is not None
-        for _ in range(30):
-            again = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
-            ops.gemm(a, w, again)
-            assert torch.equal(first, again)
+    ops.use_tiled_gemm = False
+    try:
+        for M, N, K in ((32, 4096, 4096), (9, 3100, 8192), (30, 12288, 2048)):
+            a = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
+            w = dev((torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16))
+            ops._mid_work = None
+            first = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+            ops.gemm(a, w, first)
+            assert ops._mid_work is not None
+            for _ in range(30):
+                again = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+                ops.gemm(a, w, again)
+                assert torch.equal(first, again)
+    finally:
+        ops.use_tiled_gemm = True
     # prompt attention: one long portion over scrambled pages, both walks of the keys
     H, Hkv, D, ps = 16, 8, 128, 16
     for T in (700, 2048):
