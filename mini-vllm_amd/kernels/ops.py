@@ -62,7 +62,9 @@ LIBRARY_TALL_WEIGHT_GATED = 240 * 1000 * 1000
 # 29; 32B decode at batch 8 2.4 % faster) unless a norm can be folded into the weight-streaming product instead
 # (8B down: 24.9 us with the norm in it against 23.7 and a norm kernel of 5). Fewer rows stay where they were:
 # in the model a 32B step of one sequence was 2 % slower with the tiled product, and the gated 8B pair behind a
-# folded norm at 8 rows made the step 4 % slower although the product alone was 4 us faster.
+# folded norm at 8 rows made the step 4 % slower although the product alone was 4 us faster. The largest weights
+# (MID_ALWAYS_WEIGHT: 32B down) take it from the first row on: 48 us in the model against the K-splitting kernel's
+# 58, 32B decode at 1 / 4 / 8 sequences 1-6 / 3-6 / 6 % faster.
 TILE_MIN_WEIGHT = 4 * 1024 * 1024             # bytes: smaller weights were not measured and stay where they were
 TILE_GATED_MIN_M = 32
 TILE_GATED_MAX_M = 1536
@@ -489,7 +491,8 @@ class Ops:
                 and self._library_product(a, w, bias, out)):
             return None
         if fast and lda % 8 == 0 and a.data_ptr() % 16 == 0 and self.wants_tile(
-                M, N, K, fold_offered=fold is not None and self._fold_serves(fold, out, M, N)):
+                M, N, K, fold_offered=(fold is not None and self._fold_serves(fold, out, M, N)
+                                       and not (self.wants_mid(M, N, K) and self.lib.has("mv_gemm_mid")))):
             if defer_sum and out.dtype == self.dtype and out.is_contiguous():
                 pending = self._gemm_tile_sums(a, lda, w, bias, out, M, N, K)
                 if pending is not None:
@@ -644,6 +647,8 @@ class Ops:
             return False
         if weight_bytes >= TILE_BIG_WEIGHT:
             if M < TILE_BIG_MIN_M:
+                if N * K >= MID_ALWAYS_WEIGHT:
+                    return True
                 return M >= TILE_HUGE_MIN_M and weight_bytes >= TILE_HUGE_WEIGHT and not fold_offered
             return M <= TILE_BIG_MAX_M
         return N >= TILE_SMALL_MIN_N and TILE_SMALL_MIN_M <= M <= TILE_SMALL_MAX_M

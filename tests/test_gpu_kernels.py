@@ -914,7 +914,7 @@ def test_gemm_tiled_behind_a_folded_norm(M, N, K, gated, with_bias):
     (32, 4096, 1024, False, "mv_gemm_skinny"), (100, 1024, 2048, False, "mv_gemm_lt"), (64, 4096, 4096, False, "mv_gemm_tile"),
     (200, 4096, 12288, False, "mv_gemm_tile"), (32, 4096, 4096, False, "mv_gemm_tile"), (40, 6144, 1024, True, "mv_gemm_tile"),
     (9, 4096, 4096, False, "mv_gemm_tile"), (8, 4096, 4096, False, "mv_gemm_skinny"), (8, 4096, 12288, False, "mv_gemm_tile"),
-    (7, 4096, 12288, False, "mv_gemm_skinny"), (4, 5120, 25600, False, "mv_gemm_mid"), (12, 24576, 4096, True, "mv_gemm_tile"),
+    (7, 4096, 12288, False, "mv_gemm_skinny"), (4, 5120, 25600, False, "mv_gemm_tile"), (12, 24576, 4096, True, "mv_gemm_tile"),
     (8, 24576, 4096, True, "mv_gemm_skinny_swiglu"), (20, 6144, 2048, True, "mv_gemm_mid"),
     (1024, 6144, 1024, True, "mv_gemm_tile"), (24, 6144, 1024, True, "mv_gemm_skinny_swiglu"),
     (40, 1024, 256, True, "mv_gemm_skinny_swiglu"),
