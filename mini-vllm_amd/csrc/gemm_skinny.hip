@@ -21,6 +21,10 @@
 // pieces the last eight are the other half. Two MFMAs a load instead of one (the matrix unit is idle
 // anyway), two accumulators, added across the lane halves once behind the loop, which also restores
 // the usual result layout. 8B-sized gate/up at 8 rows: 45.6 -> 39.4 us, down 27.4 -> 25.1.
+// PAIRED == 2 (up to 8 rows): the tokens' loads take whole lines the same way — lane l holds piece
+// 2 (l / 16) + (l % 16) / 8 of token (l % 16) % 8 — and one MFMA a load is enough: its result rows
+// 0-7 x columns 0-7 are the dot products' even halves, rows 8-15 x columns 8-15 the odd halves of
+// the same (weight row, token) pairs, the other two quarters are not used.
 //
 // A fused variant computes the gated activation of a feed-forward in the same pass:
 //     out[M, I] = silu(A Wg^T) * (A Wu^T)  with Wg = W[0:I], Wu = W[I:2I].
@@ -55,7 +59,7 @@ struct NormInput {
 // Every workgroup normalises the (few) rows for itself into LDS, which costs less than a kernel
 // launch; workgroup 0 also writes x to resid_out (a buffer other than resid_in: the other
 // workgroups still read that one).
-template <int R, int TM, bool SWIGLU, bool NORM, typename TC, int EPI = EPI_NONE, bool PAIRED = false>
+template <int R, int TM, bool SWIGLU, bool NORM, typename TC, int EPI = EPI_NONE, int PAIRED = 0>
 __global__ void __launch_bounds__(64 * SK_MAX_WAVES)
 gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict__ W, const bf16* __restrict__ bias,
                    TC* __restrict__ C, long ldc, int M, int N, int K, int groups, int blocks, int rows,
@@ -123,7 +127,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
         }
     // operand u (0 .. U-1, U even when PAIRED) of the stage that starts at k-step k
     auto w_at = [&](int r, int k, int u) -> uint4 {
-        if constexpr (PAIRED) return wrow[r][u & 1][(size_t)(k + (u & ~1)) * 4];
+        if constexpr (PAIRED != 0) return wrow[r][u & 1][(size_t)(k + (u & ~1)) * 4];
         else return wrow[r][0][(size_t)(k + u) * 4];
     };
     // k-steps per register stage of the main loop (see there)
@@ -223,21 +227,32 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 #pragma unroll
         for (int t = 0; t < TM; ++t) {
             const int tok = 16 * t + i;
-            avalid[t] = tok < M;
-            arow[t] = reinterpret_cast<const uint4*>(sA + (size_t)(avalid[t] ? tok : 0) * lds_ld) + (PAIRED ? 2 * g : g);
+            if (PAIRED == 2) {
+                avalid[t] = i % 8 < M;
+                arow[t] = reinterpret_cast<const uint4*>(sA + (size_t)(avalid[t] ? i % 8 : 0) * lds_ld) + (2 * g + i / 8);
+            } else {
+                avalid[t] = tok < M;
+                arow[t] = reinterpret_cast<const uint4*>(sA + (size_t)(avalid[t] ? tok : 0) * lds_ld) + (PAIRED ? 2 * g : g);
+            }
         }
     } else {
 #pragma unroll
         for (int t = 0; t < TM; ++t) {
             const int tok = 16 * t + i;
-            avalid[t] = tok < M;
-            arow[t] = reinterpret_cast<const uint4*>(A + (size_t)(avalid[t] ? tok : 0) * lda) + (PAIRED ? 2 * g : g);
+            if (PAIRED == 2) {
+                avalid[t] = i % 8 < M;
+                arow[t] = reinterpret_cast<const uint4*>(A + (size_t)(avalid[t] ? i % 8 : 0) * lda) + (2 * g + i / 8);
+            } else {
+                avalid[t] = tok < M;
+                arow[t] = reinterpret_cast<const uint4*>(A + (size_t)(avalid[t] ? tok : 0) * lda) + (PAIRED ? 2 * g : g);
+            }
         }
     }
-    // (PAIRED: operand u of a stage is piece 2 g + u % 2 of chunk u / 2)
+    // (PAIRED: operand u of a stage is piece 2 g + u % 2 of chunk u / 2; PAIRED == 2: one operand a chunk, the even u)
     auto a_at = [&](int t, int k, int u) -> uint4 {
-        if (!avalid[t]) return uint4{0u, 0u, 0u, 0u};
-        if constexpr (PAIRED) return arow[t][(size_t)(k + (u & ~1)) * 4 + (u & 1)];
+        if (!avalid[t] || (PAIRED == 2 && (u & 1))) return uint4{0u, 0u, 0u, 0u};
+        if constexpr (PAIRED == 2) return arow[t][(size_t)(k + u) * 4];
+        else if constexpr (PAIRED == 1) return arow[t][(size_t)(k + (u & ~1)) * 4 + (u & 1)];
         else return arow[t][(size_t)(k + u) * 4];
     };
 
@@ -308,7 +323,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
     };
     // PAIRED: accp[r][t][h][q] = weight operand of half h times the tokens' pieces of parity q
     floatx4_t accp[PAIRED ? R : 1][PAIRED ? TM : 1][2][2];
-    if constexpr (PAIRED) {
+    if constexpr (PAIRED != 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -328,7 +343,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
         }
     };
     auto multiply = [&](const Stage& st) {
-        if constexpr (PAIRED) {
+        if constexpr (PAIRED != 0) {
 #pragma unroll
             for (int c = 0; c < U / 2; ++c)
 #pragma unroll
@@ -338,7 +353,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
 #pragma unroll
                         for (int h = 0; h < 2; ++h)
 #pragma unroll
-                            for (int q = 0; q < 2; ++q)
+                            for (int q = 0; q < (PAIRED == 2 ? 1 : 2); ++q)
                                 accp[r][t][h][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                                     st.w[2 * c + h][r].v, st.a[2 * c + q][t].v, accp[r][t][h][q], 0, 0, 0);
         } else {
@@ -388,18 +403,18 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
         for (int r = 0; r < R; ++r)
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
-                if constexpr (PAIRED) {
+                if constexpr (PAIRED != 0) {
 #pragma unroll
                     for (int h = 0; h < 2; ++h)
 #pragma unroll
-                        for (int q = 0; q < 2; ++q)
+                        for (int q = 0; q < (PAIRED == 2 ? 1 : 2); ++q)
                             accp[r][t][h][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[h][r].v, a[q][t].v, accp[r][t][h][q], 0, 0, 0);
                 } else {
                     acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[0][r].v, a[0][t].v, acc[r][t], 0, 0, 0);
                 }
             }
     }
-    if constexpr (PAIRED) {
+    if constexpr (PAIRED != 0) {
         // Result rows 0-7 of a tile: the first half's products with the even pieces (they sit in lane
         // groups 0 and 1, where rows 0-7 belong) plus its products with the odd pieces (result rows
         // 8-15 of that MFMA: lane groups 2 and 3). Rows 8-15: the second half's products with the odd
@@ -411,9 +426,19 @@ gemm_skinny_kernel(const bf16* __restrict__ A, long lda, const bf16* __restrict_
             for (int t = 0; t < TM; ++t)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float odd_of_first = __shfl_xor(accp[r][t][0][1][e], 32, MV_WAVE);
-                    const float even_of_second = __shfl_xor(accp[r][t][1][0][e], 32, MV_WAVE);
-                    acc[r][t][e] = g < 2 ? accp[r][t][0][0][e] + odd_of_first : accp[r][t][1][1][e] + even_of_second;
+                    if constexpr (PAIRED == 2) {
+                        // (token j < 8, lane group G): rows 0-7 of the first half = its even halves here plus its
+                        // odd halves at (j + 8, G + 2); rows 8-15 = the second half's even halves at (j, G - 2)
+                        // plus its odd halves at (j + 8, G). Lanes of tokens 8-15 hold nothing that is stored.
+                        const float odd_of_first = __shfl_xor(accp[r][t][0][0][e], 40, MV_WAVE);
+                        const float even_of_second = __shfl_xor(accp[r][t][1][0][e], 32, MV_WAVE);
+                        const float odd_of_second = __shfl_xor(accp[r][t][1][0][e], 8, MV_WAVE);
+                        acc[r][t][e] = g < 2 ? accp[r][t][0][0][e] + odd_of_first : even_of_second + odd_of_second;
+                    } else {
+                        const float odd_of_first = __shfl_xor(accp[r][t][0][1][e], 32, MV_WAVE);
+                        const float even_of_second = __shfl_xor(accp[r][t][1][0][e], 32, MV_WAVE);
+                        acc[r][t][e] = g < 2 ? accp[r][t][0][0][e] + odd_of_first : accp[r][t][1][1][e] + even_of_second;
+                    }
                 }
     }
 
@@ -571,9 +596,14 @@ static void launch_skinny(const void* A, long lda, const void* W, const void* bi
     const size_t lds = skinny_lds_bytes(S, R, TM, false, M, K, EPI == EPI_SCALED);
     if constexpr (TM == 1 && R <= 2) {
         if (skinny_paired(M, SWIGLU ? 2L * N : N, K)) {
-            hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC, EPI, true>), dim3(grid), dim3(64 * S), lds,
-                               stream, (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K,
-                               groups, blocks, rows, NormInput{}, fold);
+            if (M <= 8)
+                hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC, EPI, 2>), dim3(grid), dim3(64 * S), lds,
+                                   stream, (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K,
+                                   groups, blocks, rows, NormInput{}, fold);
+            else
+                hipLaunchKernelGGL((gemm_skinny_kernel<R, TM, SWIGLU, false, TC, EPI, 1>), dim3(grid), dim3(64 * S), lds,
+                                   stream, (const bf16*)A, lda, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K,
+                                   groups, blocks, rows, NormInput{}, fold);
             return;
         }
     }
@@ -589,9 +619,14 @@ static void launch_skinny_norm(const NormInput& norm, const void* W, const void*
     const int blocks = skinny_blocks(N, rows);
     const size_t lds = skinny_lds_bytes(S, R, 1, true, M, K);
     if (skinny_paired(M, SWIGLU ? 2L * N : N, K)) {
-        hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC, EPI_NONE, true>), dim3(blocks), dim3(64 * S), lds,
-                           stream, (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N, K,
-                           1, blocks, rows, norm, RowsInput{});
+        if (M <= 8)
+            hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC, EPI_NONE, 2>), dim3(blocks), dim3(64 * S), lds,
+                               stream, (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N,
+                               K, 1, blocks, rows, norm, RowsInput{});
+        else
+            hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC, EPI_NONE, 1>), dim3(blocks), dim3(64 * S), lds,
+                               stream, (const bf16*)nullptr, (long)K, (const bf16*)W, (const bf16*)bias, (TC*)C, ldc, M, N,
+                               K, 1, blocks, rows, norm, RowsInput{});
         return;
     }
     hipLaunchKernelGGL((gemm_skinny_kernel<R, 1, SWIGLU, true, TC>), dim3(blocks), dim3(64 * S), lds, stream,
