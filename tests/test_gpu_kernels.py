@@ -697,7 +697,9 @@ def test_attention_decode_fused_kernel(H, Hkv, D, ps, window, with_norm, with_ro
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 70, 96), (8, 1024, 1024), (17, 4100, 64), (64, 333, 3072), (33, 2048, 512),
-                                    (5, 151936 // 8, 1024), (5, 5120, 256), (16, 6144, 128), (3, 330, 64)])
+                                    (5, 151936 // 8, 1024), (5, 5120, 256), (16, 6144, 128), (3, 330, 64),
+                                    # weights of 16 MB and more: the loads of whole lines, up to 8 rows and 9 to 16
+                                    (8, 4100, 2112), (2, 4099, 2112), (7, 4096, 12288)])
 def test_gemm_weight_streaming(out_dtype, M, N, K):
     """The weight-streaming product, also at sizes where a workgroup takes a number of output
     columns that is no multiple of a tile (5120 and 6144 columns: 20 and 24 each; 330: 8, the last
@@ -723,6 +725,30 @@ def test_gemm_weight_streaming(out_dtype, M, N, K):
     ops.gemm(dev(a[M - 1:M]), dev(w), out_one)
     assert torch.equal(out_w[M - 1:M], out_one)
     assert rel_err(out_w.cpu().numpy(), want.numpy()) <= 3e-6
+
+
+@pytest.mark.parametrize("M,N,K", [(12, 5000, 2048), (16, 8200, 1024), (9, 4099, 2112)])
+def test_gemm_weight_streaming_whole_lines_for_9_to_16_rows(M, N, K):
+    """Weights of 16 MB and more at 9 to 16 rows go to the tiled product; the weight-streaming kernel's
+    variant for them (whole-line loads of the weights, two MFMAs a load) serves the fused norm and
+    callers of the entry point. Here with the tiled product switched off: right, and a row's bits are
+    those of the same row alone (the variant for up to 8 rows)."""
+    from minivllm_amd.kernels.ops import Ops
+    ops = Ops(torch.bfloat16)
+    ops.use_tiled_gemm = False
+    g = torch.Generator().manual_seed(18)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    want = a.double() @ w.double().T + b.double()
+    ops.ledger = []
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ops.gemm(dev(a), dev(w), out, dev(b))
+    assert [l[0] for l in ops.ledger] == ["mv_gemm_skinny"]
+    assert rel_err(out.cpu().numpy(), want.numpy()) <= 3e-6
+    one = torch.empty(1, N, dtype=torch.float32, device="cuda")
+    ops.gemm(dev(a[M - 1:M]), dev(w), one, dev(b))
+    assert torch.equal(out[M - 1:M], one)
 
 
 @pytest.mark.parametrize("M,N,K,swiglu,out_dtype", [
@@ -937,7 +963,8 @@ def test_which_product_takes_which_rows(M, N, K, gated, kernel):
     assert seen == ([kernel] if kernel else []), seen
 
 
-@pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 3072, 1024), (40, 100, 96), (64, 560, 256)])
+@pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 3072, 1024), (40, 100, 96), (64, 560, 256),
+                                   (6, 4104, 2048), (13, 4100, 2048)])     # (16 MB and more: loads of whole lines)
 def test_gemm_swiglu_fused(M, I, K):
     ops = ops_for(torch.bfloat16)
     g = torch.Generator().manual_seed(18)
@@ -1126,7 +1153,9 @@ def test_sampling_frequencies():
 
 
 @pytest.mark.parametrize("M,N,K,swiglu", [(1, 4096, 1024, False), (8, 1000, 1024, False), (16, 96, 64, False),
-                                          (8, 3072, 1024, True), (3, 200, 128, True), (5, 333, 2048, False)])
+                                          (8, 3072, 1024, True), (3, 200, 128, True), (5, 333, 2048, False),
+                                          # (16 MB and more: loads of whole lines)
+                                          (7, 6144, 2048, False), (8, 8200, 1536, False), (4, 2 * 4112, 2048, True)])
 @pytest.mark.parametrize("with_delta", [True, False])
 def test_gemm_with_fused_add_and_norm(M, N, K, swiglu, with_delta):
     """Residual add + RMSNorm + product (or gated pair) as one kernel, through the deferred-norm
