@@ -345,9 +345,10 @@ static TilePlan tile_plan(int M, int n_out, int K, bool gated, int force) {
     if (force > 0) return make((force / 10000) % 10, (force / 100) % 100, force % 100, force / 10000 >= 10);
     const bool big = (double)(gated ? 2 : 1) * n_out * K * 2 >= 16.0 * 1024 * 1024;
     const int m_cap = (M + 63) / 64 * 64;
-    // (a gated pair is never split, so the tiles alone have to fill the chip: with one tile of tokens the
-    // 64-row tile's 384 workgroups beat the 128-row tile's 192 on 8B-sized pairs, 41.5 against 46.5 us)
-    const int need = big ? (gated && m_cap <= 64 ? 256 : 64) : 192;
+    // (a gated pair is never split, so the tiles alone have to fill the chip: up to 48 rows the 64-row
+    // tile's 384 workgroups beat the 128-row tile's 192 on 8B-sized pairs, 41.5 against 46.5 us at 12 rows;
+    // at 64 rows the larger tile is ahead again, 45.9 against 47.6)
+    const int need = big ? (gated && M <= 48 ? 256 : 64) : 192;
     const int shapes[4][2] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}};
     TilePlan pick = make(2, 2, 1, false);
     for (int s = 0; s < 4; ++s) {
