@@ -341,6 +341,46 @@ def test_layer_sizes_of_the_0_6b_shape(tmp_path, kind):
             torch.cuda.empty_cache()
 
 
+def test_layer_sizes_of_the_8b_shape(tmp_path):
+    """Two layers of the Qwen3-8B sizes (hidden 4096, 32/8 heads of 128, intermediate 12288; a small
+    vocabulary, untied head) in bfloat16 against the plain model: weights of 34 to 200 MB are what the
+    whole-line variants of the weight-streaming product (steps of up to 8 rows, norms folded into them),
+    the tiled product with its sums left to the norm (9 rows and more) and the library serve, none of which
+    the smaller shapes of the other cases reach. Cuttings: whole, the last 32 one by one, portions, mixed,
+    and twelve requests decoded beside each other."""
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
+           "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 12288,
+           "vocab_size": 2048, "max_position_embeddings": 40960, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+           "tie_word_embeddings": False, "attention_bias": False, "hidden_act": "silu", "torch_dtype": "bfloat16"}
+    weights = make_weights(cfg, seed=8, stored=torch.bfloat16, std=0.02)
+    path = write_model_dir(str(tmp_path / "shape8b"), cfg, weights)
+    reqs = {"p": random_tokens(cfg, 75, seed=1), "q": random_tokens(cfg, 40, seed=2)}
+    crowd = {f"c{i}": random_tokens(cfg, 14 + i % 3, seed=20 + i) for i in range(12)}
+    w64 = {k: v.double() for k, v in weights.items()}
+    want = {r: plain_logits(cfg, w64, t, device="cuda") for r, t in {**reqs, **crowd}.items()}
+    emulated = {r: plain_logits_bf16(cfg, w64, t, device="cuda") for r, t in {**reqs, **crowd}.items()}
+    del w64
+    bf16_err = max(rel_err(emulated[r][p], want[r][p]) for r in want for p in range(len(want[r])))
+    tol = min(bf16_tolerance(bf16_err), MILD_BF16_BOUND)
+    cuttings = {"whole": (reqs, trace_tools.whole(reqs)), "last 32 one by one": (reqs, trace_tools.tail_decode(reqs, tail=32)),
+                "portions": (reqs, trace_tools.portions(reqs, sizes=(7, 40, 2, 17, 3, 29))),
+                "mixed": (reqs, trace_tools.mixed(reqs, {"p": 60, "q": 33}, max_live=2, seed=3, max_portion=40)),
+                "twelve beside each other": (crowd, trace_tools.crowd(crowd, {r: 8 for r in crowd}, seed=4, max_portion=8))}
+    from minivllm_amd.engine.trace import TraceRunner
+    for what, (which, steps) in cuttings.items():
+        runner = TraceRunner(path, "bfloat16", trace_tools.max_live_tokens(steps), page_size=16)
+        seen, note = set(), runner.executor.ops._note
+        runner.executor.ops._note = lambda entry, *rest: (seen.add(entry), note(entry, *rest))[1]
+        got = trace_tools.collect(steps, runner.run_step)
+        _check_rows(got, want, tol, f"8B layer sizes, {what} [bfloat16] (emulated {bf16_err:.2e})")
+        if what == "last 32 one by one":
+            assert {"mv_gemm_skinny_fold", "mv_gemm_skinny_scaled"} <= seen, seen
+        if what == "twelve beside each other":
+            assert "mv_gemm_tile" in seen and "mv_add_rmsnorm_split" in seen, seen
+        del runner
+        torch.cuda.empty_cache()
+
+
 def _check_rows(got, want, tol, what):
     worst, where = 0.0, None
     for (rid, pos), row in got.items():
