@@ -1,4 +1,6 @@
-// Matrix product for many rows (prompt portions, decode steps of more than 64 sequences):
+// Matrix product for the steps between a few rows and thousands (decode steps of 9 sequences and
+// more against large weights, of 32 and more against small ones, prompt portions of up to 1,536
+// tokens; the caller's rules say which):
 //     C[M, N] = A[M, K] * W[N, K]^T (+ bias)      or      C[M, I] = silu(A Wg^T) * (A Wu^T),
 // bf16 inputs, float accumulation, on the MFMA units of gfx950 (v_mfma_f32_16x16x32_bf16).
 //
