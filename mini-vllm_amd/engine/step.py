@@ -80,6 +80,14 @@ class AttentionPlan:
             return tokens // unit_tokens + seqs
         return sum(-(-ql // unit_tokens) for ql in self.q_lens)
 
+    def busy_units(self, unit_tokens: int) -> int:
+        """The units that hold tokens, for rules that weigh the work against the device: the count
+        itself, or, of a bound, the units its tokens fill (the rest of ``units`` are spares that end
+        at once)."""
+        if self.bound is not None:
+            return max(1, self.bound[0] // unit_tokens)
+        return self.units(unit_tokens)
+
 
 class StepContext:
     """Device tensors (int32) and host facts describing the step, handed to every part.

@@ -1068,22 +1068,24 @@ class Ops:
         # 128 columns per workgroup (each operand read from LDS feeds two MFMAs) when that still leaves
         # two workgroups for every compute unit, else 64 (measured on MI355X: 2048 tokens of one
         # sequence with 8 kv heads are faster with 64, 4096 tokens or 8 x 512 with 128)
-        nt, n_units = 0, 0
+        nt, n_units, n_busy = 0, 0, 0
         for cand in (2, 1):
             u = self.lib.dll.mv_attention_prefill_unit_tokens(group, cand)
             if u > 0:
-                units = plan.units(u)
-                if cand == 2 and units * Hkv < 2 * self.compute_units and \
+                units, busy = plan.units(u), plan.busy_units(u)
+                if cand == 2 and busy * Hkv < 2 * self.compute_units and \
                         self.lib.dll.mv_attention_prefill_unit_tokens(group, 1) > 0:
                     continue
-                nt, n_units = cand, units
+                nt, n_units, n_busy = cand, units, busy
                 break
         if nt == 0:
             return False
         # two key groups per workgroup (eight waves) halve the walk over long contexts; they pay while
         # the grid leaves compute units waiting for the longest walk (measured on MI355X: faster up
         # to two workgroups per compute unit, slower beyond)
-        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_units * Hkv <= 2 * self.compute_units else 1
+        # (a recorded step's grid is sized for the most units its size class can have; the rule goes by
+        # the units its tokens fill, as an eager step's does)
+        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_busy * Hkv <= 2 * self.compute_units else 1
         self._note_attention("mv_attention_prefill", plan, q.shape[0], H, Hkv, D, 2)
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
