@@ -625,7 +625,11 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, i
 // fastest over the lanes, so that tokens that follow each other in a sequence fill neighbouring
 // slots and the two-byte stores of a wave merge into 32-byte segments (a store per token and
 // head scatters them 2 bytes at a time). `tile` has a row pitch of W >= D + 1 floats.
-template <typename T, int W>
+// VEC (the caller vouches for 16-byte aligned rows, D a multiple of 8): the rows come in with one
+// 16-byte load a lane, and where eight tokens in a row fill eight neighbouring slots from a slot
+// that is a multiple of eight (the usual case inside a prompt) a lane writes those eight values of
+// one d with one store instead of eight.
+template <typename T, int W, bool VEC = false>
 __device__ __forceinline__ void
 store_v_tile(int tok0, int kvh, const T* __restrict__ qkv, long row_stride, int v_off,
              const int* __restrict__ positions, const int* __restrict__ token_seq,
@@ -645,12 +649,48 @@ store_v_tile(int tok0, int kvh, const T* __restrict__ qkv, long row_stride, int 
         }
         dst_base[tid] = base;
     }
-    for (int idx = tid; idx < 16 * D; idx += 256) {
-        const int j = idx / D, d = idx % D;
-        const int tok = tok0 + j;
-        tile[j][d] = tok < n ? to_f(qkv[(size_t)tok * row_stride + v_off + (size_t)kvh * D + d]) : 0.f;
+    if (VEC) {
+        const int pieces = D / 8;
+        for (int idx = tid; idx < 16 * pieces; idx += 256) {
+            const int j = idx / pieces, d0 = (idx % pieces) * 8;
+            const int tok = tok0 + j;
+            float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (tok < n) Vec8<T>::load(qkv + (size_t)tok * row_stride + v_off + (size_t)kvh * D + d0, x);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) tile[j][d0 + e] = x[e];
+        }
+    } else {
+        for (int idx = tid; idx < 16 * D; idx += 256) {
+            const int j = idx / D, d = idx % D;
+            const int tok = tok0 + j;
+            tile[j][d] = tok < n ? to_f(qkv[(size_t)tok * row_stride + v_off + (size_t)kvh * D + d]) : 0.f;
+        }
     }
     __syncthreads();
+    if (VEC) {
+        // lane (d, h): the eight tokens 8 h .. 8 h + 7 of the tile at this d
+        for (int idx = tid; idx < 2 * D; idx += 256) {
+            const int d = idx / 2, h = idx % 2;
+            const long b0 = dst_base[8 * h];
+            bool run = b0 >= 0 && page_size % 8 == 0;
+#pragma unroll
+            for (int e = 1; e < 8; ++e) run = run && dst_base[8 * h + e] == b0 + e;
+            T* dst = v_pages + b0 + (long)d * page_size;
+            if (run && ((uintptr_t)dst % (8 * sizeof(T))) == 0) {
+                float x[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = tile[8 * h + e][d];
+                Vec8<T>::store(dst, x);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const long base = dst_base[8 * h + e];
+                    if (base >= 0) v_pages[base + (long)d * page_size] = from_f<T>(tile[8 * h + e][d]);
+                }
+            }
+        }
+        return;
+    }
     const int j = tid % 16;
     const long base = dst_base[j];
     if (base < 0) return;
@@ -675,8 +715,8 @@ qkv_prompt_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, int k_off
     __shared__ float tile[16][8 * L + 1];
     __shared__ long dst_base[16];
     const int vb = (int)blockIdx.x - qk_blocks;
-    store_v_tile<T, 8 * L + 1>((vb / Hkv) * 16, vb % Hkv, qkv, row_stride, v_off, positions, token_seq, block_table,
-                               bt_width, page_size, v_pages, n, Hkv, 8 * L, tile, dst_base);
+    store_v_tile<T, 8 * L + 1, true>((vb / Hkv) * 16, vb % Hkv, qkv, row_stride, v_off, positions, token_seq,
+                                     block_table, bt_width, page_size, v_pages, n, Hkv, 8 * L, tile, dst_base);
 }
 
 template <typename T>

@@ -1,7 +1,6 @@
-// What the weight-streaming product (gemm_skinny.hip) and the chained products (gemm_chain.hip)
-// share: operand fragments, the inputs of the variants that take a norm apart, and the launch
-// rules (waves, weight tiles and output columns per workgroup), so that a product gives the same
-// bits whichever of the two kernels runs it.
+// The shapes of the weight-streaming product (gemm_skinny.hip), apart from its kernel: operand
+// fragments, the inputs of the variants that take a norm apart, and the launch rules (waves,
+// weight tiles and output columns per workgroup).
 #pragma once
 #include "dispatch.h"
 
