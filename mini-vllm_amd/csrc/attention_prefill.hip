@@ -195,97 +195,97 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     // one d row (V). Everything that does not depend on the block is worked out once. The block
     // number is the same for a wave, so its page ids are scalar loads, asked for a round before they
     // are used.
+    // The page ids of a block are per-lane loads: a lane brings in keys of one half of the block and
+    // values of one half (the halves differ), so it asks for exactly the two ids it needs, a round
+    // before they are used, and nothing of the addressing lives in scalar registers.
     struct PageIds {
-        int pg[2];    // the pages of the block's two halves of 16 keys
+        int k, v;     // the pages of the lane's key half and value half
     };
     const int rho = lane % 16;
     // K: row rho of score tile t is key 8*(rho/4) + 4t + rho%4; the half of the block it lies in
     // does not depend on t
     const int k_half = rho / 8;
-    unsigned k_off[KREP];
-#pragma unroll
-    for (int rep = 0; rep < KREP; ++rep) {
-        const int pair = cw + AP_WAVES * rep;   // (score tile, k-step): LDS chunks pair * 64 ...
-        const int t = pair / DS, ks = pair % DS;
-        const int slot = 8 * ((rho / 4) % 2) + 4 * t + rho % 4;    // within its half
-        k_off[rep] = (unsigned)((slot * D + 32 * ks + 8 * g) * sizeof(bf16));
-    }
-    // V: lane group g holds keys 8g .. 8g+7 of d row 16*dt + rho
     const int v_half = g / 2;
-    unsigned v_off[VREP];
-#pragma unroll
-    for (int rep = 0; rep < VREP; ++rep) {
-        const int dt = cw + AP_WAVES * rep;
-        v_off[rep] = (unsigned)(((16 * dt + rho) * page_size + 8 * (g % 2)) * sizeof(bf16));
-    }
     const int page_mask = page_size - 1;
+    // a page's bytes per tensor, and where this key/value head starts in it (K [slot][d] and V [d][slot]
+    // have the same size)
+    const unsigned page_bytes = (unsigned)Hkv * page_size * D * sizeof(bf16);
+    const char* const k_head = reinterpret_cast<const char*>(k_pages) + (size_t)kvh * page_size * D * sizeof(bf16);
+    const char* const v_head = reinterpret_cast<const char*>(v_pages) + (size_t)kvh * page_size * D * sizeof(bf16);
+    // what of a lane's addresses does not depend on the block: head, the slot of its half within a
+    // page (pages of 16: none), its chunk of the first load
+    const char* k_lane;
+    const char* v_lane;
+    unsigned k_step[KREP], v_step[VREP];   // further loads: constant distances from the first
+    {
+        const int hk = (16 * k_half) & page_mask, hv = (16 * v_half) & page_mask;
+        unsigned k_off[KREP], v_off[VREP];
+#pragma unroll
+        for (int rep = 0; rep < KREP; ++rep) {
+            const int pair = cw + AP_WAVES * rep;   // (score tile, k-step): LDS chunks pair * 64 ...
+            const int t = pair / DS, ks = pair % DS;
+            const int slot = 8 * ((rho / 4) % 2) + 4 * t + rho % 4;    // within its half
+            k_off[rep] = (unsigned)((slot * D + 32 * ks + 8 * g) * sizeof(bf16));
+            k_step[rep] = k_off[rep] - k_off[0];
+        }
+        // V: lane group g holds keys 8g .. 8g+7 of d row 16*dt + rho
+#pragma unroll
+        for (int rep = 0; rep < VREP; ++rep) {
+            const int dt = cw + AP_WAVES * rep;
+            v_off[rep] = (unsigned)(((16 * dt + rho) * page_size + 8 * (g % 2)) * sizeof(bf16));
+            v_step[rep] = v_off[rep] - v_off[0];
+        }
+        k_lane = k_head + (size_t)hk * D * sizeof(bf16) + k_off[0];
+        v_lane = v_head + (size_t)hv * sizeof(bf16) + v_off[0];
+    }
     // round j of the walk: key group kg has block b0 + j * KW + kg
     auto block_of = [&](int j) { return b0 + j * KW + kg; };
     auto page_ids = [&](int j) {
         int b = block_of(j);
         b = b < b1 ? b : b1;    // past the unit's range: some valid entry (the block is not fetched)
         PageIds ids;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            int pidx = (32 * b + 16 * t) >> page_shift;
-            pidx = pidx < bt_width ? pidx : bt_width - 1;
-            ids.pg[t] = bt[pidx];
-        }
+        int pk = (32 * b + 16 * k_half) >> page_shift, pv = (32 * b + 16 * v_half) >> page_shift;
+        pk = pk < bt_width ? pk : bt_width - 1;
+        pv = pv < bt_width ? pv : bt_width - 1;
+        ids.k = bt[pk];
+        ids.v = bt[pv];
         return ids;
     };
-    // a page's bytes per tensor, and where this key/value head starts in it (K [slot][d] and V [d][slot]
-    // have the same size)
-    const unsigned page_bytes = (unsigned)Hkv * page_size * D * sizeof(bf16);
-    const char* const k_head = reinterpret_cast<const char*>(k_pages) + (size_t)kvh * page_size * D * sizeof(bf16);
-    const char* const v_head = reinterpret_cast<const char*>(v_pages) + (size_t)kvh * page_size * D * sizeof(bf16);
     // Asks for the block of round j (at most the unit's last one: the same block again does no harm).
-    // Returns a bit per half whose page was given back (its keys lie below every column's range):
-    // some page is read in its place and the values are cleared when they have landed.
+    // A page that was given back (its keys lie below every column's range) has a negative id: some
+    // page is read in its place and the values are cleared when they have landed.
     auto fetch = [&](int j, const PageIds& ids, uint4* stage) {
         int b = block_of(j);
         b = b < b1 ? b : b1;
-        const char* kbase[2];
-        const char* vbase[2];
-        int gone = 0;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            int pg = ids.pg[t];
-            if (pg < 0) {
-                gone |= 1 << t;
-                pg = 0;
-            }
-            const unsigned slot0 = (unsigned)((32 * b + 16 * t) & page_mask);
-            const size_t page_off = (size_t)(unsigned)pg * page_bytes;
-            kbase[t] = k_head + page_off + slot0 * (unsigned)(D * sizeof(bf16));
-            vbase[t] = v_head + page_off + slot0 * (unsigned)sizeof(bf16);
-        }
-        const char* kb = k_half ? kbase[1] : kbase[0];
-        const char* vb = v_half ? vbase[1] : vbase[0];
+        const unsigned sb = (unsigned)((32 * b) & page_mask);     // the block's first slot within its page
+        const unsigned pgk = ids.k < 0 ? 0u : (unsigned)ids.k, pgv = ids.v < 0 ? 0u : (unsigned)ids.v;
+        const char* kb = k_lane + (size_t)pgk * page_bytes + sb * (unsigned)(D * sizeof(bf16));
+        const char* vb = v_lane + (size_t)pgv * page_bytes + sb * (unsigned)sizeof(bf16);
         uint4* tile = stage + kg * TILE;
 #pragma unroll
         for (int rep = 0; rep < KREP; ++rep)
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(kb + k_off[rep]),
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(kb + k_step[rep]),
                                              (lds_ptr_t)(tile + (cw + AP_WAVES * rep) * 64), 16, 0, 0);
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep)
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(vb + v_off[rep]),
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(vb + v_step[rep]),
                                              (lds_ptr_t)(tile + KCHUNKS + (cw + AP_WAVES * rep) * 64), 16, 0, 0);
-        return gone;
+        return ids.v < 0;
     };
     // After the wave's own loads of round j have landed: clears the values of keys that were never
     // written (above the unit's newest key) or whose page was given back. Each lane mends the chunks
     // it brought in, so no other wave is involved before the barrier.
-    auto mend = [&](int j, int gone, uint4* stage) {
+    auto mend = [&](int j, bool gone, uint4* stage) {
         const int b = block_of(j);
         const bool tail = 32 * b + 31 > hi_g;
-        if (!tail && gone == 0) return;
+        if (!tail && !(window >= 0 && __any(gone))) return;
         uint4* sV = stage + kg * TILE + KCHUNKS;
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep) {
             const int idx = (cw + AP_WAVES * rep) * 64 + lane;
             Frag f;
             f.u = sV[idx];
-            if ((gone >> v_half) & 1) {
+            if (gone) {
                 f.u = uint4{0u, 0u, 0u, 0u};
             } else {
 #pragma unroll
@@ -325,9 +325,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         Frag kop[2][DS];
         Frag vop[DT];   // asked for with the keys; they arrive while the softmax is worked out
     };
-    auto wanted = [&](int j) {   // whether the wave has anything to do with the block of round j
+    // the blocks the wave has anything to do with, and those of them that need no mask
+    const int bw_hi = (hi_w >> 5) < b1 ? (hi_w >> 5) : b1, bw_lo = lo_w >> 5;
+    const int bm_hi = (wave_full && full_hi >= 31) ? (full_hi - 31) >> 5 : -1, bm_lo = (full_lo + 31) >> 5;
+    auto wanted = [&](int j) {
         const int b = block_of(j);
-        return b <= b1 && 32 * b <= hi_w && 32 * b + 31 >= lo_w;
+        return b <= bw_hi && b >= bw_lo;
     };
     auto read_operands = [&](const uint4* stage, Operands& op) {
         const uint4* sK = stage + kg * TILE;
@@ -342,7 +345,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     // ... then the two products with the softmax between them
     auto compute = [&](int j, const Operands& op) {
         const int base = 32 * block_of(j);
-        const bool masked = !(wave_full && base + 31 <= full_hi && base >= full_lo);
+        const bool masked = block_of(j) > bm_hi || block_of(j) < bm_lo;
         // scores^T for the two 16-key tiles
         float p[NT][2][4];
 #pragma unroll
@@ -428,7 +431,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     auto two_rounds = [&](int j, uint4* cur0, uint4* cur1, uint4* nxt0, uint4* nxt1) {
         const bool more = j + 2 < rounds;
         const bool busy0 = wanted(j), busy1 = wanted(j + 1);
-        int gone_a = 0, gone_b = 0;
+        bool gone_a = false, gone_b = false;
         Operands op;
         if (busy0) read_operands(cur0, op);
         if (more) {
@@ -451,8 +454,8 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     };
     {
         const PageIds i0 = page_ids(0), i1 = page_ids(1);
-        const int gone0 = fetch(0, i0, stage0);
-        const int gone1 = fetch(1, i1, stage1);
+        const bool gone0 = fetch(0, i0, stage0);
+        const bool gone1 = fetch(1, i1, stage1);
         ids_a = page_ids(2);
         ids_b = page_ids(3);
         AP_WAIT_VMCNT(0);
