@@ -6,9 +6,12 @@
 // sequence. Each wave owns 16*NT columns. The workgroup walks the keys the unit may see in blocks
 // of 32. Every block's K tile [32 keys x D] and V tile [D x 32 keys] go from the cache pages
 // straight into LDS (global_load_lds: no registers in between, no LDS store instructions), in the
-// order the MFMA operands are read (so the reads are conflict-free 16-byte loads), into stages
-// that are filled ahead of the computation: two blocks are computed between barriers while the
-// next two land in another pair of stages.
+// order the MFMA operands are read (so the reads are conflict-free 16-byte loads), into four stages
+// in two pairs that are filled ahead of the computation: two blocks are computed to a barrier while
+// the next two land in the other pair. With four waves the barrier stands between the two blocks
+// of a pair and a block's operands come from LDS while the block before is computed (keys a block
+// ahead, values behind the score product); with eight waves both blocks are read and computed
+// between two barriers.
 //
 //   scores^T = K Q^T     A operand: 16 keys x 32 d from LDS, B operand: the wave's queries (registers);
 //                        result: lane l holds column l%16 and rows 4*(l/16)+0..3 of the tile.
@@ -319,31 +322,35 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     for (int ct = 0; ct < NT; ++ct) all_cols = all_cols && col_ok[ct];
     const bool wave_full = __all(all_cols);
 
-    // A round's computation comes in two parts, so that the loads of a later round can be asked for
-    // in between: first the operands of the block are read from LDS into registers ...
-    struct Operands {
-        Frag kop[2][DS];
-        Frag vop[DT];   // asked for with the keys; they arrive while the softmax is worked out
-    };
     // the blocks the wave has anything to do with, and those of them that need no mask
     const int bw_hi = (hi_w >> 5) < b1 ? (hi_w >> 5) : b1, bw_lo = lo_w >> 5;
-    const int bm_hi = (wave_full && full_hi >= 31) ? (full_hi - 31) >> 5 : -1, bm_lo = (full_lo + 31) >> 5;
     auto wanted = [&](int j) {
         const int b = block_of(j);
         return b <= bw_hi && b >= bw_lo;
     };
-    auto read_operands = [&](const uint4* stage, Operands& op) {
+    const int bm_hi = (wave_full && full_hi >= 31) ? (full_hi - 31) >> 5 : -1, bm_lo = (full_lo + 31) >> 5;
+    // The operands of a block come from LDS in two parts, each asked for a phase before it is used:
+    // the keys of block b + 1 and the values of block b behind block b's score product.
+    struct KOps {
+        Frag kop[2][DS];
+    };
+    struct VOps {
+        Frag vop[DT];
+    };
+    auto read_k = [&](const uint4* stage, KOps& op) {
         const uint4* sK = stage + kg * TILE;
-        const uint4* sV = sK + KCHUNKS;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int s = 0; s < DS; ++s) op.kop[t][s].u = sK[(t * DS + s) * 64 + lane];
+    };
+    auto read_v = [&](const uint4* stage, VOps& op) {
+        const uint4* sV = stage + kg * TILE + KCHUNKS;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) op.vop[dt].u = sV[dt * 64 + lane];
     };
     // ... then the two products with the softmax between them
-    auto compute = [&](int j, const Operands& op) {
+    auto compute = [&](int j, const KOps& op, const VOps& vo, const uint4* k_next, KOps& op_next, const uint4* v_now, VOps& vo_w, const bool ask_k, const bool ask_v) {
         const int base = 32 * block_of(j);
         const bool masked = block_of(j) > bm_hi || block_of(j) < bm_lo;
         // scores^T for the two 16-key tiles
@@ -360,6 +367,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 for (int r = 0; r < 4; ++r) p[ct][t][r] = sacc[r];
             }
         }
+        // the keys of the next block are asked for behind the score products (in front of them the
+        // wait for this block's keys could not leave them in flight: the counter has four bits)
+        __builtin_amdgcn_sched_barrier(0);
+        if (ask_v) read_v(v_now, vo_w);
+        if (ask_k) read_k(k_next, op_next);
+        __builtin_amdgcn_sched_barrier(0);
         if (masked) {
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct)
@@ -416,57 +429,124 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct)
-                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op.vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
+                acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vo.vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
     };
 
     const int rounds = (b1 - b0 + KW) / KW;    // the same for every wave: they meet at the barriers
-    // Two rounds to a barrier: read the operands of round j, ask for rounds j+2 and j+3 (into the
-    // pair of stages that was computed last time), compute rounds j and j+1, make sure the loads
-    // have landed, meet. The barrier orders the operand reads of a pair before the loads that
-    // refill it, and makes every wave's loads visible to the others (each wave has waited for its
-    // own). With two blocks between barriers the waves drift apart and one wave's products overlap
-    // another's softmax (measured on MI355X against one block per barrier: up to a quarter faster
-    // with four waves to a workgroup, the same with eight).
     PageIds ids_a, ids_b;
-    auto two_rounds = [&](int j, uint4* cur0, uint4* cur1, uint4* nxt0, uint4* nxt1) {
-        const bool more = j + 2 < rounds;
-        const bool busy0 = wanted(j), busy1 = wanted(j + 1);
+    KOps k_even, k_odd;
+    VOps vals;
+    if constexpr (KW == 1) {
+        // Two rounds to a barrier, the barrier between the two: with blocks j and j + 1 in one pair of
+        // stages and j + 2, j + 3 landing in the other,
+        //   block j is computed (its values and the keys of j + 1 come from LDS behind its score product);
+        //   values of j + 1 are asked for; the wave's loads of the other pair have landed, its reads of
+        //   this pair are back: the workgroup meets;
+        //   blocks j + 4 and j + 5 are asked for into this pair (nobody reads it any more); block j + 1 is
+        //   computed from registers, the keys of j + 2 come from the other pair behind its score product.
+        // So the reads from LDS run while a block is computed, and the loads from the pages have two
+        // blocks' computation to land. (A block the wave has nothing to do with is computed all the
+        // same: every key of it is masked; the walk has no branches around the reads and the products.)
         bool gone_a = false, gone_b = false;
-        Operands op;
-        if (busy0) read_operands(cur0, op);
-        if (more) {
-            gone_a = fetch(j + 2, ids_a, nxt0);
-            gone_b = fetch(j + 3, ids_b, nxt1);
-            ids_a = page_ids(j + 4);
-            ids_b = page_ids(j + 5);
+        auto two_rounds = [&](int j, uint4* cur0, uint4* cur1, uint4* nxt0, uint4* nxt1) {
+            compute(j, k_even, vals, cur1, k_odd, cur0, vals, true, true);
+            read_v(cur1, vals);
+            // (asked for here and not a block earlier: 32 columns a wave have no registers to spare
+            // for them during the block, and the wait that follows is for the loads of two blocks)
+            const PageIds nid_a = page_ids(j + 6), nid_b = page_ids(j + 7);
+            AP_WAIT_VMCNT(0);
+            if (j + 2 < rounds) {
+                mend(j + 2, gone_a, nxt0);
+                mend(j + 3, gone_b, nxt1);      // past the walk's end too: the block is computed
+            }
+            AP_WAIT_LDS();
+            __builtin_amdgcn_s_barrier();
+            if (j + 4 < rounds) {
+                gone_a = fetch(j + 4, ids_a, cur0);
+                gone_b = fetch(j + 5, ids_b, cur1);
+            }
+            ids_a = nid_a;
+            ids_b = nid_b;
+            compute(j + 1, k_odd, vals, nxt0, k_even, nxt0, vals, true, false);
+        };
+        {
+            const PageIds i0 = page_ids(0), i1 = page_ids(1);
+            AP_WAIT_VMCNT(0);
+            const bool gone0 = fetch(0, i0, stage0);
+            const bool gone1 = fetch(1, i1, stage1);
+            ids_a = page_ids(2);
+            ids_b = page_ids(3);
+            AP_WAIT_VMCNT(0);
+            mend(0, gone0, stage0);
+            mend(1, gone1, stage1);
+            __builtin_amdgcn_s_barrier();
+            if (rounds > 2) {
+                gone_a = fetch(2, ids_a, stage2);
+                gone_b = fetch(3, ids_b, stage3);
+            }
+            ids_a = page_ids(4);
+            ids_b = page_ids(5);
+            AP_WAIT_LDS();
+            read_k(stage0, k_even);
         }
-        if (busy0) compute(j, op);
-        if (busy1) {
-            read_operands(cur1, op);
-            compute(j + 1, op);
+        for (int j = 0; j < rounds; j += 4) {
+            two_rounds(j, stage0, stage1, stage2, stage3);
+            if (j + 2 >= rounds) break;
+            two_rounds(j + 2, stage2, stage3, stage0, stage1);
         }
         AP_WAIT_VMCNT(0);
-        if (more) {
-            mend(j + 2, gone_a, nxt0);
-            if (j + 3 < rounds) mend(j + 3, gone_b, nxt1);
+        __builtin_amdgcn_s_barrier();
+    } else {
+        // Two rounds to a barrier: read the operands of round j, ask for rounds j+2 and j+3 (into the
+        // pair of stages that was computed last time), compute rounds j and j+1, make sure the loads
+        // have landed, meet. The barrier orders the operand reads of a pair before the loads that
+        // refill it, and makes every wave's loads visible to the others (each wave has waited for its
+        // own). With two blocks between barriers the waves drift apart and one wave's products overlap
+        // another's softmax (measured on MI355X against one block per barrier: up to a quarter faster
+        // with four waves to a workgroup, the same with eight).
+        auto two_rounds = [&](int j, uint4* cur0, uint4* cur1, uint4* nxt0, uint4* nxt1) {
+            const bool more = j + 2 < rounds;
+            const bool busy0 = wanted(j), busy1 = wanted(j + 1);
+            bool gone_a = false, gone_b = false;
+            if (busy0) {
+                read_k(cur0, k_even);
+                read_v(cur0, vals);
+            }
+            if (more) {
+                gone_a = fetch(j + 2, ids_a, nxt0);
+                gone_b = fetch(j + 3, ids_b, nxt1);
+                ids_a = page_ids(j + 4);
+                ids_b = page_ids(j + 5);
+            }
+            if (busy0) compute(j, k_even, vals, cur0, k_even, cur0, vals, false, false);
+            if (busy1) {
+                read_k(cur1, k_even);
+                read_v(cur1, vals);
+                compute(j + 1, k_even, vals, cur1, k_even, cur1, vals, false, false);
+            }
+            AP_WAIT_VMCNT(0);
+            if (more) {
+                mend(j + 2, gone_a, nxt0);
+                if (j + 3 < rounds) mend(j + 3, gone_b, nxt1);
+            }
+            __builtin_amdgcn_s_barrier();
+        };
+        {
+            const PageIds i0 = page_ids(0), i1 = page_ids(1);
+            const bool gone0 = fetch(0, i0, stage0);
+            const bool gone1 = fetch(1, i1, stage1);
+            ids_a = page_ids(2);
+            ids_b = page_ids(3);
+            AP_WAIT_VMCNT(0);
+            mend(0, gone0, stage0);
+            if (rounds > 1) mend(1, gone1, stage1);
+            __builtin_amdgcn_s_barrier();
         }
-        __builtin_amdgcn_s_barrier();
-    };
-    {
-        const PageIds i0 = page_ids(0), i1 = page_ids(1);
-        const bool gone0 = fetch(0, i0, stage0);
-        const bool gone1 = fetch(1, i1, stage1);
-        ids_a = page_ids(2);
-        ids_b = page_ids(3);
-        AP_WAIT_VMCNT(0);
-        mend(0, gone0, stage0);
-        if (rounds > 1) mend(1, gone1, stage1);
-        __builtin_amdgcn_s_barrier();
-    }
-    for (int j = 0; j < rounds; j += 4) {
-        two_rounds(j, stage0, stage1, stage2, stage3);
-        if (j + 2 >= rounds) break;
-        two_rounds(j + 2, stage2, stage3, stage0, stage1);
+        for (int j = 0; j < rounds; j += 4) {
+            two_rounds(j, stage0, stage1, stage2, stage3);
+            if (j + 2 >= rounds) break;
+            two_rounds(j + 2, stage2, stage3, stage0, stage1);
+        }
     }
     // nothing is in flight any more
 
@@ -556,11 +636,13 @@ static int launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_s
 // nt: column tiles per wave (2 = 128 columns per workgroup, for long prompts; 1 = 64 columns, twice
 // the workgroups, for steps too small to fill the chip otherwise).
 // kw: key groups per workgroup (2: eight waves, the walk over a unit's keys takes half as many rounds).
-// n_units = sum over sequences of ceil(q_len / unit tokens(group, nt)). grid = (kv heads, units).
+// n_units = sum over sequences of ceil(q_len / unit tokens(group, nt)), or an upper bound of it (units
+// beyond the step's own end at once); n_busy = the units that hold tokens, as far as the caller knows
+// (n_units if it knows no better): it decides how the units are dealt out. grid = (kv heads, units).
 extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_table, int bt_width, int page_size,
-                                    const int* positions, const int* cu_seqlens, int n_seqs, int n_units, int nt,
-                                    int kw, int H, int Hkv, int D, float scale, int window, hipStream_t stream) {
+                                    const int* positions, const int* cu_seqlens, int n_seqs, int n_units, int n_busy,
+                                    int nt, int kw, int H, int Hkv, int D, float scale, int window, hipStream_t stream) {
     MV_REQUIRE(kw == 1 || kw == 2, "attention_prefill: %d key groups per workgroup (1 or 2)", kw);
     MV_REQUIRE(H > 0 && Hkv > 0 && H % Hkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", H,
                Hkv);
@@ -581,7 +663,8 @@ extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, lon
     int cus = 0, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
         cus = 256;
-    const int fold = (kw == 1 && (long)Hkv * n_units <= 2L * cus) ? 1 : 0;
+    if (n_busy <= 0 || n_busy > n_units) n_busy = n_units;
+    const int fold = (kw == 1 && (long)Hkv * n_busy <= 2L * cus) ? 1 : 0;
     int rc = 0;
 #define AP_LAUNCH(DD, NN, KK)                                                                                      \
     rc = launch_prefill<DD, NN, KK>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,       \

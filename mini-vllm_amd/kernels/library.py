@@ -110,8 +110,8 @@ _OPTIONAL_SIGNATURES = {
     "mv_embedding_gather": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_void_p]),
     "mv_attention_prefill": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                                     c_int, c_void_p]),
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     c_float, c_int, c_void_p]),
     "mv_attention_prefill_unit_tokens": (c_int, [c_int, c_int]),
     "mv_launch_empty": (c_int, [c_int, c_int, c_void_p, c_void_p]),
 }

@@ -1081,15 +1081,16 @@ class Ops:
         if nt == 0:
             return False
         # two key groups per workgroup (eight waves) halve the walk over long contexts; they pay while
-        # the grid leaves compute units waiting for the longest walk (measured on MI355X: faster up
-        # to two workgroups per compute unit, slower beyond)
+        # the grid leaves compute units waiting for the longest walk (measured on MI355X, 8 kv heads:
+        # faster below two four-wave workgroups per compute unit, 33.9 against 35.3 us at 1,792 tokens,
+        # slower from there on, 44.0 against 40.8 us at 2,048)
         # (a recorded step's grid is sized for the most units its size class can have; the rule goes by
         # the units its tokens fill, as an eager step's does)
-        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_busy * Hkv <= 2 * self.compute_units else 1
+        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_busy * Hkv < 2 * self.compute_units else 1
         self._note_attention("mv_attention_prefill", plan, q.shape[0], H, Hkv, D, 2)
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
-                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, nt, kw, H, Hkv, D,
+                      positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, n_busy, nt, kw, H, Hkv, D,
                       float(scale), window, self._stream())
         return True
 
