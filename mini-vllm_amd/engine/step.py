@@ -64,6 +64,9 @@ class AttentionPlan:
     # decode steps: over how many workgroups a sequence's keys are dealt out; None lets the launch
     # rule choose (tests force counts)
     decode_splits: Optional[int] = None
+    # prompt steps: (column tiles per wave, key groups per workgroup) of the MFMA kernel; None lets the
+    # launch rule choose (tests force variants)
+    prefill_variant: Optional[tuple] = None
     # steps recorded into a graph that serves any cut of up to (tokens, sequences): the kernels' grids
     # are then sized for the worst cut, not for ``q_lens`` (workgroups without work end at once)
     bound: Optional[tuple] = None

@@ -1078,6 +1078,12 @@ class Ops:
                     continue
                 nt, n_units, n_busy = cand, units, busy
                 break
+        if plan.prefill_variant is not None:
+            nt = int(plan.prefill_variant[0])
+            u = self.lib.dll.mv_attention_prefill_unit_tokens(group, nt)
+            if u <= 0:
+                raise KernelLibraryError(f"attention: {nt} column tiles a wave do not serve {group} heads per kv head")
+            n_units, n_busy = plan.units(u), plan.busy_units(u)
         if nt == 0:
             return False
         # two key groups per workgroup (eight waves) halve the walk over long contexts; they pay while
@@ -1087,6 +1093,8 @@ class Ops:
         # (a recorded step's grid is sized for the most units its size class can have; the rule goes by
         # the units its tokens fill, as an eager step's does)
         kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_busy * Hkv < 2 * self.compute_units else 1
+        if plan.prefill_variant is not None:
+            kw = int(plan.prefill_variant[1])
         self._note_attention("mv_attention_prefill", plan, q.shape[0], H, Hkv, D, 2)
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,

@@ -344,6 +344,63 @@ def test_attention_general(dtype, with_plan, H, Hkv, D, ps, window):
     assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= tol
 
 
+@pytest.mark.parametrize("nt,kw", [(1, 1), (1, 2), (2, 1), (2, 2)])
+@pytest.mark.parametrize("H,Hkv,D,ps,window", [(4, 2, 128, 16, None), (8, 2, 64, 32, 150), (16, 2, 128, 64, 70)])
+def test_attention_prompt_variants(nt, kw, H, Hkv, D, ps, window):
+    """Every variant of the MFMA prompt kernel (16 or 32 columns a wave, four or eight waves a
+    workgroup) on the same step, whatever the launch rule would choose for it: portions that end
+    inside a unit and inside a block of keys, walks of one, two, three and many rounds (the stages
+    are used again from the third pair of blocks on), a window with pages given back, and slots
+    beyond a sequence's end that hold NaN."""
+    ops = ops_for(torch.bfloat16)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(67)
+    ctx_lens = [19, 61, 100, 333, 517]
+    q_lens = [19, 40, 7, 333, 130]
+    k_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    v_all = [torch.randn(c, Hkv, D, generator=g).to(dtype).double() for c in ctx_lens]
+    pages_per = [-(-c // ps) for c in ctx_lens]
+    num_pages = sum(pages_per) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, cur = [], 0
+    for n_p in pages_per:
+        tables.append(perm[cur:cur + n_p]); cur += n_p
+    if window is not None:
+        for s, (c, ql) in enumerate(zip(ctx_lens, q_lens)):
+            for i in range(max(0, (c - ql) - window) // ps):
+                tables[s][i] = -1
+    kp, vp = fill_pages(k_all, v_all, tables, ps, Hkv, D, num_pages, dtype)
+    bt = torch.full((len(tables), max(pages_per) + 2), -1, dtype=torch.int32)
+    for s, t in enumerate(tables):
+        bt[s, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    positions, token_seq = [], []
+    for s, (c, ql) in enumerate(zip(ctx_lens, q_lens)):
+        positions += list(range(c - ql, c)); token_seq += [s] * ql
+    n = len(positions)
+    positions = torch.tensor(positions, dtype=torch.int32)
+    token_seq = torch.tensor(token_seq, dtype=torch.int32)
+    q = torch.randn(n, H, D, generator=g)
+    starts = np.cumsum([0] + q_lens)
+    for s in range(len(q_lens)):          # the last query of every sequence looks at a far key (or the window's edge)
+        far = 0 if window is None else max(0, ctx_lens[s] - 1 - window)
+        q[starts[s + 1] - 1] = 6.0 * k_all[s][far].float().repeat_interleave(H // Hkv, dim=0) / math.sqrt(D)
+    q = q.to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.full((n, H * D), float("nan"), dtype=dtype, device="cuda")
+    plan = make_plan(q_lens, ctx_lens)
+    plan.prefill_variant = (nt, kw)
+    ledger, ops.ledger = ops.ledger, []
+    try:
+        ops.attention(dev(q.view(n, H * D)), out, kp, vp, dev(bt), ps, dev(positions), dev(token_seq), H, Hkv, D, scale,
+                      window, plan=plan)
+        seen = [line[0] for line in ops.ledger]
+    finally:
+        ops.ledger = ledger
+    assert seen == ["mv_attention_prefill"], seen
+    want = reference_attention(q.double(), k_all, v_all, positions, token_seq, H, Hkv, scale, window)
+    assert rel_err(out.float().cpu().view(n, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]
+
+
 @pytest.mark.parametrize("H,Hkv,D,ps,window", [(4, 2, 128, 16, None), (8, 2, 64, 32, 300), (8, 1, 128, 16, None)])
 @pytest.mark.parametrize("ctx_lens,q_lens", [([1203, 1170, 1050], [1203, 70, 1]), ([5003, 6100, 2050], [5003, 650, 1])])
 def test_attention_prompts_with_long_contexts(H, Hkv, D, ps, window, ctx_lens, q_lens):
