@@ -329,8 +329,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         return b <= bw_hi && b >= bw_lo;
     };
     const int bm_hi = (wave_full && full_hi >= 31) ? (full_hi - 31) >> 5 : -1, bm_lo = (full_lo + 31) >> 5;
-    // The operands of a block come from LDS in two parts, each asked for a phase before it is used:
-    // the keys of block b + 1 and the values of block b behind block b's score product.
+    // The operands of a block come from LDS in two parts (keys, values). The walk of four waves asks
+    // for them a phase before they are used: the keys of block b + 1 and the values of block b behind
+    // block b's score product; the walk of eight waves reads both in front of the block.
     struct KOps {
         Frag kop[2][DS];
     };
@@ -349,7 +350,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) op.vop[dt].u = sV[dt * 64 + lane];
     };
-    // ... then the two products with the softmax between them
+    // The two products with the softmax between them. ask_k / ask_v: behind the score product, ask
+    // for the keys of the next block (from k_next into op_next) and for this block's values (from
+    // v_now into vo_w, which is `vo`).
     auto compute = [&](int j, const KOps& op, const VOps& vo, const uint4* k_next, KOps& op_next, const uint4* v_now, VOps& vo_w, const bool ask_k, const bool ask_v) {
         const int base = 32 * block_of(j);
         const bool masked = block_of(j) > bm_hi || block_of(j) < bm_lo;
@@ -367,8 +370,8 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 for (int r = 0; r < 4; ++r) p[ct][t][r] = sacc[r];
             }
         }
-        // the keys of the next block are asked for behind the score products (in front of them the
-        // wait for this block's keys could not leave them in flight: the counter has four bits)
+        // (behind the score products, not in front: there the wait for this block's keys could not
+        // leave sixteen younger reads in flight, the counter of LDS reads has four bits)
         __builtin_amdgcn_sched_barrier(0);
         if (ask_v) read_v(v_now, vo_w);
         if (ask_k) read_k(k_next, op_next);
