@@ -30,7 +30,7 @@ import numpy as np
 
 from ..parts.base import Retention
 from .page_pool import OutOfPages, PagePool, page_hash
-from .state_slots import OutOfSlots, StateSlots
+from .state_slots import StateSlots
 
 
 @dataclass(frozen=True)

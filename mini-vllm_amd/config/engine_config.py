@@ -16,7 +16,7 @@ has them (``model``, ``max_model_len``, ``max_num_batched_tokens``, ``max_num_ba
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Optional, Tuple
 
 

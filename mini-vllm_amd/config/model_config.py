@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import json
 import os
-from dataclasses import dataclass, field, fields, asdict
+from dataclasses import dataclass
 from typing import Any, ClassVar, Dict, Optional, Tuple
 
 

@@ -16,7 +16,6 @@ import logging
 import time
 from typing import Dict, List, Optional, Sequence, Tuple, Union
 
-import torch
 
 from ..config.engine_config import EngineConfig
 from ..config.sampling_params import SamplingParams

@@ -10,7 +10,7 @@ from __future__ import annotations
 import copy
 import enum
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from itertools import count
 from typing import List, Optional
 

@@ -19,7 +19,6 @@ from __future__ import annotations
 
 import json
 import os
-import sys
 from typing import IO, Dict, List, Optional
 
 import numpy as np

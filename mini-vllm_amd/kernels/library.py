@@ -6,7 +6,6 @@ per file); when that is impossible the import of an operation fails with the rea
 from __future__ import annotations
 
 import ctypes
-import os
 import threading
 from typing import Dict
 

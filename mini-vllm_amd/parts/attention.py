@@ -12,12 +12,11 @@ per-head norms, the rotary embedding and the cache write are one kernel.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Optional, Tuple
+from typing import Dict, Optional
 
 import torch
 
-from .base import (CacheNeed, KeepAll, KeepWindow, KeyValueNeed, Mixer, PartSpec, POSITION_ENCODINGS, Runtime,
-                   TensorDecl, register_mixer)
+from .base import CacheNeed, KeepAll, KeepWindow, KeyValueNeed, Mixer, PartSpec, Runtime, TensorDecl, register_mixer
 
 
 @dataclass(frozen=True)

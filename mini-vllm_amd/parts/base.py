@@ -21,8 +21,8 @@ nothing else in the engine changes.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Any, Callable, ClassVar, Dict, List, Mapping, Optional, Sequence, Tuple, Type
+from dataclasses import dataclass
+from typing import Any, ClassVar, Dict, List, Optional, Sequence, Tuple
 
 import torch
 

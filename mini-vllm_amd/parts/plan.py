@@ -7,8 +7,8 @@ earlier call wrote instead of keeping one (``cache_from``).
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, Mapping, Optional, Tuple
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
 
 from .base import PartSpec
 

@@ -14,7 +14,7 @@ from typing import Dict, Optional, Tuple
 
 import torch
 
-from .base import PartSpec, PositionEncoding, Runtime, TensorDecl, register_position_encoding
+from .base import PartSpec, PositionEncoding, Runtime, register_position_encoding
 
 
 @dataclass(frozen=True)

@@ -10,7 +10,7 @@ by (seed, index of the token being drawn), so what it draws does not depend on t
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import List, Sequence
 
 import numpy as np
 import torch

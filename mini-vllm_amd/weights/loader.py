@@ -11,10 +11,9 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional, Tuple
 
-import torch
 
 from ..parts.base import TensorDecl
-from .source import KEPT_FLOAT_TYPES, DeviceTensors, SafetensorsSource, TensorSource
+from .source import KEPT_FLOAT_TYPES, SafetensorsSource, TensorSource
 
 
 class WeightError(ValueError):

@@ -15,7 +15,7 @@ from __future__ import annotations
 import glob
 import os
 import weakref
-from typing import Dict, Iterable, List, Optional, Tuple
+from typing import Dict, List, Tuple
 
 import torch
 
